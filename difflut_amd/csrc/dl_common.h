@@ -1,0 +1,36 @@
+// Shared helpers for the gfx950 kernels of libdifflut_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/difflut_hip.h"
+
+#define DL_WAVE 64
+
+static inline int dl_launch_status() {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? DL_OK : (int)e;
+}
+
+static inline size_t dl_align256(size_t v) { return (v + 255) & ~(size_t)255; }
+static inline int dl_ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
+
+// Value of `v` held by lane `src_lane` (0..63) of the same wavefront.
+__device__ __forceinline__ float dl_lane_read(float v, int src_lane) {
+    return __int_as_float(__builtin_amdgcn_ds_bpermute(src_lane << 2, __float_as_int(v)));
+}
+
+// Wave-uniform value into a scalar register so that loads addressed by it become scalar loads.
+__device__ __forceinline__ int dl_uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// Optional per-kernel timing (dl_profile_enable / dl_profile_read): when switched on, every
+// launch site records a HIP event before and after its kernel on the launch stream.
+void dl_prof_begin(const char *kernel_name, hipStream_t s);
+void dl_prof_end(hipStream_t s);
+#define DL_TIMED(name, s, ...) \
+    do {                       \
+        dl_prof_begin(name, s); \
+        __VA_ARGS__;           \
+        dl_prof_end(s);        \
+    } while (0)

@@ -1,0 +1,212 @@
+// RandomLayer index gather and its adjoint, LearnableLayer hard selection, thermometer
+// encoding and GroupSum: the streaming pieces either side of the node kernels.
+#include "dl_common.h"
+
+// m[b,n,j] = x[b, idx[n,j]]: one block per (row, slab of the flattened [N*k] axis).  The row of
+// x is read through the cache (random but inside one 4*I-byte row), writes are coalesced.
+template <typename index_t>
+__global__ __launch_bounds__(256) void gather_fwd_kernel(const float *__restrict__ x, const index_t *__restrict__ idx,
+                                                          float *__restrict__ m, int I, long long NK) {
+    const int b = blockIdx.y;
+    const float *xrow = x + (size_t)b * I;
+    float *out = m + (size_t)b * NK;
+    for (long long p = (long long)blockIdx.x * 1024 + threadIdx.x; p < min(NK, ((long long)blockIdx.x + 1) * 1024);
+         p += 256)
+        out[p] = xrow[idx[p]];
+}
+
+// gx[b,i] = sum over CSR entries of input i of gm[b, pos]; fixed order, no atomics.
+__global__ __launch_bounds__(256) void gather_bwd_kernel(const float *__restrict__ gm, const int *__restrict__ inv_ptr,
+                                                          const int *__restrict__ inv_pos, float *__restrict__ gx,
+                                                          int I, long long NK) {
+    const int b = blockIdx.y;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= I) return;
+    const float *row = gm + (size_t)b * NK;
+    float acc = 0.0f;
+    for (int e = inv_ptr[i]; e < inv_ptr[i + 1]; ++e) acc += row[inv_pos[e]];
+    gx[(size_t)b * I + i] = acc;
+}
+
+// One wavefront per row of W; lowest index wins ties.
+__global__ __launch_bounds__(256) void row_argmax_kernel(const float *__restrict__ W, int *__restrict__ sel, int M, int I) {
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= M) return;
+    const float *w = W + (size_t)row * I;
+    float best = -INFINITY;
+    int arg = 0x7fffffff;
+    for (int i = lane; i < I; i += 64) {
+        const float v = w[i];
+        if (v > best || (v == best && i < arg) || arg == 0x7fffffff) { best = v; arg = i; }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ob = __shfl_xor(best, off);
+        const int oa = __shfl_xor(arg, off);
+        if (oa != 0x7fffffff && (arg == 0x7fffffff || ob > best || (ob == best && oa < arg))) { best = ob; arg = oa; }
+    }
+    if (lane == 0) sel[row] = arg;
+}
+
+__global__ __launch_bounds__(256) void thermometer_kernel(const float *__restrict__ x, const float *__restrict__ thr,
+                                                           float *__restrict__ bits, long long total, int FB, int nbits) {
+    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= total) return;
+    const long long b = gid / FB;
+    const int fb = (int)(gid % FB);
+    const int f = fb / nbits;
+    bits[gid] = x[b * (FB / nbits) + f] > thr[fb] ? 1.0f : 0.0f;  // strict compare
+}
+
+// One wavefront per (row, group): sum a contiguous run of group_size features.
+__global__ __launch_bounds__(256) void group_sum_fwd_kernel(const float *__restrict__ x, float *__restrict__ y, int B,
+                                                             int F, int groups, int gsize, float inv_tau) {
+    const long long w = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (w >= (long long)B * groups) return;
+    const int b = (int)(w / groups), g = (int)(w % groups);
+    const float *row = x + (size_t)b * F;
+    float acc = 0.0f;
+    for (int f = g * gsize + lane; f < min(F, (g + 1) * gsize); f += 64) acc += row[f];
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+    if (lane == 0) y[w] = acc * inv_tau;
+}
+
+__global__ __launch_bounds__(256) void group_sum_bwd_kernel(const float *__restrict__ gy, float *__restrict__ gx,
+                                                             long long total, int F, int groups, int gsize,
+                                                             float inv_tau) {
+    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= total) return;
+    const long long b = gid / F;
+    const int f = (int)(gid % F);
+    gx[gid] = gy[b * groups + f / gsize] * inv_tau;
+}
+
+// ---------------------------------------------------------------------------------
+extern "C" int dl_gather_fwd(const float *x, const void *idx, int idx_bits, float *m, int B, int I, int N, int k,
+                             void *stream) {
+    if (!x || !idx || !m) return DL_ERR_NULL;
+    if (B <= 0 || I <= 0 || N <= 0 || k <= 0) return DL_ERR_SHAPE;
+    if (idx_bits != 16 && idx_bits != 32) return DL_ERR_UNSUPPORTED;
+    const long long NK = (long long)N * k;
+    dim3 grid(dl_ceil_div(NK, 1024), B);
+    if (idx_bits == 16)
+        gather_fwd_kernel<int16_t><<<grid, 256, 0, (hipStream_t)stream>>>(x, (const int16_t *)idx, m, I, NK);
+    else
+        gather_fwd_kernel<int32_t><<<grid, 256, 0, (hipStream_t)stream>>>(x, (const int32_t *)idx, m, I, NK);
+    return dl_launch_status();
+}
+
+extern "C" int dl_gather_bwd(const float *gm, const int32_t *inv_ptr, const int32_t *inv_pos, float *gx, int B, int I,
+                             int N, int k, void *stream) {
+    if (!gm || !inv_ptr || !inv_pos || !gx) return DL_ERR_NULL;
+    if (B <= 0 || I <= 0 || N <= 0 || k <= 0) return DL_ERR_SHAPE;
+    gather_bwd_kernel<<<dim3(dl_ceil_div(I, 256), B), 256, 0, (hipStream_t)stream>>>(gm, inv_ptr, inv_pos, gx, I,
+                                                                                    (long long)N * k);
+    return dl_launch_status();
+}
+
+extern "C" int dl_row_argmax(const float *W, int32_t *sel, int M, int I, void *stream) {
+    if (!W || !sel) return DL_ERR_NULL;
+    if (M <= 0 || I <= 0) return DL_ERR_SHAPE;
+    row_argmax_kernel<<<dl_ceil_div(M, 4), 256, 0, (hipStream_t)stream>>>(W, sel, M, I);
+    return dl_launch_status();
+}
+
+extern "C" int dl_hard_select_fwd(const float *x, const int32_t *sel, float *m, int B, int I, int M, void *stream) {
+    return dl_gather_fwd(x, sel, 32, m, B, I, M, 1, stream);
+}
+
+extern "C" int dl_hard_select_bwd(const float *gm, const int32_t *inv_ptr, const int32_t *inv_pos, float *gx, int B,
+                                  int I, int M, void *stream) {
+    return dl_gather_bwd(gm, inv_ptr, inv_pos, gx, B, I, M, 1, stream);
+}
+
+extern "C" int dl_thermometer_encode(const float *x, const float *thr, float *bits, int B, int F, int nbits,
+                                     void *stream) {
+    if (!x || !thr || !bits) return DL_ERR_NULL;
+    if (B <= 0 || F <= 0 || nbits <= 0) return DL_ERR_SHAPE;
+    const long long total = (long long)B * F * nbits;
+    thermometer_kernel<<<dl_ceil_div(total, 256), 256, 0, (hipStream_t)stream>>>(x, thr, bits, total, F * nbits, nbits);
+    return dl_launch_status();
+}
+
+extern "C" int dl_group_sum_fwd(const float *x, float *y, int B, int F, int groups, float tau, void *stream) {
+    if (!x || !y) return DL_ERR_NULL;
+    if (B <= 0 || F <= 0 || groups <= 0 || !(tau > 0.0f)) return DL_ERR_SHAPE;
+    const int gsize = (F + groups - 1) / groups;  // features zero-padded up to groups * gsize
+    group_sum_fwd_kernel<<<dl_ceil_div((long long)B * groups, 4), 256, 0, (hipStream_t)stream>>>(x, y, B, F, groups,
+                                                                                                gsize, 1.0f / tau);
+    return dl_launch_status();
+}
+
+extern "C" int dl_group_sum_bwd(const float *gy, float *gx, int B, int F, int groups, float tau, void *stream) {
+    if (!gy || !gx) return DL_ERR_NULL;
+    if (B <= 0 || F <= 0 || groups <= 0 || !(tau > 0.0f)) return DL_ERR_SHAPE;
+    const int gsize = (F + groups - 1) / groups;
+    const long long total = (long long)B * F;
+    group_sum_bwd_kernel<<<dl_ceil_div(total, 256), 256, 0, (hipStream_t)stream>>>(gy, gx, total, F, groups, gsize,
+                                                                                  1.0f / tau);
+    return dl_launch_status();
+}
+
+// ---------------------------------------------------------------------------------
+// per-kernel timing
+#define DL_PROF_MAX 64
+static struct {
+    int on, count, created;
+    hipEvent_t ev[2 * DL_PROF_MAX];
+    const char *name[DL_PROF_MAX];
+} g_prof;
+
+void dl_prof_begin(const char *kernel_name, hipStream_t s) {
+    if (!g_prof.on || g_prof.count >= DL_PROF_MAX) return;
+    while (g_prof.created < 2 * (g_prof.count + 1)) hipEventCreate(&g_prof.ev[g_prof.created++]);
+    g_prof.name[g_prof.count] = kernel_name;
+    hipEventRecord(g_prof.ev[2 * g_prof.count], s);
+}
+void dl_prof_end(hipStream_t s) {
+    if (!g_prof.on || g_prof.count >= DL_PROF_MAX) return;
+    hipEventRecord(g_prof.ev[2 * g_prof.count + 1], s);
+    ++g_prof.count;
+}
+
+extern "C" int dl_profile_enable(int on) {
+    g_prof.on = on ? 1 : 0;
+    g_prof.count = 0;
+    return DL_OK;
+}
+
+extern "C" int dl_profile_read(char *names, size_t names_bytes, float *ms, int max_entries) {
+    int n = g_prof.count < max_entries ? g_prof.count : max_entries;
+    size_t used = 0;
+    if (names && names_bytes) names[0] = 0;
+    for (int i = 0; i < n; ++i) {
+        hipEventSynchronize(g_prof.ev[2 * i + 1]);
+        float t = 0.0f;
+        hipEventElapsedTime(&t, g_prof.ev[2 * i], g_prof.ev[2 * i + 1]);
+        if (ms) ms[i] = t;
+        if (names) {
+            const char *nm = g_prof.name[i];
+            for (size_t c = 0; nm[c] && used + 2 < names_bytes; ++c) names[used++] = nm[c];
+            if (used + 1 < names_bytes) names[used++] = ';';
+            names[used] = 0;
+        }
+    }
+    g_prof.count = 0;
+    return n;
+}
+
+extern "C" int dl_version(void) { return 100; }
+
+extern "C" const char *dl_error_string(int code) {
+    switch (code) {
+        case DL_OK: return "ok";
+        case DL_ERR_NULL: return "a required pointer is null";
+        case DL_ERR_SHAPE: return "a size is not positive or sizes are inconsistent";
+        case DL_ERR_UNSUPPORTED: return "k, O or an option is outside what the kernels cover";
+        case DL_ERR_WORKSPACE: return "workspace is smaller than the matching *_workspace_bytes()";
+        case DL_ERR_INDEX: return "an index is outside [0, I)";
+        default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
+    }
+}

@@ -1,0 +1,295 @@
+"""Layer-level operators: torch.autograd.Functions over the C ABI of libdifflut_hip.so.
+
+These are the callers of the drop-in boundary.  They keep the conventions of the
+reference's autograd wrappers (difflut/layers/random_layer.py:34-100,
+difflut/nodes/dwn_node.py:58-128, difflut/nodes/probabilistic_node.py:39-129,
+difflut/layers/learnable_layer.py:58-123): inputs are made contiguous fp32, outputs
+are new tensors, non-tensor arguments get no gradient.  Unlike the reference, one
+call covers a whole layer, kernels go to torch's current stream and nothing
+synchronises the device.
+"""
+import torch
+
+from . import _native as nat
+
+FAST_K = 6
+
+
+def _f32(t):
+    return t.contiguous().float()
+
+
+def _bytes(n, device):
+    return torch.empty(max(int(n), 256), dtype=torch.uint8, device=device)
+
+
+class MappingPlan:
+    """Device-side form of an index table idx [N,k] over I inputs.
+
+    idx32   int32 [N,k]         the table widened (the reference registers int16 below 32768 inputs)
+    inv_ptr int32 [I+1]         CSR row pointers of the inverse mapping
+    inv_pos int32 [N*k]         flat positions n*k+j, grouped by input, ascending inside a group
+    Built once per table with torch ops (sort + bincount); the kernels only read it.
+    """
+
+    def __init__(self, idx, input_size):
+        if idx.dim() != 2:
+            raise ValueError(f"mapping indices must be 2D (nodes, inputs per node), got {tuple(idx.shape)}")
+        if idx.dtype not in (torch.int16, torch.int32, torch.int64):
+            raise TypeError(f"mapping indices must be int16, int32 or int64, got {idx.dtype}")
+        self.N, self.k = idx.shape
+        self.I = int(input_size)
+        flat = idx.reshape(-1).long()
+        if flat.numel() and (int(flat.min()) < 0 or int(flat.max()) >= self.I):
+            raise IndexError(f"mapping index outside [0, {self.I})")
+        self.idx32 = idx.to(torch.int32).contiguous()
+        order = torch.argsort(flat, stable=True)
+        counts = torch.bincount(flat, minlength=self.I)
+        self.inv_ptr = torch.cat([counts.new_zeros(1), counts.cumsum(0)]).to(torch.int32).contiguous()
+        self.inv_pos = order.to(torch.int32).contiguous()
+        self.device = idx.device
+        self.source_ptr = idx.data_ptr()
+        self.source_version = idx._version
+
+    def matches(self, idx):
+        return (idx.device == self.device and idx.data_ptr() == self.source_ptr
+                and idx._version == self.source_version and tuple(idx.shape) == (self.N, self.k))
+
+    @staticmethod
+    def identity(k, device):
+        return MappingPlan(torch.arange(k, dtype=torch.int32, device=device).view(1, k), k)
+
+
+# ----------------------------------------------------------------------------- gather
+class GatherFunction(torch.autograd.Function):
+    """m[b,n,j] = x[b, idx[n,j]]  (RandomLayer.get_mapping)."""
+
+    @staticmethod
+    def forward(ctx, x, idx, plan):
+        nat.require_device(x, idx)
+        x = _f32(x)
+        B, I = x.shape
+        N, k = idx.shape
+        bits = {torch.int16: 16, torch.int32: 32}.get(idx.dtype)
+        if bits is None:
+            raise TypeError("Unsupported index type for mapping kernel. Use int16 or int32.")
+        m = torch.empty((B, N, k), dtype=torch.float32, device=x.device)
+        nat.check(nat.lib().dl_gather_fwd(nat.ptr(x), nat.ptr(idx.contiguous()), bits, nat.ptr(m), B, I, N, k,
+                                          nat.stream()))
+        ctx.plan = plan
+        ctx.shape = (B, I, N, k)
+        return m
+
+    @staticmethod
+    def backward(ctx, gm):
+        B, I, N, k = ctx.shape
+        gm = _f32(gm)
+        gx = torch.empty((B, I), dtype=torch.float32, device=gm.device)
+        p = ctx.plan
+        nat.check(nat.lib().dl_gather_bwd(nat.ptr(gm), nat.ptr(p.inv_ptr), nat.ptr(p.inv_pos), nat.ptr(gx), B, I, N, k,
+                                          nat.stream()))
+        return gx, None, None
+
+
+# ----------------------------------------------------------------------------- DWN
+class DWNLayerFunction(torch.autograd.Function):
+    """y[b, n*O+d] = luts[n,d,addr(b,n)] with the extended-finite-difference backward."""
+
+    @staticmethod
+    def forward(ctx, x, luts, plan, alpha, beta):
+        nat.require_device(x, luts)
+        x, luts = _f32(x), _f32(luts)
+        B, I = x.shape
+        N, O, L = luts.shape
+        k = plan.k
+        if (N, 1 << k, I) != (plan.N, L, plan.I):
+            raise RuntimeError(f"shape mismatch: x {tuple(x.shape)}, luts {tuple(luts.shape)}, mapping [{plan.N},{k}] "
+                               f"over {plan.I} inputs")
+        lib = nat.lib()
+        dims = (B, I, N, k, O)
+        y = torch.empty((B, N * O), dtype=torch.float32, device=x.device)
+        saved = _bytes(lib.dl_dwn_saved_bytes(*dims), x.device)
+        ws = _bytes(lib.dl_dwn_fwd_workspace_bytes(*dims), x.device)
+        nat.check(lib.dl_dwn_layer_fwd(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(luts), nat.ptr(y), nat.ptr(saved),
+                                       nat.ptr(ws), ws.numel(), *dims, nat.stream()))
+        ctx.save_for_backward(luts, saved, x if k > FAST_K else None)
+        ctx.plan, ctx.ab, ctx.dims = plan, (float(alpha), float(beta)), dims
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        luts, saved, x = ctx.saved_tensors
+        B, I, N, k, O = ctx.dims
+        plan = ctx.plan
+        gy = _f32(gy)
+        lib = nat.lib()
+        gx = torch.empty((B, I), dtype=torch.float32, device=gy.device) if ctx.needs_input_grad[0] else None
+        gl = torch.empty_like(luts)
+        ws = _bytes(lib.dl_dwn_bwd_workspace_bytes(*ctx.dims), gy.device)
+        nat.check(lib.dl_dwn_layer_bwd(nat.ptr(x), nat.ptr(saved), nat.ptr(plan.idx32), nat.ptr(plan.inv_ptr),
+                                       nat.ptr(plan.inv_pos), nat.ptr(luts), nat.ptr(gy), ctx.ab[0], ctx.ab[1],
+                                       nat.ptr(gx), nat.ptr(gl), nat.ptr(ws), ws.numel(), *ctx.dims, nat.stream()))
+        return gx, gl, None, None, None
+
+
+def dwn_layer_eval(x, luts, plan):
+    nat.require_device(x, luts)
+    x, luts = _f32(x), _f32(luts)
+    B, I = x.shape
+    N, O, _ = luts.shape
+    y = torch.empty((B, N * O), dtype=torch.float32, device=x.device)
+    nat.check(nat.lib().dl_dwn_layer_eval(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(luts), nat.ptr(y), B, I, N, plan.k, O,
+                                          nat.stream()))
+    return y
+
+
+# ----------------------------------------------------------------------------- Probabilistic
+class ProbLayerFunction(torch.autograd.Function):
+    """y[b, n*O+d] = sum_a sigmoid(raw[n,a,d]/T) prod_j (x_j a_j + (1-x_j)(1-a_j))."""
+
+    @staticmethod
+    def forward(ctx, x, raw, plan, temperature):
+        nat.require_device(x, raw)
+        x, raw = _f32(x), _f32(raw)
+        B, I = x.shape
+        N, L, O = raw.shape
+        k = plan.k
+        if (N, 1 << k, I) != (plan.N, L, plan.I):
+            raise RuntimeError(f"shape mismatch: x {tuple(x.shape)}, raw_weights {tuple(raw.shape)}, mapping "
+                               f"[{plan.N},{k}] over {plan.I} inputs")
+        y = torch.empty((B, N * O), dtype=torch.float32, device=x.device)
+        dims = (B, I, N, k, O)
+        nat.check(nat.lib().dl_prob_layer_fwd(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(raw), float(temperature),
+                                              nat.ptr(y), *dims, nat.stream()))
+        ctx.save_for_backward(x, raw)
+        ctx.plan, ctx.T, ctx.dims = plan, float(temperature), dims
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        x, raw = ctx.saved_tensors
+        plan = ctx.plan
+        gy = _f32(gy)
+        lib = nat.lib()
+        B, I = x.shape
+        gx = torch.empty((B, I), dtype=torch.float32, device=gy.device) if ctx.needs_input_grad[0] else None
+        graw = torch.empty_like(raw)
+        ws = _bytes(lib.dl_prob_bwd_workspace_bytes(*ctx.dims), gy.device)
+        nat.check(lib.dl_prob_layer_bwd(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(plan.inv_ptr), nat.ptr(plan.inv_pos),
+                                        nat.ptr(raw), ctx.T, nat.ptr(gy), nat.ptr(gx), nat.ptr(graw), nat.ptr(ws),
+                                        ws.numel(), *ctx.dims, nat.stream()))
+        return gx, graw, None, None
+
+
+def prob_layer_eval(x, raw, plan, temperature):
+    nat.require_device(x, raw)
+    x, raw = _f32(x), _f32(raw)
+    B, I = x.shape
+    N, _, O = raw.shape
+    y = torch.empty((B, N * O), dtype=torch.float32, device=x.device)
+    nat.check(nat.lib().dl_prob_layer_eval(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(raw), float(temperature),
+                                           nat.ptr(y), B, I, N, plan.k, O, nat.stream()))
+    return y
+
+
+# ----------------------------------------------------------------------------- Learnable mapping
+class SoftMapFunction(torch.autograd.Function):
+    """m = x @ softmax(W / tau, dim=-1).T without materialising the softmax."""
+
+    @staticmethod
+    def forward(ctx, x, W, tau, precision):
+        nat.require_device(x, W)
+        x, W = _f32(x), _f32(W)
+        B, I = x.shape
+        M = W.shape[0]
+        if W.shape[1] != I:
+            raise RuntimeError(f"shape mismatch: x {tuple(x.shape)} vs W {tuple(W.shape)}")
+        lib = nat.lib()
+        m = torch.empty((B, M), dtype=torch.float32, device=x.device)
+        stats = torch.empty((2 * M,), dtype=torch.float32, device=x.device)
+        ws = _bytes(lib.dl_soft_map_workspace_bytes(B, I, M, precision), x.device)
+        nat.check(lib.dl_soft_map_fwd(nat.ptr(x), nat.ptr(W), float(tau), nat.ptr(m), nat.ptr(stats), nat.ptr(ws),
+                                      ws.numel(), B, I, M, precision, nat.stream()))
+        ctx.save_for_backward(x, W, m, stats)
+        ctx.tau, ctx.precision = float(tau), precision
+        return m
+
+    @staticmethod
+    def backward(ctx, gm):
+        x, W, m, stats = ctx.saved_tensors
+        gm = _f32(gm)
+        B, I = x.shape
+        M = W.shape[0]
+        lib = nat.lib()
+        gx = torch.empty_like(x)
+        gW = torch.empty_like(W)
+        ws = _bytes(lib.dl_soft_map_workspace_bytes(B, I, M, ctx.precision), x.device)
+        nat.check(lib.dl_soft_map_bwd(nat.ptr(x), nat.ptr(W), ctx.tau, nat.ptr(m), nat.ptr(stats), nat.ptr(gm),
+                                      nat.ptr(gx), nat.ptr(gW), nat.ptr(ws), ws.numel(), B, I, M, ctx.precision,
+                                      nat.stream()))
+        return gx, gW, None, None
+
+
+def row_argmax(W):
+    nat.require_device(W)
+    W = _f32(W)
+    sel = torch.empty((W.shape[0],), dtype=torch.int32, device=W.device)
+    nat.check(nat.lib().dl_row_argmax(nat.ptr(W), nat.ptr(sel), W.shape[0], W.shape[1], nat.stream()))
+    return sel
+
+
+class HardSelectFunction(torch.autograd.Function):
+    """m[b,o] = x[b, sel[o]] with the straight scatter-add backward."""
+
+    @staticmethod
+    def forward(ctx, x, sel, plan):
+        nat.require_device(x, sel)
+        x = _f32(x)
+        B, I = x.shape
+        M = sel.numel()
+        m = torch.empty((B, M), dtype=torch.float32, device=x.device)
+        nat.check(nat.lib().dl_hard_select_fwd(nat.ptr(x), nat.ptr(sel.contiguous().int()), nat.ptr(m), B, I, M,
+                                               nat.stream()))
+        ctx.plan, ctx.shape = plan, (B, I, M)
+        return m
+
+    @staticmethod
+    def backward(ctx, gm):
+        B, I, M = ctx.shape
+        gm = _f32(gm)
+        gx = torch.empty((B, I), dtype=torch.float32, device=gm.device)
+        p = ctx.plan
+        nat.check(nat.lib().dl_hard_select_bwd(nat.ptr(gm), nat.ptr(p.inv_ptr), nat.ptr(p.inv_pos), nat.ptr(gx), B, I, M,
+                                               nat.stream()))
+        return gx, None, None
+
+
+# ----------------------------------------------------------------------------- encoder / head
+def thermometer_encode(x, thresholds):
+    nat.require_device(x, thresholds)
+    x, thr = _f32(x), _f32(thresholds)
+    B, F = x.shape
+    nbits = thr.shape[1]
+    bits = torch.empty((B, F, nbits), dtype=torch.float32, device=x.device)
+    nat.check(nat.lib().dl_thermometer_encode(nat.ptr(x), nat.ptr(thr), nat.ptr(bits), B, F, nbits, nat.stream()))
+    return bits
+
+
+class GroupSumFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, groups, tau):
+        nat.require_device(x)
+        x = _f32(x)
+        B, F = x.shape
+        y = torch.empty((B, groups), dtype=torch.float32, device=x.device)
+        nat.check(nat.lib().dl_group_sum_fwd(nat.ptr(x), nat.ptr(y), B, F, groups, float(tau), nat.stream()))
+        ctx.args = (B, F, groups, float(tau))
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        B, F, groups, tau = ctx.args
+        gy = _f32(gy)
+        gx = torch.empty((B, F), dtype=torch.float32, device=gy.device)
+        nat.check(nat.lib().dl_group_sum_bwd(nat.ptr(gy), nat.ptr(gx), B, F, groups, tau, nat.stream()))
+        return gx, None, None

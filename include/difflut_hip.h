@@ -1,0 +1,174 @@
+/* difflut_hip.h - C ABI of the MI355X (gfx950) DiffLUT hot path.
+ *
+ * One shared library, libdifflut_hip.so, built from difflut_amd/csrc/ by hipcc.
+ * Plain pointers and sizes only; every pointer is DEVICE memory unless it says
+ * host.  `stream` is a hipStream_t passed as void*.  Nothing here allocates or
+ * frees device memory and nothing synchronises the device: outputs and
+ * workspaces come from the caller, kernels are enqueued on `stream`.
+ *
+ * Return value of every int function: 0 = ok, negative = argument error
+ * (DL_ERR_*), positive = a hipError_t from a launch.  dl_error_string() turns
+ * either into text.
+ *
+ * Each entry point names the reference interface it replaces (paths relative
+ * to the aplesner/difflut checkout).
+ *
+ * Shapes: B batch rows, I layer inputs, N nodes, k inputs per node, L = 2^k
+ * table entries, O outputs per node, M = N*k selections of a learnable layer.
+ * All float tensors are fp32, row-major, contiguous.
+ */
+#ifndef DIFFLUT_HIP_H
+#define DIFFLUT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DL_OK 0
+#define DL_ERR_NULL (-1)        /* a required pointer is null */
+#define DL_ERR_SHAPE (-2)       /* a size is <= 0 or inconsistent */
+#define DL_ERR_UNSUPPORTED (-3) /* k, O or an option outside what the kernels cover */
+#define DL_ERR_WORKSPACE (-4)   /* workspace smaller than the matching *_workspace_bytes() */
+#define DL_ERR_INDEX (-5)       /* an index table entry is outside [0, I) (host-checked entry points only) */
+
+#define DL_MAX_FAST_K 6  /* tables of up to 64 entries sit one-per-lane in a wavefront */
+#define DL_MAX_K 16      /* generic kernels */
+
+int dl_version(void);
+const char *dl_error_string(int code);
+
+/* ------------------------------------------------------------------------
+ * RandomLayer mapping gather.
+ * Replaces mapping_cuda.forward / .backward
+ *   (difflut/layers/cuda/mapping_cuda.cpp:25-74, mapping_cuda_kernel.cu:30-56,136-162),
+ * called from RandomLayer.get_mapping (difflut/layers/random_layer.py:258-304).
+ * idx is [N,k]; idx_bits says whether it holds int16 (16) or int32 (32) entries,
+ * the two dtypes the reference registers (random_layer.py:214).
+ * ------------------------------------------------------------------------ */
+/* m[b,n,j] = x[b, idx[n,j]]          x [B,I] -> m [B,N,k] */
+int dl_gather_fwd(const float *x, const void *idx, int idx_bits, float *m,
+                  int B, int I, int N, int k, void *stream);
+/* gx[b,i] = sum_{(n,j): idx[n,j]=i} gm[b,n,j]; gx [B,I] is overwritten.
+ * inv_ptr [I+1] / inv_pos [N*k] is the inverse of idx in CSR form (inv_pos holds
+ * flat positions n*k+j, ascending inside each input): the sum is a gather in a
+ * fixed order, so results are run-to-run identical (the reference uses atomics). */
+int dl_gather_bwd(const float *gm, const int32_t *inv_ptr, const int32_t *inv_pos, float *gx,
+                  int B, int I, int N, int k, void *stream);
+
+/* ------------------------------------------------------------------------
+ * RandomLayer + DWN nodes, whole layer in one call.
+ * Replaces the per-node loop of RandomLayer.forward (random_layer.py:306-340)
+ * over efd_cuda.forward/.backward (difflut/nodes/cuda/efd_cuda.cpp:22-45,
+ * efd_cuda_kernel.cu:12-43,79-189) and the layer-wide efd_fused_cuda.forward/
+ * .backward (efd_fused_cuda.cpp:19-34, efd_fused_cuda_kernel.cu:11-197).
+ *   idx32 [N,k] int32 (the registered int16/int32 table widened once by the host)
+ *   luts  [N,O,L]     (the N node tables [O,L] of dwn_node.py:423 stacked)
+ *   y     [B,N*O]
+ * Training forward: addr = sum_j [x[b,idx[n,j]] >= 0.5] << j;  y[b,n,d] = luts[n,d,addr].
+ * `saved` (dl_dwn_saved_bytes) receives what the backward needs instead of x:
+ * for k <= DL_MAX_FAST_K the address of every (node, row), node-major.
+ * `ws` (dl_dwn_fwd_workspace_bytes) is scratch that may be reused after the call.
+ * ------------------------------------------------------------------------ */
+size_t dl_dwn_saved_bytes(int B, int I, int N, int k, int O);
+size_t dl_dwn_fwd_workspace_bytes(int B, int I, int N, int k, int O);
+size_t dl_dwn_bwd_workspace_bytes(int B, int I, int N, int k, int O);
+int dl_dwn_layer_fwd(const float *x, const int32_t *idx32, const float *luts, float *y,
+                     void *saved, void *ws, size_t ws_bytes,
+                     int B, int I, int N, int k, int O, void *stream);
+/* Extended-finite-difference backward (dwn_node.py:167-229):
+ *   gx[b,i]     = sum_{(n,j): idx=i} alpha * sum_d gy[b,n,d] *
+ *                 sum_kappa s(kappa_j) luts[n,d,kappa] beta^popc((addr ^ kappa) & ~(1<<j))
+ *   gluts[n,d,e] = sum_b [addr(b,n) = e] gy[b,n,d]
+ * gx may be null (input does not need a gradient); gx and gluts are overwritten.
+ * x is only read when k > DL_MAX_FAST_K (then `saved` is unused) and may be null otherwise. */
+int dl_dwn_layer_bwd(const float *x, const void *saved, const int32_t *idx32,
+                     const int32_t *inv_ptr, const int32_t *inv_pos,
+                     const float *luts, const float *gy, float alpha, float beta,
+                     float *gx, float *gluts, void *ws, size_t ws_bytes,
+                     int B, int I, int N, int k, int O, void *stream);
+/* Eval forward (DWNNode.forward_eval, dwn_node.py:457-483): addr = floor(sum_j x_j 2^j)
+ * with no thresholding of x (clamped to the table), y = (luts[n,d,addr] >= 0.5) as 0/1. */
+int dl_dwn_layer_eval(const float *x, const int32_t *idx32, const float *luts, float *y,
+                      int B, int I, int N, int k, int O, void *stream);
+
+/* ------------------------------------------------------------------------
+ * RandomLayer + Probabilistic nodes, whole layer in one call.
+ * Replaces the node loop over probabilistic_cuda.forward/.backward
+ * (difflut/nodes/cuda/probabilistic_cuda.cpp:22-49, probabilistic_cuda_kernel.cu:7-307)
+ * and the CPU branch of ProbabilisticNode.forward_train (probabilistic_node.py:284-300).
+ *   raw_w [N,L,O] (the node parameters raw_weights [L,O] stacked), temperature T:
+ *   y[b,n,d] = sum_a sigmoid(raw_w[n,a,d] / max(T,1e-6)) * prod_j (x_j a_j + (1-x_j)(1-a_j)),
+ *   x_j = x[b, idx[n,j]] used as given (no clamping: inputs are probabilities).
+ * Backward is the exact derivative of that expression (what autograd gives the
+ * reference's CPU path): gx [B,I] (nullable), graw [N,L,O]; both overwritten.
+ * ------------------------------------------------------------------------ */
+size_t dl_prob_bwd_workspace_bytes(int B, int I, int N, int k, int O);
+int dl_prob_layer_fwd(const float *x, const int32_t *idx32, const float *raw_w, float temperature,
+                      float *y, int B, int I, int N, int k, int O, void *stream);
+int dl_prob_layer_bwd(const float *x, const int32_t *idx32,
+                      const int32_t *inv_ptr, const int32_t *inv_pos,
+                      const float *raw_w, float temperature, const float *gy,
+                      float *gx, float *graw, void *ws, size_t ws_bytes,
+                      int B, int I, int N, int k, int O, void *stream);
+/* Eval forward (probabilistic_node.py:302-328): y = (sigmoid(raw_w[n,addr,d]/T) >= 0.5). */
+int dl_prob_layer_eval(const float *x, const int32_t *idx32, const float *raw_w, float temperature,
+                       float *y, int B, int I, int N, int k, int O, void *stream);
+
+/* ------------------------------------------------------------------------
+ * LearnableLayer soft connectivity (training) and hard selection (eval).
+ * Replaces F.softmax(W / tau, -1) followed by torch.matmul(x, S.t()) and its
+ * autograd (difflut/layers/learnable_layer.py:254-255), the forward-only
+ * learnable_mapping_cuda.soft_forward (learnable_mapping_cuda_kernel.cu:99-223),
+ * and learnable_mapping_cuda.forward/.backward for argmax selection
+ * (learnable_mapping_cuda_kernel.cu:22-81,236-257; learnable_layer.py:216-236).
+ *   x [B,I], W [M,I], m [B,M];   S = softmax(W / tau) along I, never materialised.
+ * precision: 0 = fp32 operands on the fp32 matrix cores (reference numerics),
+ *            1 = bf16 operands, fp32 accumulation (tolerance documented with the tests).
+ * stats [2*M] floats is written by the forward (row max and 1/sum of exp) and
+ * read by the backward.
+ *   gx = gm * S,   gW = S * (G - r) / tau with G = gm^T x and r[o] = sum_b gm[b,o] m[b,o].
+ * ------------------------------------------------------------------------ */
+size_t dl_soft_map_workspace_bytes(int B, int I, int M, int precision);
+int dl_soft_map_fwd(const float *x, const float *W, float tau, float *m, float *stats,
+                    void *ws, size_t ws_bytes, int B, int I, int M, int precision, void *stream);
+int dl_soft_map_bwd(const float *x, const float *W, float tau, const float *m, const float *stats,
+                    const float *gm, float *gx, float *gW, void *ws, size_t ws_bytes,
+                    int B, int I, int M, int precision, void *stream);
+/* sel[o] = argmax_i W[o,i] (lowest index on ties), int32 [M]. */
+int dl_row_argmax(const float *W, int32_t *sel, int M, int I, void *stream);
+/* m[b,o] = x[b, sel[o]] */
+int dl_hard_select_fwd(const float *x, const int32_t *sel, float *m, int B, int I, int M, void *stream);
+/* gx[b,i] = sum_{o: sel[o]=i} gm[b,o]; CSR inverse of sel as for dl_gather_bwd (k = 1). */
+int dl_hard_select_bwd(const float *gm, const int32_t *inv_ptr, const int32_t *inv_pos, float *gx,
+                       int B, int I, int M, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Either side of the layers in the training configurations.
+ * Thermometer encode (difflut/encoder/thermometer.py:89-116):
+ *   bits[b, f*nbits + j] = (x[b,f] > thr[f,j]) as 0/1, x [B,F], thr [F,nbits].
+ * GroupSum (difflut/utils/modules.py:116-163): features zero-padded to a multiple of
+ *   groups, y[b,g] = sum of group g / tau; backward gx[b,f] = gy[b, f / group_size] / tau.
+ * ------------------------------------------------------------------------ */
+int dl_thermometer_encode(const float *x, const float *thr, float *bits, int B, int F, int nbits,
+                          void *stream);
+int dl_group_sum_fwd(const float *x, float *y, int B, int F, int groups, float tau, void *stream);
+int dl_group_sum_bwd(const float *gy, float *gx, int B, int F, int groups, float tau, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Per-kernel timing.  No counterpart in the reference (it has no tracing at all).
+ * After dl_profile_enable(1) every kernel launched by the entry points above is
+ * bracketed by HIP events on its stream (at most 64 kernels between two reads).
+ * dl_profile_read waits for those events, writes the elapsed milliseconds in
+ * launch order to ms[], the kernel names separated by ';' to names (host
+ * buffers), returns the number of entries and starts a new recording.
+ * ------------------------------------------------------------------------ */
+int dl_profile_enable(int on);
+int dl_profile_read(char *names, size_t names_bytes, float *ms, int max_entries);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DIFFLUT_HIP_H */

@@ -1,0 +1,285 @@
+"""GPU parity: every kernel family, called through the C ABI, against the CPU oracle on the same
+seeded inputs.  Integer/selection work (addresses, gathered values, table lookups, eval outputs,
+thermometer bits, argmax) must be bit-exact; floating-point sums are held to rtol 1e-5 with an
+absolute floor of a few fp32 ulps of the operand scale (stated per test)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle
+from oracle import difflut_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+def _ops():
+    from difflut_amd import ops
+    return ops
+
+
+def dev(a, dtype=torch.float32):
+    return torch.as_tensor(np.ascontiguousarray(a)).to(DEV, dtype)
+
+
+def make_case(seed, B, I, N, k, O, lo=-1.0, hi=1.0, binary=False):
+    rng = np.random.default_rng(seed)
+    x = rng.integers(0, 2, (B, I)).astype(np.float32) if binary else rng.random((B, I)).astype(np.float32)
+    idx = orc.random_mapping(I, N, k, seed=seed + 1).numpy().astype(np.int64)
+    tab = rng.uniform(lo, hi, (N, O, 1 << k)).astype(np.float32)
+    gy = rng.standard_normal((B, N, O)).astype(np.float32)
+    return x, idx, tab, gy
+
+
+DWN_SHAPES = [  # (B, I, N, k, O)
+    (100, 25, 36, 6, 1),   # reference tests/test_layers/test_fused_kernels.py:26-36
+    (10, 16, 25, 4, 1),    # test_fused_kernels.py:62-72
+    (8, 256, 128, 4, 1),   # tests/test_layers/test_layer_functionality.py:37-55
+    (70, 40, 33, 3, 2),
+    (64, 128, 256, 6, 1),
+    (130, 300, 77, 5, 3),
+    (1, 7, 5, 1, 1),
+    (65, 9, 300, 2, 1),
+    (200, 1030, 515, 6, 2),
+    (9, 30, 11, 7, 2),     # k > 6: generic kernels
+    (5, 64, 6, 9, 1),
+]
+
+
+@pytest.mark.parametrize("shape", DWN_SHAPES)
+def test_dwn_layer_forward_backward(shape):
+    B, I, N, k, O = shape
+    ops = _ops()
+    x, idx, luts, gy = make_case(sum(shape), *shape)
+    plan = ops.MappingPlan(dev(idx, torch.int32), I)
+    xt = dev(x).requires_grad_()
+    lt = dev(luts).requires_grad_()
+    alpha, beta = 0.5 * 0.75 ** (k - 1), 1.0 / 3.0
+    y = ops.DWNLayerFunction.apply(xt, lt, plan, alpha, beta)
+    want = orc.dwn_layer_forward(x, idx, luts).reshape(B, N * O)
+    assert np.array_equal(y.detach().cpu().numpy(), want)  # bit exact
+    y.backward(dev(gy.reshape(B, N * O)))
+    gx, gl = orc.dwn_layer_backward(x, idx, luts, gy, np.float32(alpha), np.float32(beta))
+    # gx sums <= fan-in terms of size alpha*|gy|*|D| ~ 0.1..1: rtol 1e-5, floor 2e-6
+    np.testing.assert_allclose(xt.grad.cpu().numpy(), gx, rtol=1e-5, atol=2e-6)
+    # table gradients are plain sums of gy over the rows that hit an entry
+    np.testing.assert_allclose(lt.grad.cpu().numpy(), gl, rtol=1e-5, atol=1e-5)
+
+
+def test_dwn_threshold_is_inclusive_and_exact_at_half():
+    ops = _ops()
+    x = np.array([[0.5, 0.49999997, 0.50000006, 0.0, 1.0, -3.0]], dtype=np.float32)
+    idx = np.arange(6)[None]
+    luts = np.arange(64, dtype=np.float32)[None, None]
+    plan = ops.MappingPlan(dev(idx, torch.int32), 6)
+    y = ops.DWNLayerFunction.apply(dev(x), dev(luts), plan, 0.1, 0.3)
+    assert y.item() == float(0b010101)
+
+
+@pytest.mark.parametrize("beta", [0.0, 1.0, 0.9])
+def test_dwn_backward_other_alpha_beta(beta):
+    ops = _ops()
+    shape = (33, 20, 17, 4, 2)
+    x, idx, luts, gy = make_case(5, *shape)
+    B, I, N, k, O = shape
+    plan = ops.MappingPlan(dev(idx, torch.int32), I)
+    xt = dev(x).requires_grad_(); lt = dev(luts).requires_grad_()
+    ops.DWNLayerFunction.apply(xt, lt, plan, 0.7, beta).backward(dev(gy.reshape(B, -1)))
+    gx, gl = orc.dwn_layer_backward(x, idx, luts, gy, np.float32(0.7), np.float32(beta))
+    np.testing.assert_allclose(xt.grad.cpu().numpy(), gx, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(lt.grad.cpu().numpy(), gl, rtol=1e-5, atol=1e-5)
+
+
+def test_dwn_no_input_grad_and_unused_inputs():
+    ops = _ops()
+    B, I, N, k, O = 40, 50, 3, 2, 1  # 44 of the 50 inputs feed no node: their gradient must be 0
+    x, idx, luts, gy = make_case(11, B, I, N, k, O)
+    plan = ops.MappingPlan(dev(idx, torch.int32), I)
+    lt = dev(luts).requires_grad_()
+    ops.DWNLayerFunction.apply(dev(x), lt, plan, 0.2, 0.3).backward(dev(gy.reshape(B, -1)))
+    _, gl = orc.dwn_layer_backward(x, idx, luts, gy, np.float32(0.2), np.float32(0.3))
+    np.testing.assert_allclose(lt.grad.cpu().numpy(), gl, rtol=1e-5, atol=1e-5)
+    xt = dev(x).requires_grad_()
+    ops.DWNLayerFunction.apply(xt, dev(luts), plan, 0.2, 0.3).backward(dev(gy.reshape(B, -1)))
+    unused = np.setdiff1d(np.arange(I), idx.reshape(-1))
+    assert np.all(xt.grad.cpu().numpy()[:, unused] == 0.0)
+
+
+@pytest.mark.parametrize("shape", [(12, 20, 9, 6, 2), (70, 33, 140, 3, 1), (4, 30, 5, 8, 1)])
+def test_dwn_eval_forward(shape):
+    ops = _ops()
+    B, I, N, k, O = shape
+    x, idx, luts, _ = make_case(3, *shape, lo=0.0, hi=1.0, binary=True)
+    plan = ops.MappingPlan(dev(idx, torch.int32), I)
+    y = ops.dwn_layer_eval(dev(x), dev(luts), plan).cpu().numpy().reshape(B, N, O)
+    m = orc.gather_forward(x, idx)
+    for n in range(N):
+        assert np.array_equal(y[:, n], orc.dwn_eval_forward(m[:, n], luts[n]))
+
+
+@pytest.mark.parametrize("tag", ["k6o2", "k4o1", "k2o3"])
+def test_dwn_node_against_reference_vectors(golden, tag):
+    """Same inputs the reference's own CPU path was run on (tests/golden)."""
+    from difflut_amd.nodes.dwn_node import efd_forward
+
+    g = golden
+    a, b = (float(v) for v in g[f"dwn_{tag}_ab"])
+    xt = dev(g[f"dwn_{tag}_x"]).requires_grad_()
+    lt = dev(g[f"dwn_{tag}_luts"]).requires_grad_()
+    y = efd_forward(xt, lt, a, b)
+    assert np.array_equal(y.detach().cpu().numpy(), g[f"dwn_{tag}_y"])
+    y.backward(dev(g[f"dwn_{tag}_gy"]))
+    np.testing.assert_allclose(xt.grad.cpu().numpy(), g[f"dwn_{tag}_gx"], rtol=1e-5, atol=2e-6)
+    np.testing.assert_allclose(lt.grad.cpu().numpy(), g[f"dwn_{tag}_gl"], rtol=1e-5, atol=1e-6)
+
+
+# ------------------------------------------------------------------------------ gather
+@pytest.mark.parametrize("dtype", [torch.int16, torch.int32])
+def test_gather_forward_backward(dtype):
+    ops = _ops()
+    B, I, N, k = 37, 211, 90, 5
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((B, I)).astype(np.float32)
+    idx = orc.random_mapping(I, N, k, seed=9).numpy().astype(np.int64)
+    it = dev(idx, dtype)
+    xt = dev(x).requires_grad_()
+    m = ops.GatherFunction.apply(xt, it, ops.MappingPlan(it, I))
+    assert np.array_equal(m.detach().cpu().numpy(), orc.gather_forward(x, idx))
+    gm = rng.standard_normal((B, N, k)).astype(np.float32)
+    m.backward(dev(gm))
+    np.testing.assert_allclose(xt.grad.cpu().numpy(), orc.gather_backward(gm, idx, I), rtol=1e-6, atol=1e-6)
+
+
+# ------------------------------------------------------------------------------ probabilistic
+PROB_SHAPES = [(32, 40, 24, 4, 2), (64, 128, 300, 4, 1), (17, 30, 9, 6, 1), (20, 9, 5, 1, 1), (10, 50, 7, 2, 3),
+               (6, 40, 5, 7, 2)]
+
+
+@pytest.mark.parametrize("shape", PROB_SHAPES)
+@pytest.mark.parametrize("T", [1.0, 0.5])
+def test_prob_layer_forward_backward(shape, T):
+    ops = _ops()
+    B, I, N, k, O = shape
+    rng = np.random.default_rng(sum(shape))
+    x = (1 / (1 + np.exp(-rng.standard_normal((B, I))))).astype(np.float32)
+    idx = orc.random_mapping(I, N, k, seed=4).numpy().astype(np.int64)
+    raw = rng.uniform(0, 1, (N, 1 << k, O)).astype(np.float32)
+    gy = rng.standard_normal((B, N, O)).astype(np.float32)
+    plan = ops.MappingPlan(dev(idx, torch.int32), I)
+    xt = dev(x).requires_grad_(); wt = dev(raw).requires_grad_()
+    y = ops.ProbLayerFunction.apply(xt, wt, plan, T)
+    want = orc.prob_layer_forward(x, idx, raw, T, dtype=torch.float64).reshape(B, N * O)
+    np.testing.assert_allclose(y.detach().cpu().numpy(), want, rtol=1e-5, atol=1e-6)  # outputs lie in (0,1)
+    y.backward(dev(gy.reshape(B, -1)))
+    gx, gw = orc.prob_layer_backward(x, idx, raw, gy, T)
+    np.testing.assert_allclose(xt.grad.cpu().numpy(), gx, rtol=1e-5, atol=2e-6)
+    np.testing.assert_allclose(wt.grad.cpu().numpy(), gw, rtol=1e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("tag", ["k4o2", "k6o1"])
+def test_prob_node_against_reference_vectors(golden, tag):
+    from difflut_amd.nodes.probabilistic_node import probabilistic_forward
+    ops = _ops()
+
+    g = golden
+    T = float(g[f"prob_{tag}_T"][0])
+    xt = dev(g[f"prob_{tag}_x"]).requires_grad_()
+    wt = dev(g[f"prob_{tag}_w"]).requires_grad_()
+    y = probabilistic_forward(xt, wt, T)
+    np.testing.assert_allclose(y.detach().cpu().numpy(), g[f"prob_{tag}_y"], rtol=1e-5, atol=1e-6)
+    y.backward(dev(g[f"prob_{tag}_gy"]))
+    np.testing.assert_allclose(xt.grad.cpu().numpy(), g[f"prob_{tag}_gx"], rtol=1e-5, atol=2e-6)
+    np.testing.assert_allclose(wt.grad.cpu().numpy(), g[f"prob_{tag}_gw"], rtol=1e-5, atol=2e-6)
+    k = g[f"prob_{tag}_x"].shape[1]
+    plan = ops.MappingPlan.identity(k, DEV)
+    ye = ops.prob_layer_eval(dev(g[f"prob_{tag}_eval_x"]), wt.detach().unsqueeze(0), plan, T)
+    assert np.array_equal(ye.cpu().numpy(), g[f"prob_{tag}_eval_y"])
+
+
+# ------------------------------------------------------------------------------ learnable mapping
+@pytest.mark.parametrize("shape,tau", [((5, 20, 21), 1.0), ((70, 130, 200), 0.3), ((64, 64, 64), 1.0),
+                                       ((33, 257, 18), 0.05)])
+def test_soft_mapping_forward_backward_fp32(shape, tau):
+    ops = _ops()
+    B, I, M = shape
+    rng = np.random.default_rng(sum(shape))
+    x = rng.random((B, I)).astype(np.float32)
+    W = (rng.standard_normal((M, I)) * 0.5).astype(np.float32)
+    gm = rng.standard_normal((B, M)).astype(np.float32)
+    xt = dev(x).requires_grad_(); Wt = dev(W).requires_grad_()
+    m = ops.SoftMapFunction.apply(xt, Wt, tau, 0)
+    np.testing.assert_allclose(m.detach().cpu().numpy(), orc.soft_mapping_forward(x, W, tau, torch.float64),
+                               rtol=1e-5, atol=1e-6)  # m is a convex mix of inputs in [0,1)
+    m.backward(dev(gm))
+    gx, gW = orc.soft_mapping_backward(x, W, gm, tau)
+    np.testing.assert_allclose(xt.grad.cpu().numpy(), gx, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(Wt.grad.cpu().numpy(), gW, rtol=1e-4, atol=1e-5 / tau)
+
+
+def test_soft_and_hard_mapping_against_reference_vectors(golden):
+    ops = _ops()
+    g = golden
+    for tau_key, mk, gxk, gWk in [("soft_tau", "soft_m", "soft_gx", "soft_gW"),
+                                  ("soft_tau_500", "soft500_m", "soft500_gx", "soft500_gW")]:
+        tau = float(g[tau_key][0])
+        xt = dev(g["soft_x"]).requires_grad_(); Wt = dev(g["soft_W"]).requires_grad_()
+        m = ops.SoftMapFunction.apply(xt, Wt, tau, 0)
+        np.testing.assert_allclose(m.detach().cpu().numpy(), g[mk].reshape(5, -1), rtol=1e-5, atol=1e-6)
+        m.backward(dev(g["soft_gm"].reshape(5, -1)))
+        np.testing.assert_allclose(xt.grad.cpu().numpy(), g[gxk], rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(Wt.grad.cpu().numpy(), g[gWk], rtol=1e-4, atol=1e-5)
+    sel = ops.row_argmax(dev(g["soft_W"]))
+    assert np.array_equal(sel.cpu().numpy().reshape(7, 3), g["hard_idx"])
+    plan = ops.MappingPlan(sel.view(-1, 1), 20)
+    xt = dev(g["soft_x"]).requires_grad_()
+    hm = ops.HardSelectFunction.apply(xt, sel, plan)
+    assert np.array_equal(hm.detach().cpu().numpy(), g["hard_m"].reshape(5, -1))
+    gm = np.random.default_rng(1).standard_normal(hm.shape).astype(np.float32)
+    hm.backward(dev(gm))
+    want = orc.gather_backward(gm[:, :, None], sel.cpu().numpy().reshape(-1, 1), 20)
+    np.testing.assert_allclose(xt.grad.cpu().numpy(), want, rtol=1e-6, atol=1e-6)
+
+
+def test_row_argmax_ties_and_sizes():
+    ops = _ops()
+    rng = np.random.default_rng(2)
+    W = rng.standard_normal((300, 1000)).astype(np.float32)
+    W[5, 17] = W[5, 900] = 9.0   # tie: lowest index wins
+    W[6, :] = -1.0
+    sel = ops.row_argmax(dev(W)).cpu().numpy()
+    assert np.array_equal(sel, W.argmax(1)) and sel[5] == 17 and sel[6] == 0
+
+
+# ------------------------------------------------------------------------------ encoder / head
+def test_thermometer_and_group_sum(golden):
+    ops = _ops()
+    g = golden
+    bits = ops.thermometer_encode(dev(g["thermo_x"]), dev(g["thermo_thr"]))
+    assert np.array_equal(bits.cpu().numpy().reshape(9, -1), g["thermo_bits"])
+    xt = dev(g["groupsum_x"]).requires_grad_()
+    y = ops.GroupSumFunction.apply(xt, 5, 2.0)
+    np.testing.assert_allclose(y.detach().cpu().numpy(), g["groupsum_y"], rtol=1e-6, atol=1e-6)
+    gy = np.random.default_rng(0).standard_normal((6, 5)).astype(np.float32)
+    y.backward(dev(gy))
+    np.testing.assert_allclose(xt.grad.cpu().numpy(), np.repeat(gy, 4, 1) / 2.0, rtol=1e-6)
+    x = np.random.default_rng(1).standard_normal((3, 10)).astype(np.float32)  # 10 features, 4 groups: padded
+    y = ops.GroupSumFunction.apply(dev(x), 4, 1.0)
+    np.testing.assert_allclose(y.cpu().numpy(), orc.group_sum(x, 4, 1.0), rtol=1e-6, atol=1e-6)
+
+
+# ------------------------------------------------------------------------------ error paths
+def test_argument_errors_are_reported_not_launched():
+    from difflut_amd import _native as nat
+    lib = nat.lib()
+    assert lib.dl_dwn_layer_fwd(None, None, None, None, None, None, 0, 1, 1, 1, 1, 1, None) == -1
+    t = torch.zeros(64, device=DEV)
+    p = t.data_ptr()
+    assert lib.dl_dwn_layer_fwd(p, p, p, p, p, p, 0, 4, 4, 4, 2, 1, None) == -4   # workspace too small
+    assert lib.dl_dwn_layer_fwd(p, p, p, p, p, p, 1 << 20, 4, 4, 4, 17, 1, None) == -3  # k beyond DL_MAX_K
+    assert lib.dl_gather_fwd(p, p, 8, p, 1, 1, 1, 1, None) == -3
+    assert lib.dl_prob_layer_fwd(p, p, p, 1.0, p, 0, 1, 1, 1, 1, None) == -2
+    with pytest.raises(RuntimeError, match="ROCm devices only"):
+        _ops().DWNLayerFunction.apply(torch.zeros(2, 2), torch.zeros(1, 1, 4), None, 0.1, 0.1)
+    with pytest.raises(IndexError):
+        _ops().MappingPlan(torch.tensor([[0, 7]], device=DEV, dtype=torch.int32), 4)

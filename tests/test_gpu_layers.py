@@ -1,0 +1,247 @@
+"""GPU tests through the public layer/node API, shaped after the reference's own tests
+(tests/test_layers/test_fused_kernels.py, test_layer_functionality.py,
+tests/test_nodes/test_node_functionality.py, test_residual_initialization.py) with the CPU oracle
+standing in for the reference's CPU path, plus size-independent properties at the full benchmark
+shape (batch 4096 x 16384 inputs x 8192 nodes)."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle
+from oracle import difflut_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _api():
+    from difflut_amd import REGISTRY
+    from difflut_amd.nodes import NodeConfig
+    from difflut_amd.nodes.utils import residual_init, uniform_init
+    return REGISTRY, NodeConfig, uniform_init, residual_init
+
+
+def stacked(layer, name):
+    return torch.stack([getattr(n, name).detach() for n in layer.nodes]).cpu().numpy()
+
+
+def test_basic_functionality_fused_shapes():
+    """test_fused_kernels.py:16-49: I=25, N=36, k=6, batch 100 of randn inputs."""
+    REGISTRY, NodeConfig, _, _ = _api()
+    layer = REGISTRY.get_layer("random")(input_size=25, output_size=36, node_type=REGISTRY.get_node("dwn"),
+                                         node_kwargs=NodeConfig(input_dim=6, output_dim=1), seed=42).cuda()
+    x = torch.randn(100, 25).cuda()
+    out = layer(x)
+    assert out.shape == (100, 36) and not torch.isnan(out).any()
+    assert hasattr(layer.nodes[0], "forward_with_mapping")
+    want = orc.dwn_layer_forward(x.cpu().numpy(), layer._mapping_indices.cpu().numpy(), stacked(layer, "luts"))
+    assert np.array_equal(out.detach().cpu().numpy(), want[:, :, 0])
+    # the fused layer call equals the per-node path on the gathered inputs (test_fused_kernels.py:98-156)
+    mapped = layer.get_mapping(x)
+    per_node = torch.cat([node(mapped[:, i, :]) for i, node in enumerate(layer.nodes)], dim=1)
+    assert torch.equal(per_node, out)
+    shared = layer.nodes[3].forward_with_mapping(x, layer.get_mapping_indices())
+    assert shared.shape == (100, 36, 1)
+    want = orc.dwn_layer_forward(x.cpu().numpy(), layer._mapping_indices.cpu().numpy(),
+                                 np.repeat(stacked(layer, "luts")[3:4], 36, 0))
+    assert np.array_equal(shared.detach().cpu().numpy(), want)
+
+
+def test_gradient_flow_every_parameter():
+    """test_fused_kernels.py:52-95: I=16, N=25, k=4, batch 10; every luts gets a non-zero gradient."""
+    REGISTRY, NodeConfig, _, _ = _api()
+    layer = REGISTRY.get_layer("random")(input_size=16, output_size=25, node_type=REGISTRY.get_node("dwn"),
+                                         node_kwargs=NodeConfig(input_dim=4, output_dim=1), seed=42).cuda()
+    x = torch.randn(10, 16, device="cuda", requires_grad=True)
+    out = layer(x)
+    assert out.shape == (10, 25)
+    out.sum().backward()
+    assert x.grad is not None and x.grad.abs().sum() > 0
+    count = 0
+    for name, p in layer.named_parameters():
+        assert p.grad is not None and p.grad.abs().sum() > 0, name
+        count += 1
+    assert count == 25
+    gx, gl = orc.dwn_layer_backward(x.detach().cpu().numpy(), layer._mapping_indices.cpu().numpy(),
+                                    stacked(layer, "luts"), np.ones((10, 25, 1), np.float32),
+                                    np.float32(0.5 * 0.75 ** 3), np.float32(1 / 3))
+    np.testing.assert_allclose(x.grad.cpu().numpy(), gx, rtol=1e-5, atol=2e-6)
+    np.testing.assert_allclose(torch.stack([n.luts.grad for n in layer.nodes]).cpu().numpy(), gl, rtol=1e-6)
+
+
+@pytest.mark.parametrize("layer_name", ["random", "learnable"])
+@pytest.mark.parametrize("node_name", ["dwn", "probabilistic"])
+def test_layer_shape_range_grads_and_device_roundtrip(layer_name, node_name):
+    """test_layer_functionality.py:37-123 (input 256, 128 nodes, k=4, batch 8) for every layer x node."""
+    REGISTRY, NodeConfig, _, _ = _api()
+    torch.manual_seed(42)
+    kwargs = dict(input_size=256, output_size=128, node_type=REGISTRY.get_node(node_name),
+                  node_kwargs=NodeConfig(input_dim=4, output_dim=1))
+    cpu_layer = REGISTRY.get_layer(layer_name)(**kwargs)
+    torch.manual_seed(42)
+    layer = REGISTRY.get_layer(layer_name)(**kwargs).cuda()
+    layer.load_state_dict(cpu_layer.state_dict())  # state built on the host loads into the device layer
+    for k, v in cpu_layer.state_dict().items():
+        assert torch.equal(v, layer.state_dict()[k].cpu()), k
+    torch.manual_seed(42)
+    x = torch.rand(8, 256, device="cuda", requires_grad=True)
+    layer.train()
+    out = layer(x)
+    assert out.shape == (8, 128)
+    out.sum().backward()
+    for name, p in layer.named_parameters():
+        assert p.grad is not None and torch.isfinite(p.grad).all(), name
+    assert any(p.grad.abs().sum() > 0 for p in layer.parameters())
+    layer.eval()
+    for seed in (42, 123, 456):
+        torch.manual_seed(seed)
+        with torch.no_grad():
+            e = layer(torch.rand(8, 256, device="cuda"))
+        assert e.min() >= 0.0 and e.max() <= 1.0 and set(e.unique().tolist()) <= {0.0, 1.0}
+
+
+def test_learnable_layer_train_and_eval_against_oracle():
+    REGISTRY, NodeConfig, uniform_init, _ = _api()
+    torch.manual_seed(7)
+    layer = REGISTRY.get_layer("learnable")(
+        input_size=60, output_size=20, node_type=REGISTRY.get_node("dwn"),
+        node_kwargs=NodeConfig(input_dim=3, output_dim=1, init_fn=uniform_init, init_kwargs={"a": -1.0, "b": 1.0}),
+        tau=1.0, tau_start=1.0, tau_min=1e-4, tau_decay_iters=1000.0, use_cuda_soft=False).cuda()
+    x = torch.rand(33, 60, device="cuda", requires_grad=True)
+    W = layer.mapping.W.detach().cpu().numpy()
+    luts = stacked(layer, "luts")
+    ident = np.arange(60).reshape(20, 3)
+    layer.train()
+    out = layer(x)
+    m = orc.soft_mapping_forward(x.detach().cpu().numpy(), W, 1.0)
+    mt = layer.get_mapping(x)
+    np.testing.assert_allclose(mt.detach().cpu().numpy().reshape(33, -1), m, rtol=1e-5, atol=1e-6)
+    # node stage checked on the device's own mapped values (thresholding is discontinuous)
+    want = orc.dwn_layer_forward(mt.detach().cpu().numpy().reshape(33, -1), ident, luts)[:, :, 0]
+    assert np.array_equal(out.detach().cpu().numpy(), want)
+    gy = torch.randn_like(out)
+    out.backward(gy)
+    gmap, gl = orc.dwn_layer_backward(mt.detach().cpu().numpy().reshape(33, -1), ident, luts,
+                                      gy.cpu().numpy()[:, :, None], np.float32(0.5 * 0.75 ** 2), np.float32(1 / 3))
+    gx, gW = orc.soft_mapping_backward(x.detach().cpu().numpy(), W, gmap, 1.0)
+    np.testing.assert_allclose(x.grad.cpu().numpy(), gx, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(layer.mapping.W.grad.cpu().numpy(), gW, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(torch.stack([n.luts.grad for n in layer.nodes]).cpu().numpy(), gl, rtol=1e-5, atol=1e-5)
+    layer.eval()
+    xb = torch.randint(0, 2, (12, 60), device="cuda").float()
+    hm, sel = orc.hard_mapping(xb.cpu().numpy(), W)
+    assert np.array_equal(layer.get_mapping_matrix().cpu().numpy(), sel.reshape(20, 3))
+    want = np.stack([orc.dwn_eval_forward(hm[:, 3 * n:3 * n + 3], luts[n]) for n in range(20)], 1)[:, :, 0]
+    assert np.array_equal(layer(xb).cpu().numpy(), want)
+
+
+def test_residual_initialisation_known_answers():
+    """tests/test_nodes/test_residual_initialization.py:56-232 for DWN and Probabilistic nodes."""
+    REGISTRY, _, _, residual_init = _api()
+    corners = torch.tensor(list(itertools.product([0, 1], repeat=6)), dtype=torch.float32, device="cuda")
+    for name in ("dwn", "probabilistic"):
+        node = REGISTRY.get_node(name)(input_dim=6, output_dim=1, init_fn=residual_init,
+                                       init_kwargs={"node_type": name, "noise_factor": 0.0, "logit_clarity": 5.0,
+                                                    "input_dim": 6}).cuda()
+        node.eval()
+        with torch.no_grad():
+            assert torch.equal(node.forward_eval(corners).squeeze(), corners[:, 0])  # passes input 0 through
+        if name == "probabilistic":
+            node.train()
+            with torch.no_grad():
+                lo = node.forward_train(torch.zeros(50, 6, device="cuda")).mean().item()
+                hi = node.forward_train(torch.ones(50, 6, device="cuda")).mean().item()
+                a = torch.zeros(1, 6, device="cuda"); b = a.clone(); b[0, 1:] = 1.0
+                diff = (node.forward_train(a) - node.forward_train(b)).abs().item()
+            assert abs(lo - 1 / (1 + np.exp(5.0))) < 1e-5 and abs(hi - 1 / (1 + np.exp(-5.0))) < 1e-5 and diff < 1e-5
+        assert node.export_bitstream() == [int(c[0]) for c in corners.cpu().tolist()]
+
+
+def test_smallest_training_configuration_end_to_end(golden):
+    """thermometer -> RandomLayer+DWN -> GroupSum -> cross-entropy against the reference's numbers."""
+    REGISTRY, NodeConfig, uniform_init, _ = _api()
+    from difflut_amd.utils import GroupSum
+    g = golden
+    x = torch.tensor(g["e2e_x"]).cuda()
+    enc = REGISTRY.build_encoder("thermometer", num_bits=4).fit(x)
+    bits = enc.encode(x).requires_grad_()
+    assert np.array_equal(bits.detach().cpu().numpy(), g["e2e_bits"])
+    layer = REGISTRY.get_layer("random")(80, 30, REGISTRY.get_node("dwn"),
+                                         NodeConfig(input_dim=6, output_dim=1, init_fn=uniform_init,
+                                                    init_kwargs={"a": -1.0, "b": 1.0}), seed=42).cuda()
+    assert np.array_equal(layer._mapping_indices.cpu().numpy(), g["e2e_idx"])
+    with torch.no_grad():
+        for n, node in enumerate(layer.nodes):
+            node.luts.copy_(torch.tensor(g["e2e_luts"][n]))
+    logits = GroupSum(k=10, tau=1.0, use_randperm=False)(layer(bits))
+    np.testing.assert_allclose(logits.detach().cpu().numpy(), g["e2e_logits"], rtol=1e-6, atol=1e-6)
+    loss = torch.nn.functional.cross_entropy(logits, torch.tensor(g["e2e_labels"]).cuda())
+    assert loss.item() == pytest.approx(float(g["e2e_loss"]), rel=1e-6)
+    loss.backward()
+    np.testing.assert_allclose(bits.grad.cpu().numpy(), g["e2e_gbits"], rtol=1e-4, atol=1e-7)
+    np.testing.assert_allclose(torch.stack([n.luts.grad for n in layer.nodes]).cpu().numpy(), g["e2e_gluts"],
+                               rtol=1e-5, atol=1e-7)
+
+
+def test_adam_steps_change_tables_in_place():
+    REGISTRY, NodeConfig, uniform_init, _ = _api()
+    layer = REGISTRY.get_layer("random")(64, 40, REGISTRY.get_node("dwn"), NodeConfig(input_dim=6, output_dim=1),
+                                         seed=1).cuda()
+    opt = torch.optim.Adam(layer.parameters(), lr=0.01)
+    before = stacked(layer, "luts").copy()
+    x = torch.randint(0, 2, (128, 64), device="cuda").float()
+    target = torch.rand(128, 40, device="cuda")
+    losses = []
+    for _ in range(5):
+        opt.zero_grad()
+        loss = ((layer(x) - target) ** 2).mean()
+        loss.backward()
+        opt.step()
+        losses.append(loss.item())
+    assert losses[-1] < losses[0] and not np.array_equal(before, stacked(layer, "luts"))
+    assert layer._banks["luts"].tied()
+
+
+# ------------------------------------------------------------------------------ benchmark shape
+def test_full_size_properties_dwn_k6_b4096_n8192():
+    from difflut_amd import ops
+    torch.manual_seed(0)
+    B, I, N, k = 4096, 16384, 8192, 6
+    x = torch.bernoulli(torch.full((B, I), 0.5, device="cuda"))
+    idx = orc.random_mapping(I, N, k, seed=42)
+    plan = ops.MappingPlan(idx.cuda(), I)
+    luts = (torch.rand(N, 1, 64, device="cuda") * 2 - 1).requires_grad_()
+    gy = torch.randn(B, N, device="cuda")
+    alpha, beta = 0.5 * 0.75 ** 5, 1 / 3
+    xg = x.clone().requires_grad_()
+    y = ops.DWNLayerFunction.apply(xg, luts, plan, alpha, beta)
+    y.backward(gy)
+    gx1, gl1 = xg.grad.clone(), luts.grad.clone()
+    # every output is one of the node's own table entries, and the lookup is deterministic
+    lo, hi = luts.detach().amin(dim=(1, 2)), luts.detach().amax(dim=(1, 2))
+    assert bool(((y.detach() >= lo) & (y.detach() <= hi)).all())
+    y2 = ops.DWNLayerFunction.apply(x, luts.detach(), plan, alpha, beta)
+    assert torch.equal(y.detach(), y2)
+    # table gradient conserves the upstream gradient per node: sum_e gl[n,e] = sum_b gy[b,n]
+    torch.testing.assert_close(gl1.sum(dim=(1, 2)), gy.sum(dim=0), rtol=1e-4, atol=2e-3)
+    # backward is linear in gy; the input gradient is run-to-run identical (fixed summation order)
+    xg2 = x.clone().requires_grad_(); l2 = luts.detach().clone().requires_grad_()
+    ops.DWNLayerFunction.apply(xg2, l2, plan, alpha, beta).backward(2.0 * gy)
+    assert torch.equal(xg2.grad, 2.0 * gx1)
+    torch.testing.assert_close(l2.grad, 2.0 * gl1, rtol=1e-5, atol=1e-4)
+    # first rows against the C restatement of the reference loops
+    rows = 24
+    xs, idn = x[:rows].cpu().numpy(), idx.numpy()
+    ln = luts.detach().cpu().numpy()
+    assert np.array_equal(y[:rows].detach().cpu().numpy(), c_oracle.dwn_layer_forward(xs, idn, ln)[:, :, 0])
+    cgx, _ = c_oracle.dwn_layer_backward(xs, idn, ln, gy[:rows].cpu().numpy()[:, :, None], np.float32(alpha),
+                                         np.float32(beta))
+    np.testing.assert_allclose(gx1[:rows].cpu().numpy(), cgx, rtol=1e-5, atol=2e-6)
+    # the table gradient is a histogram of gy by address: recompute it from the outputs' addresses
+    addr = torch.zeros(B, N, dtype=torch.long, device="cuda")
+    for j in range(k):
+        addr |= (x[:, idx[:, j].long().cuda()] >= 0.5).long() << j
+    want = torch.zeros(N, 64, device="cuda", dtype=torch.float64)
+    want.scatter_add_(1, addr.t().contiguous(), gy.t().double().contiguous())
+    torch.testing.assert_close(gl1[:, 0, :].double(), want, rtol=1e-5, atol=1e-4)

@@ -1,0 +1,159 @@
+"""CPU-only checks: the C-ABI library exports every declared symbol, the host-side mirror of the
+reference interface builds the same state (mapping table, per-node tables, generator position,
+state-dict keys) and refuses to compute on CPU tensors."""
+import ctypes
+import os
+import re
+import warnings
+
+import numpy as np
+import pytest
+import torch
+
+warnings.filterwarnings("ignore")
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    from difflut_amd import _native as nat
+
+    if not nat.is_built():
+        import difflut_amd.build as b
+        b.build()
+    header = open(os.path.join(ROOT, "include", "difflut_hip.h")).read()
+    declared = set(re.findall(r"\b(dl_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(nat.SIGNATURES), declared ^ set(nat.SIGNATURES)
+    handle = ctypes.CDLL(nat.LIB_PATH)
+    for name in declared:
+        assert hasattr(handle, name), name
+    assert handle.dl_version() >= 100
+    nat.lib()
+    assert nat.lib().dl_error_string(-4).decode().startswith("workspace")
+    # size queries are host-only arithmetic: callable without a GPU
+    assert nat.lib().dl_dwn_saved_bytes(4096, 16384, 8192, 6, 1) == 4096 * 8192
+    assert nat.lib().dl_dwn_fwd_workspace_bytes(4096, 16384, 8192, 6, 1) == 64 * 16384 * 8
+
+
+def test_registry_names_and_errors():
+    from difflut_amd import REGISTRY
+    from difflut_amd.layers import LearnableLayer, RandomLayer
+    from difflut_amd.nodes import DWNNode, ProbabilisticNode
+
+    assert REGISTRY.get_node("dwn") is DWNNode and REGISTRY.get_node("probabilistic") is ProbabilisticNode
+    assert REGISTRY.get_layer("random") is RandomLayer and REGISTRY.get_layer("learnable") is LearnableLayer
+    assert "thermometer" in REGISTRY.list_encoders() and "uniform" in REGISTRY.list_initializers()
+    with pytest.raises(ValueError, match="not found"):
+        REGISTRY.get_node("nope")
+    enc = REGISTRY.build_encoder("thermometer", num_bits=3)
+    assert enc.num_bits == 3 and not enc.is_fitted
+
+
+@pytest.mark.parametrize("tag", ["fused_a", "fused_b", "layer_fn", "exact3", "cfg1", "nocover"])
+def test_random_layer_construction_matches_reference(golden, tag):
+    from difflut_amd.layers import RandomLayer
+    from difflut_amd.nodes import DWNNode, NodeConfig
+
+    I, N, k, seed, cover = (int(v) for v in golden[f"map_{tag}_meta"])
+    torch.manual_seed(1234)
+    layer = RandomLayer(I, N, DWNNode, NodeConfig(input_dim=k, output_dim=1), seed=seed,
+                        ensure_full_input_coverage=bool(cover))
+    assert layer._mapping_indices.dtype == torch.int16
+    assert np.array_equal(layer._mapping_indices.numpy(), golden[f"map_{tag}_idx"])
+    assert np.array_equal(layer.nodes[0].luts.detach().numpy(), golden[f"map_{tag}_lut_first"])
+    assert np.array_equal(layer.nodes[N - 1].luts.detach().numpy(), golden[f"map_{tag}_lut_last"])
+    assert np.array_equal(torch.rand(4).numpy(), golden[f"map_{tag}_next_rand"])  # generator position
+    assert layer.n == k and layer.output_dim_per_node == 1 and len(layer.nodes) == N
+
+
+def test_state_dict_keys_and_parameter_views():
+    from difflut_amd.layers import LearnableLayer, RandomLayer
+    from difflut_amd.nodes import DWNNode, NodeConfig, ProbabilisticNode
+
+    layer = RandomLayer(20, 6, DWNNode, NodeConfig(input_dim=3, output_dim=2), seed=1)
+    keys = set(layer.state_dict().keys())
+    assert {"_mapping_indices", "nodes.0.luts", "nodes.0.alpha", "nodes.0.beta", "nodes.5.luts"} <= keys
+    assert layer.nodes[2].luts.shape == (2, 8) and len(list(layer.parameters())) == 6
+    flat = layer._banks["luts"].tensor()
+    with torch.no_grad():
+        layer.nodes[4].luts.fill_(0.25)  # a per-node parameter is a view of the layer's table tensor
+    assert torch.all(flat[4] == 0.25)
+    other = RandomLayer(20, 6, DWNNode, NodeConfig(input_dim=3, output_dim=2), seed=1)
+    other.load_state_dict(layer.state_dict())
+    assert torch.equal(other._banks["luts"].tensor().detach(), flat.detach())
+    # gradients: one tensor for the layer, per-node .grad are its rows; zero_grad clears it
+    flat.grad = torch.ones_like(flat)
+    assert torch.all(layer.nodes[1].luts.grad == 1)
+    opt = torch.optim.SGD(layer.parameters(), lr=0.5)
+    opt.step()
+    assert torch.allclose(layer.nodes[4].luts.detach(), torch.full((2, 8), -0.25))
+    opt.zero_grad()
+    assert layer.nodes[1].luts.grad is None and flat.grad is None
+    moved = layer.double()  # Module._apply re-allocates every parameter: the layer re-ties them
+    assert moved._banks["luts"].tied() and moved.nodes[4].luts.dtype == torch.float64
+
+    p = RandomLayer(16, 4, ProbabilisticNode, NodeConfig(input_dim=2, output_dim=1), seed=1)
+    assert {"nodes.0.raw_weights", "nodes.0.temperature", "nodes.0.binary_combinations"} <= set(p.state_dict())
+    assert p.nodes[0].raw_weights.shape == (4, 1)
+    assert p.nodes[0].binary_combinations.tolist() == [[0, 0], [1, 0], [0, 1], [1, 1]]  # LSB first
+    torch.manual_seed(3)
+    l = LearnableLayer(20, 7, DWNNode, NodeConfig(input_dim=3, output_dim=1), tau=1.0, tau_start=1.0, tau_min=1e-4,
+                       tau_decay_iters=1000.0, use_cuda_soft=False)
+    assert l.mapping.W.shape == (21, 20) and "mapping.W" in l.state_dict()
+    l.update_tau(500)
+    assert l.tau == pytest.approx(10 ** -0.5) and l.mapping.tau == l.tau
+    l.update_tau(10 ** 9)
+    assert l.tau == 1e-4
+
+
+def test_learnable_layer_W_matches_reference_draw(golden):
+    from difflut_amd.layers import LearnableLayer
+    from difflut_amd.nodes import DWNNode, NodeConfig
+
+    torch.manual_seed(3)
+    l = LearnableLayer(20, 7, DWNNode, NodeConfig(input_dim=3, output_dim=1), tau=1.0, tau_start=1.0, tau_min=1e-4,
+                       tau_decay_iters=1000.0, use_cuda_soft=False)
+    assert np.array_equal(l.mapping.W.detach().numpy(), golden["soft_W"])
+
+
+def test_constructor_validation_and_cpu_refusal():
+    from difflut_amd.layers import LayerConfig, RandomLayer
+    from difflut_amd.nodes import DWNNode, NodeConfig
+    from difflut_amd.utils import GroupSum
+
+    cfg = NodeConfig(input_dim=2, output_dim=1)
+    with pytest.raises(ValueError):
+        RandomLayer(0, 4, DWNNode, cfg)
+    with pytest.raises(ValueError):
+        RandomLayer(8, -1, DWNNode, cfg)
+    with pytest.raises(ValueError):
+        DWNNode(input_dim=0, output_dim=1)
+    with pytest.raises(TypeError):
+        DWNNode(input_dim=2, output_dim=1, init_fn=3)
+    with pytest.raises(ValueError):
+        LayerConfig(flip_probability=1.5)
+    with pytest.raises(TypeError):
+        RandomLayer(8, 4, DWNNode, cfg, layer_config={"flip_probability": 0.1})
+    with pytest.raises(ValueError):
+        GroupSum(k=0)
+    layer = RandomLayer(8, 4, DWNNode, cfg)
+    with pytest.raises(ValueError, match="2D input"):
+        layer(torch.zeros(8))
+    with pytest.raises(ValueError, match="expected input with 8 features"):
+        layer(torch.zeros(2, 9))
+    with pytest.raises(RuntimeError, match="ROCm devices only"):
+        layer(torch.zeros(2, 8))  # no CPU fallback
+    assert DWNNode(input_dim=6, output_dim=1).alpha.item() == pytest.approx(0.5 * 0.75 ** 5)
+
+
+def test_residual_initialiser_known_answer(golden):
+    from difflut_amd.nodes import DWNNode, ProbabilisticNode
+    from difflut_amd.nodes.utils import residual_init
+
+    kw = {"node_type": "dwn", "noise_factor": 0.0, "logit_clarity": 5.0, "input_dim": 6}
+    node = DWNNode(input_dim=6, output_dim=1, init_fn=residual_init, init_kwargs=kw)
+    assert np.array_equal(node.luts.detach().numpy(), golden["dwn_residual_luts"])
+    p = ProbabilisticNode(input_dim=3, output_dim=2, init_fn=residual_init,
+                          init_kwargs={"node_type": "probabilistic", "noise_factor": 0.0, "logit_clarity": 5.0,
+                                       "input_dim": 3})
+    assert p.raw_weights[:, 0].tolist() == [-5, 5, -5, 5, -5, 5, -5, 5]
