@@ -11,7 +11,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libdifflut_hip.so")
+# DIFFLUT_HIP_LIB points at another build of the same library (kernel experiments)
+LIB_PATH = os.environ.get("DIFFLUT_HIP_LIB") or os.path.join(_HERE, "lib", "libdifflut_hip.so")
 
 _P, _I, _F, _Z = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
 

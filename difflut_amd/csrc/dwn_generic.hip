@@ -1,0 +1,120 @@
+// RandomLayer + DWN nodes, generic kernels: any k up to DL_MAX_K, one thread per element, x read
+// directly, atomics for the table gradient.  Used when tables do not fit a wavefront (k > 6) and
+// for the eval-mode forward; the fast path for k <= 6 is in dwn_kernels.hip.
+#include "dl_common.h"
+#include "dwn_generic.h"
+
+// Generic kernels (any k up to DL_MAX_K): one thread per element, x read directly.
+__device__ __forceinline__ unsigned dwn_addr_generic(const float *xrow, const int *ix, int K) {
+    unsigned a = 0;
+    for (int j = 0; j < K; ++j) a |= (xrow[ix[j]] >= 0.5f ? 1u : 0u) << j;
+    return a;
+}
+
+__global__ __launch_bounds__(256) void dwn_generic_fwd(const float *__restrict__ x, const int *__restrict__ idx32,
+                                                        const float *__restrict__ luts, float *__restrict__ y,
+                                                        int B, int I, int N, int K, int O) {
+    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long NO = (long long)N * O;
+    if (gid >= (long long)B * NO) return;
+    const int b = (int)(gid / NO);
+    const long long c = gid % NO;
+    const int n = (int)(c / O);
+    const unsigned a = dwn_addr_generic(x + (size_t)b * I, idx32 + (size_t)n * K, K);
+    y[gid] = luts[(c << K) + a];
+}
+
+__global__ __launch_bounds__(256) void dwn_generic_bwd_gx(const float *__restrict__ x, const int *__restrict__ idx32,
+                                                           const int *__restrict__ inv_ptr, const int *__restrict__ inv_pos,
+                                                           const float *__restrict__ luts, const float *__restrict__ gy,
+                                                           float alpha, float beta, float *__restrict__ gx,
+                                                           int B, int I, int N, int K, int O) {
+    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= (long long)B * I) return;
+    const int b = (int)(gid / I), i = (int)(gid % I);
+    const int L = 1 << K;
+    double bp[DL_MAX_K + 1];
+    bp[0] = 1.0;
+    for (int h = 1; h <= K; ++h) bp[h] = bp[h - 1] * (double)beta;
+    float acc = 0.0f;
+    for (int e = inv_ptr[i]; e < inv_ptr[i + 1]; ++e) {
+        const int p = inv_pos[e];
+        const int n = p / K, j = p - n * K;
+        const unsigned a = dwn_addr_generic(x + (size_t)b * I, idx32 + (size_t)n * K, K);
+        const unsigned keep = ~(1u << j);
+        for (int d = 0; d < O; ++d) {
+            const float *lut = luts + (((size_t)n * O + d) << K);
+            double s = 0.0;
+            for (int kap = 0; kap < L; ++kap) {
+                const double w = bp[__popc((a ^ (unsigned)kap) & keep)];
+                s += (((unsigned)kap >> j) & 1u) ? (double)lut[kap] * w : -(double)lut[kap] * w;
+            }
+            acc += gy[((size_t)b * N + n) * O + d] * (float)((double)alpha * s);
+        }
+    }
+    gx[gid] = acc;
+}
+
+__global__ __launch_bounds__(256) void dwn_generic_bwd_luts(const float *__restrict__ x, const int *__restrict__ idx32,
+                                                             const float *__restrict__ gy, float *__restrict__ gluts,
+                                                             int B, int I, int N, int K, int O) {
+    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long NO = (long long)N * O;
+    if (gid >= (long long)B * NO) return;
+    const int b = (int)(gid / NO);
+    const long long c = gid % NO;
+    const int n = (int)(c / O);
+    const unsigned a = dwn_addr_generic(x + (size_t)b * I, idx32 + (size_t)n * K, K);
+    atomicAdd(&gluts[(c << K) + a], gy[gid]);
+}
+
+// Eval: address = floor(sum_j x_j 2^j), no thresholding of x; table value binarised at 0.5.
+__global__ __launch_bounds__(256) void dwn_eval_fwd(const float *__restrict__ x, const int *__restrict__ idx32,
+                                                     const float *__restrict__ luts, float *__restrict__ y,
+                                                     int B, int I, int N, int K, int O) {
+    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long NO = (long long)N * O;
+    if (gid >= (long long)B * NO) return;
+    const int b = (int)(gid / NO);
+    const long long c = gid % NO;
+    const int n = (int)(c / O);
+    const float *xrow = x + (size_t)b * I;
+    const int *ix = idx32 + (size_t)n * K;
+    float s = 0.0f;
+    for (int j = 0; j < K; ++j) s += xrow[ix[j]] * (float)(1 << j);
+    long long a = (long long)s;  // truncation, as tensor.long()
+    a = a < 0 ? 0 : (a > (1 << K) - 1 ? (1 << K) - 1 : a);
+    y[gid] = luts[(c << K) + a] >= 0.5f ? 1.0f : 0.0f;
+}
+
+__global__ __launch_bounds__(256) void dwn_generic_zero(float *p, long long n) {
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0.0f;
+}
+
+int dwn_generic_forward(const float *x, const int *idx32, const float *luts, float *y, int B, int I, int N, int k, int O,
+                        hipStream_t s) {
+    dwn_generic_fwd<<<dl_ceil_div((long long)B * N * O, 256), 256, 0, s>>>(x, idx32, luts, y, B, I, N, k, O);
+    return dl_launch_status();
+}
+
+int dwn_generic_backward(const float *x, const int *idx32, const int *inv_ptr, const int *inv_pos, const float *luts,
+                         const float *gy, float alpha, float beta, float *gx, float *gluts, int B, int I, int N, int k,
+                         int O, hipStream_t s) {
+    const long long NO = (long long)N * O;
+    dwn_generic_zero<<<dl_ceil_div(NO << k, 256), 256, 0, s>>>(gluts, NO << k);
+    dwn_generic_bwd_luts<<<dl_ceil_div((long long)B * NO, 256), 256, 0, s>>>(x, idx32, gy, gluts, B, I, N, k, O);
+    if (gx)
+        dwn_generic_bwd_gx<<<dl_ceil_div((long long)B * I, 256), 256, 0, s>>>(x, idx32, inv_ptr, inv_pos, luts, gy, alpha,
+                                                                            beta, gx, B, I, N, k, O);
+    return dl_launch_status();
+}
+
+extern "C" int dl_dwn_layer_eval(const float *x, const int32_t *idx32, const float *luts, float *y, int B, int I, int N,
+                                 int k, int O, void *stream) {
+    if (!x || !idx32 || !luts || !y) return DL_ERR_NULL;
+    if (B <= 0 || I <= 0 || N <= 0 || k <= 0 || O <= 0) return DL_ERR_SHAPE;
+    if (k > DL_MAX_K) return DL_ERR_UNSUPPORTED;
+    dwn_eval_fwd<<<dl_ceil_div((long long)B * N * O, 256), 256, 0, (hipStream_t)stream>>>(x, idx32, luts, y, B, I, N, k, O);
+    return dl_launch_status();
+}

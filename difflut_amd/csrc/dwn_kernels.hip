@@ -5,23 +5,33 @@
 // belongs to a node - its k input indices, its 2^k-entry table, its EFD coefficient
 // rows - is then wave-uniform: indices and bit-plane words come through scalar loads,
 // a table sits one entry per lane in a single VGPR and a lookup is one ds_bpermute.
-// The random RandomLayer mapping costs nothing in this layout; what it costs instead
-// is one transpose through LDS wherever a tensor crosses the [batch, feature] boundary
-// (y out, gy in, gx out).
+// The random RandomLayer mapping costs nothing in this layout (it is scalar addressing);
+// what it costs instead is one transpose through LDS wherever a tensor crosses the
+// [batch, feature] boundary (y out, gy in, gx out).
 //
 //   forward   pack_planes : x [B,I] fp32 -> planes [B/64][I] u64 (bit r = x[64t+r][i] >= 0.5)
 //             lookup_fwd  : planes + idx + luts -> y [B,N*O] (LDS-transposed tiles) and
-//                           addrT [N][B] u8, the address of every (node,row), kept for backward
+//                           addrT [B/64][N][64] u8, the address of every (node,row), kept for backward
 //   backward  efd_table   : luts -> D[n][d][j][a'] = alpha * sum_kappa s(kappa_j) lut[kappa]
-//                           beta^popc((a^kappa)&~(1<<j)), a' = address with bit j squeezed out
-//             transpose_hist : gy [B,N*O] -> gyT [N*O][B]; per-node 2^k-bin histogram of gy
+//                           beta^popc((a^kappa)&~(1<<j)), a' = address with bit j squeezed out;
+//                           also clears the table-gradient output
+//             transpose_hist : gy [B,N*O] -> gyT [B/64][N*O][64]; per-node 2^k-bin histogram of gy
 //                           in LDS, one float atomic per bin per block into gluts
 //             bwd_gx      : for every input i the (node,slot) pairs that read it (CSR):
 //                           gx[b,i] = sum gyT[c][b] * D[c][j][a'(b)]  - a gather in fixed order
-// k > 6 falls back to plain one-thread-per-element kernels further down.
+// k > 6 goes to the one-thread-per-element kernels of dwn_generic.hip.
 #include "dl_common.h"
+#include "dwn_generic.h"
 
 typedef unsigned long long u64;
+
+// addr <- 2*addr + (bit `lane` of mask): the 64-bit scalar is used directly as a per-lane carry-in.
+__device__ __forceinline__ unsigned dwn_shift_in(unsigned addr, u64 mask) {
+    unsigned out;
+    u64 carry_out;
+    asm("v_addc_co_u32_e64 %0, %1, %2, %2, %3" : "=v"(out), "=s"(carry_out) : "v"(addr), "s"(mask));
+    return out;
+}
 
 // ---------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void dl_fill_zero_kernel(float *p, long long n) {
@@ -80,243 +90,299 @@ __global__ __launch_bounds__(256) void dwn_pack_planes(const float *__restrict__
 
 // ---------------------------------------------------------------------------------
 // lookup_fwd: grid (ceil(N*O / 128), B/64), 256 threads = 4 wavefronts, lane = batch row.
+// A wavefront walks 32 consecutive columns (column = node*O + output) in groups of 4 so that the
+// two dependent scalar loads per input (index, then bit-plane word) of a whole group are in flight
+// together.  Per column: k add-with-carry steps build the address, one bpermute reads the table.
 #define DWN_TC 128
-template <int K>
+#define DWN_CG 4
+template <int K, bool O1>
 __global__ __launch_bounds__(256) void dwn_lookup_fwd(const u64 *__restrict__ planes, const int *__restrict__ idx32,
                                                        const float *__restrict__ luts, float *__restrict__ y,
-                                                       uint8_t *__restrict__ addrT, int B, int I, int N, int O, int BP) {
-    __shared__ float tile[64][DWN_TC + 1];
+                                                       uint8_t *__restrict__ addrT, int B, int I, int N, int O, int BT) {
+    __shared__ float tile[DWN_TC][65];  // [column][row]
     constexpr int L = 1 << K;
-    const int t = blockIdx.y;
-    const int c0 = blockIdx.x * DWN_TC;
     const int NO = N * O;
+    int ctile, t;
+    if (!dl_xcd_map((NO + DWN_TC - 1) / DWN_TC, BT, ctile, t)) return;
+    const int c0 = ctile * DWN_TC;
     const int lane = threadIdx.x & 63;
     const int wave = dl_uniform(threadIdx.x >> 6);
     const u64 *pl = planes + (size_t)t * I;
     const int cend = min(DWN_TC, NO - c0);
-    for (int cc = wave; cc < cend; cc += 4) {
-        const int c = c0 + cc;
-        const int n = c / O;
-        unsigned addr = 0;
+    const int wbeg = wave * (DWN_TC / 4);
+    for (int g = 0; g < DWN_TC / 4; g += DWN_CG) {
+        if (wbeg + g >= cend) break;
+        int node[DWN_CG], src[DWN_CG][K];
+        u64 w[DWN_CG][K];
+        float entry[DWN_CG];
 #pragma unroll
-        for (int j = 0; j < K; ++j) {
-            const int src = idx32[n * K + j];  // wave-uniform: scalar load
-            const u64 w = pl[src];             // wave-uniform: scalar load
-            const unsigned half = lane < 32 ? (unsigned)w : (unsigned)(w >> 32);
-            addr |= ((half >> (lane & 31)) & 1u) << j;
+        for (int q = 0; q < DWN_CG; ++q) {
+            const int c = min(c0 + wbeg + g + q, NO - 1);  // clamp: loads of a ragged last group stay in range
+            node[q] = O1 ? c : c / O;
+#pragma unroll
+            for (int j = 0; j < K; ++j) src[q][j] = idx32[node[q] * K + j];
+            entry[q] = luts[(size_t)c * L + (lane & (L - 1))];
         }
-        const float entry = luts[(size_t)c * L + (lane & (L - 1))];  // table, one entry per lane
-        tile[lane][cc] = dl_lane_read(entry, (int)addr);
-        if (c - n * O == 0) addrT[(size_t)n * BP + t * 64 + lane] = (uint8_t)addr;
+#pragma unroll
+        for (int q = 0; q < DWN_CG; ++q)
+#pragma unroll
+            for (int j = 0; j < K; ++j) w[q][j] = pl[src[q][j]];
+#pragma unroll
+        for (int q = 0; q < DWN_CG; ++q) {
+            const int cc = wbeg + g + q;
+            unsigned addr = 0;
+#pragma unroll
+            for (int j = K - 1; j >= 0; --j) addr = dwn_shift_in(addr, w[q][j]);
+            const float v = dl_lane_read(entry[q], (int)addr);
+            if (cc < cend) {
+                tile[cc][lane] = v;
+                if (O1 || (c0 + cc) - node[q] * O == 0) addrT[((size_t)t * N + node[q]) * 64 + lane] = (uint8_t)addr;
+            }
+        }
     }
     __syncthreads();
     for (int e = threadIdx.x; e < 64 * DWN_TC; e += 256) {
         const int r = e / DWN_TC, cc = e % DWN_TC;
         const int b = t * 64 + r;
-        if (b < B && cc < cend) y[(size_t)b * NO + c0 + cc] = tile[r][cc];
+        if (b < B && cc < cend) y[(size_t)b * NO + c0 + cc] = tile[cc][r];
     }
 }
 
 // ---------------------------------------------------------------------------------
-// efd_table: one thread per coefficient.  Double accumulation, one rounding to float.
+// efd_table: one wavefront per table (column), lane = table entry.  For every input j the table is
+// smoothed along all other inputs (v <- v + beta * v[entry ^ bit]) and differenced along j; lanes
+// whose bit j is clear hold the coefficient.  Double precision, one rounding to float.  The same
+// wavefront clears the table's gradient row.
 __global__ __launch_bounds__(256) void dwn_efd_table(const float *__restrict__ luts, float *__restrict__ D,
-                                                      int NO, int K, float alpha, float beta) {
-    const int Lh = 1 << (K - 1), L = 1 << K;
-    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (gid >= (long long)NO * K * Lh) return;
-    const int ap = (int)(gid % Lh);
-    const int j = (int)((gid / Lh) % K);
-    const long long c = gid / ((long long)Lh * K);
-    const unsigned a = ((unsigned)ap & ((1u << j) - 1u)) | (((unsigned)ap >> j) << (j + 1));  // bit j = 0
-    double bp[DL_MAX_FAST_K + 1];
-    bp[0] = 1.0;
-#pragma unroll
-    for (int h = 1; h <= DL_MAX_FAST_K; ++h) bp[h] = bp[h - 1] * (double)beta;
-    const unsigned keep = ~(1u << j);
-    const float *lut = luts + c * L;
-    double acc = 0.0;
-    for (int kap = 0; kap < L; ++kap) {
-        const int h = __popc((a ^ (unsigned)kap) & keep);
-        double w = 1.0;
-#pragma unroll
-        for (int q = 1; q <= DL_MAX_FAST_K; ++q) w = (h == q) ? bp[q] : w;
-        acc += (((unsigned)kap >> j) & 1u) ? (double)lut[kap] * w : -(double)lut[kap] * w;
+                                                      float *__restrict__ gluts, int NO, int K, float alpha, float beta) {
+    const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int a = threadIdx.x & 63;
+    if (c >= NO) return;
+    const int L = 1 << K, Lh = L >> 1;
+    const bool live = a < L;
+    const double v0 = live ? (double)luts[(size_t)c * L + a] : 0.0;
+    if (live) gluts[(size_t)c * L + a] = 0.0f;
+    for (int j = 0; j < K; ++j) {
+        double v = v0;
+        for (int m = 0; m < K; ++m) {
+            const double other = __shfl_xor(v, 1 << m);
+            if (m != j) v += (double)beta * other;
+        }
+        const double upper = __shfl_xor(v, 1 << j);
+        if (live && !((a >> j) & 1)) {
+            const int ap = (a & ((1 << j) - 1)) | ((a >> (j + 1)) << j);
+            D[((size_t)c * K + j) * Lh + ap] = (float)((double)alpha * (upper - v));
+        }
     }
-    D[gid] = (float)((double)alpha * acc);
 }
 
 // ---------------------------------------------------------------------------------
-// transpose_hist: grid (ceil(N*O / 128), chunks), block streams `tiles_per_chunk` 64-row tiles.
+// transpose_hist: grid (ceil(N*O / 64), chunks); a block streams `tiles_per_chunk` 64-row tiles
+// of its 64 columns.  The next tile (gy values and their addresses) is prefetched into registers
+// while the current one sits in LDS.  Each wavefront owns 16 of the columns:
+//   * lane = batch row: reads a column of the LDS tile and stores 256 contiguous bytes of gyT;
+//   * lane = (column, row mod 4): adds gy into the column's 2^k-bin histogram with a plain LDS
+//     read-modify-write - the four lanes of a column are one quad, so equal addresses inside a
+//     step are merged with quad permutes first and no two lanes of the block ever update the same
+//     word at once (float atomics in LDS are far slower than this).
+#define DWN_HC 64
+__device__ __forceinline__ float dwn_quad_read(float v, int src) {  // value of lane (quad base + src)
+    return __int_as_float(__builtin_amdgcn_ds_bpermute(((threadIdx.x & ~3) | src) << 2, __float_as_int(v)));
+}
 template <bool WRITE_T>
 __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__restrict__ gy, const uint8_t *__restrict__ addrT,
                                                                float *__restrict__ gyT, float *__restrict__ gluts,
                                                                int B, int NO, int O, int L, int BP, int BT,
                                                                int tiles_per_chunk) {
-    __shared__ float tile[64][DWN_TC + 1];
-    __shared__ float hist[DWN_TC * 64];
-    const int c0 = blockIdx.x * DWN_TC;
+    __shared__ float tile[64][DWN_HC + 1];       // [row][column]
+    __shared__ float hist[DWN_HC][65];           // [column][bin]
+    __shared__ uint8_t atile[DWN_HC][64 + 4];    // [column][row] addresses
+    const int c0 = blockIdx.x * DWN_HC;
     const int lane = threadIdx.x & 63;
     const int wave = dl_uniform(threadIdx.x >> 6);
-    const int cend = min(DWN_TC, NO - c0);
-    for (int e = threadIdx.x; e < DWN_TC * 64; e += 256) hist[e] = 0.0f;
+    const int cend = min(DWN_HC, NO - c0);
+    for (int e = threadIdx.x; e < DWN_HC * 65; e += 256) (&hist[0][0])[e] = 0.0f;
     const int t_begin = blockIdx.y * tiles_per_chunk;
     const int t_end = min(BT, t_begin + tiles_per_chunk);
-    const bool vec4 = (NO % 4 == 0);
-    for (int t = t_begin; t < t_end; ++t) {
-        __syncthreads();
-        if (vec4) {  // 32 threads x 16 B cover one 128-column row piece; 8 rows per pass
-            const int q = threadIdx.x & 31, rr = threadIdx.x >> 5;
+    const bool vec4 = (NO % 4 == 0) && cend == DWN_HC;
+    const int q = threadIdx.x & 15, rr = threadIdx.x >> 4;  // 16 threads x 16 B cover one 64-column row piece
+    const int N = NO / O;
+    const int wc0 = wave * (DWN_HC / 4);  // my wavefront's first column
+    float4 pre[4];
+    unsigned apre[DWN_HC / 4];  // addresses of my 16 columns for the tile being fetched (lane = row)
+    auto fetch = [&](int t) {
 #pragma unroll
-            for (int r8 = 0; r8 < 64; r8 += 8) {
-                const int r = r8 + rr, b = t * 64 + r, cc = q * 4;
-                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (b < B && cc < cend) v = *reinterpret_cast<const float4 *>(gy + (size_t)b * NO + c0 + cc);
-                tile[r][cc] = v.x; tile[r][cc + 1] = v.y; tile[r][cc + 2] = v.z; tile[r][cc + 3] = v.w;
-            }
-        } else {
-            for (int e = threadIdx.x; e < 64 * DWN_TC; e += 256) {
-                const int r = e / DWN_TC, cc = e % DWN_TC;
-                const int b = t * 64 + r;
-                tile[r][cc] = (b < B && cc < cend) ? gy[(size_t)b * NO + c0 + cc] : 0.0f;
+        for (int p = 0; p < 4; ++p) {
+            const int b = t * 64 + rr + 16 * p;
+            pre[p] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (b < B) {
+                const float *src = gy + (size_t)b * NO + c0 + q * 4;
+                if (vec4) {
+                    pre[p] = *reinterpret_cast<const float4 *>(src);
+                } else {
+                    if (q * 4 + 0 < cend) pre[p].x = src[0];
+                    if (q * 4 + 1 < cend) pre[p].y = src[1];
+                    if (q * 4 + 2 < cend) pre[p].z = src[2];
+                    if (q * 4 + 3 < cend) pre[p].w = src[3];
+                }
             }
         }
+#pragma unroll
+        for (int u = 0; u < DWN_HC / 4; ++u) {
+            const int c = min(c0 + wc0 + u, NO - 1);
+            apre[u] = addrT[((size_t)t * N + c / O) * 64 + lane];
+        }
+    };
+    if (t_begin < t_end) fetch(t_begin);
+    const int hc = wc0 + (lane >> 2), hr = lane & 3;  // histogram role: column and row phase of this lane
+    for (int t = t_begin; t < t_end; ++t) {
+        __syncthreads();  // previous tile fully consumed (and hist cleared on the first pass)
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            float *dst = &tile[rr + 16 * p][q * 4];
+            dst[0] = pre[p].x; dst[1] = pre[p].y; dst[2] = pre[p].z; dst[3] = pre[p].w;
+        }
+#pragma unroll
+        for (int u = 0; u < DWN_HC / 4; ++u) atile[wc0 + u][lane] = (uint8_t)apre[u];
         __syncthreads();
-        for (int cc = wave; cc < cend; cc += 4) {
-            const int c = c0 + cc;
-            const int n = c / O;
-            const float v = tile[lane][cc];
-            if (WRITE_T) gyT[(size_t)c * BP + t * 64 + lane] = v;
-            const unsigned a = addrT[(size_t)n * BP + t * 64 + lane];
-            atomicAdd(&hist[cc * L + a], v);  // rows past B carry v = 0
+        if (t + 1 < t_end) fetch(t + 1);
+        if (WRITE_T) {
+#pragma unroll
+            for (int u = 0; u < DWN_HC / 4; ++u) {
+                const int cc = wc0 + u;
+                if (cc < cend) gyT[((size_t)t * NO + c0 + cc) * 64 + lane] = tile[lane][cc];
+            }
+        }
+        if (hc < cend) {  // whole quads share hc, so the quad permutes below stay inside active lanes
+            for (int r0 = 0; r0 < 64; r0 += 4) {
+                const float v = tile[r0 + hr][hc];  // rows past B carry 0
+                const unsigned a = atile[hc][r0 + hr];
+                float sum = v;
+                bool leader = true;
+#pragma unroll
+                for (int o = 1; o < 4; ++o) {  // the other three lanes of my quad
+                    const int other = hr ^ o;
+                    const unsigned ao = (unsigned)__float_as_int(dwn_quad_read(__int_as_float((int)a), other));
+                    const float vo = dwn_quad_read(v, other);
+                    if (ao == a) {
+                        sum += vo;
+                        if (other < hr) leader = false;
+                    }
+                }
+                if (leader) hist[hc][a] += sum;
+            }
         }
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < cend * L; e += 256) atomicAdd(&gluts[(size_t)c0 * L + e], hist[e]);
+    for (int e = threadIdx.x; e < cend * L; e += 256) atomicAdd(&gluts[(size_t)c0 * L + e], hist[e / L][e % L]);
 }
 
 // ---------------------------------------------------------------------------------
-// bwd_gx: grid (ceil(I / 128), B/64), lane = batch row, wavefront walks inputs of the slab.
+// bwd_gx: grid (ceil(I / 128), B/64), lane = batch row.  A wavefront owns 32 consecutive inputs, i.e.
+// one contiguous run of CSR entries.  The run is read 64 entries at a time into registers (one
+// entry per lane: node, slot, local input), then replayed 8 entries per step with wave-uniform
+// addressing so that the 8 x 3 vector loads of a step are in flight together.  The entries of one input are
+// consecutive, so its sum is kept in a register and written to the LDS tile once (fixed order).
 #define DWN_IS 128
-template <int K>
+#define DWN_EG 8
+template <int K, bool O1>
 __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT, const uint8_t *__restrict__ addrT,
                                                    const float *__restrict__ D, const int *__restrict__ inv_ptr,
                                                    const int *__restrict__ inv_pos, float *__restrict__ gx,
-                                                   int B, int I, int O, int BP) {
-    __shared__ float tile[DWN_IS][65];
+                                                   int B, int I, int N, int O, int BT) {
+    __shared__ float tile[DWN_IS][65];  // [input][row]
     constexpr int Lh = 1 << (K - 1);
-    const int t = blockIdx.y;
-    const int i0 = blockIdx.x * DWN_IS;
+    int slab, t;
+    if (!dl_xcd_map((I + DWN_IS - 1) / DWN_IS, BT, slab, t)) return;
+    const int i0 = slab * DWN_IS;
+    const int NO = N * O;
     const int lane = threadIdx.x & 63;
     const int wave = dl_uniform(threadIdx.x >> 6);
     const int iend = min(DWN_IS, I - i0);
-    const size_t col = (size_t)t * 64 + lane;
-    for (int ii = wave; ii < iend; ii += 4) {
-        const int e0 = inv_ptr[i0 + ii], e1 = inv_ptr[i0 + ii + 1];
-        float acc = 0.0f;
-        for (int e = e0; e < e1; ++e) {
-            const int p = inv_pos[e];
-            const int n = p / K, j = p - n * K;
-            const unsigned a = addrT[(size_t)n * BP + col];
-            const unsigned ap = (a & ((1u << j) - 1u)) | ((a >> (j + 1)) << j);
-            for (int d = 0; d < O; ++d) {
-                const size_t c = (size_t)n * O + d;
-                const float g = gyT[c * BP + col];
-                const float coef = D[(c * K + j) * Lh + (lane & (Lh - 1))];
-                acc += g * dl_lane_read(coef, (int)ap);
+    const uint8_t *addr_t = addrT + (size_t)t * N * 64 + lane;
+    const float *gy_t = gyT + (size_t)t * NO * 64 + lane;
+    const int wbeg = wave * 32;
+#pragma unroll
+    for (int r = 0; r < 32; ++r) tile[wbeg + r][lane] = 0.0f;
+    if (lane == 0)
+#pragma unroll
+        for (int r = 0; r < 32; ++r) tile[wbeg + r][64] = 0.0f;
+    // CSR pointers of my 32 inputs: lane l (0..32) holds inv_ptr[first + l], clamped at I
+    const int myptr = inv_ptr[min(i0 + wbeg + min(lane, 32), I)];
+    const int ebeg = __builtin_amdgcn_readlane(myptr, 0);
+    const int eend = __builtin_amdgcn_readlane(myptr, 32);
+    float acc = 0.0f;  // running sum of the input `cur` (entries of one input are consecutive)
+    int cur = -1;
+    for (int base = ebeg; base < eend; base += 64) {
+        const int e = base + lane;
+        const bool valid = e < eend;
+        const int p = valid ? inv_pos[e] : 0;
+        int ii = 0;  // local input of entry e = number of my inputs that end at or before e
+#pragma unroll
+        for (int l = 1; l <= 32; ++l) ii += (__builtin_amdgcn_readlane(myptr, l) <= e) ? 1 : 0;
+        const int n = p / K, j = p - n * K;
+        const int rec = valid ? ((n << 8) | (j << 5) | ii) : -1;
+        const int cnt = min(64, eend - base);
+        for (int s0 = 0; s0 < cnt; s0 += DWN_EG) {
+            int rn[DWN_EG], rj[DWN_EG], ri[DWN_EG];
+            bool live[DWN_EG];
+            unsigned a[DWN_EG];
+#pragma unroll
+            for (int q = 0; q < DWN_EG; ++q) {
+                const int r = __builtin_amdgcn_readlane(rec, s0 + q);
+                live[q] = r >= 0;
+                const int rr = r >= 0 ? r : 0;
+                rn[q] = rr >> 8; rj[q] = (rr >> 5) & 7; ri[q] = rr & 31;
+                a[q] = addr_t[(size_t)rn[q] * 64];
+            }
+            if (O1) {
+                float g[DWN_EG], coef[DWN_EG];
+#pragma unroll
+                for (int q = 0; q < DWN_EG; ++q) {
+                    g[q] = gy_t[(size_t)rn[q] * 64];
+                    coef[q] = __builtin_nontemporal_load(&D[((size_t)rn[q] * K + rj[q]) * Lh + (lane & (Lh - 1))]);
+                }
+#pragma unroll
+                for (int q = 0; q < DWN_EG; ++q) {
+                    const unsigned ap = (a[q] & ((1u << rj[q]) - 1u)) | ((a[q] >> (rj[q] + 1)) << rj[q]);
+                    if (live[q]) {  // wave-uniform
+                        if (ri[q] != cur) {
+                            if (cur >= 0) tile[wbeg + cur][lane] = acc;
+                            acc = 0.0f;
+                            cur = ri[q];
+                        }
+                        acc += g[q] * dl_lane_read(coef[q], (int)ap);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int q = 0; q < DWN_EG; ++q) {
+                    const unsigned ap = (a[q] & ((1u << rj[q]) - 1u)) | ((a[q] >> (rj[q] + 1)) << rj[q]);
+                    float term = 0.0f;
+                    for (int d = 0; d < O; ++d) {
+                        const size_t c = (size_t)rn[q] * O + d;
+                        const float coef = D[(c * K + rj[q]) * Lh + (lane & (Lh - 1))];
+                        term += gy_t[c * 64] * dl_lane_read(coef, (int)ap);
+                    }
+                    if (live[q]) {
+                        if (ri[q] != cur) {
+                            if (cur >= 0) tile[wbeg + cur][lane] = acc;
+                            acc = 0.0f;
+                            cur = ri[q];
+                        }
+                        acc += term;
+                    }
+                }
             }
         }
-        tile[ii][lane] = acc;
     }
+    if (cur >= 0) tile[wbeg + cur][lane] = acc;
     __syncthreads();
     for (int e = threadIdx.x; e < 64 * DWN_IS; e += 256) {
         const int r = e / DWN_IS, ii = e % DWN_IS;
         const int b = t * 64 + r;
         if (b < B && ii < iend) gx[(size_t)b * I + i0 + ii] = tile[ii][r];
     }
-}
-
-// ---------------------------------------------------------------------------------
-// Generic kernels (any k up to DL_MAX_K): one thread per element, x read directly.
-__device__ __forceinline__ unsigned dwn_addr_generic(const float *xrow, const int *ix, int K) {
-    unsigned a = 0;
-    for (int j = 0; j < K; ++j) a |= (xrow[ix[j]] >= 0.5f ? 1u : 0u) << j;
-    return a;
-}
-
-__global__ __launch_bounds__(256) void dwn_generic_fwd(const float *__restrict__ x, const int *__restrict__ idx32,
-                                                        const float *__restrict__ luts, float *__restrict__ y,
-                                                        int B, int I, int N, int K, int O) {
-    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
-    const long long NO = (long long)N * O;
-    if (gid >= (long long)B * NO) return;
-    const int b = (int)(gid / NO);
-    const long long c = gid % NO;
-    const int n = (int)(c / O);
-    const unsigned a = dwn_addr_generic(x + (size_t)b * I, idx32 + (size_t)n * K, K);
-    y[gid] = luts[(c << K) + a];
-}
-
-__global__ __launch_bounds__(256) void dwn_generic_bwd_gx(const float *__restrict__ x, const int *__restrict__ idx32,
-                                                           const int *__restrict__ inv_ptr, const int *__restrict__ inv_pos,
-                                                           const float *__restrict__ luts, const float *__restrict__ gy,
-                                                           float alpha, float beta, float *__restrict__ gx,
-                                                           int B, int I, int N, int K, int O) {
-    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (gid >= (long long)B * I) return;
-    const int b = (int)(gid / I), i = (int)(gid % I);
-    const int L = 1 << K;
-    double bp[DL_MAX_K + 1];
-    bp[0] = 1.0;
-    for (int h = 1; h <= K; ++h) bp[h] = bp[h - 1] * (double)beta;
-    float acc = 0.0f;
-    for (int e = inv_ptr[i]; e < inv_ptr[i + 1]; ++e) {
-        const int p = inv_pos[e];
-        const int n = p / K, j = p - n * K;
-        const unsigned a = dwn_addr_generic(x + (size_t)b * I, idx32 + (size_t)n * K, K);
-        const unsigned keep = ~(1u << j);
-        for (int d = 0; d < O; ++d) {
-            const float *lut = luts + (((size_t)n * O + d) << K);
-            double s = 0.0;
-            for (int kap = 0; kap < L; ++kap) {
-                const double w = bp[__popc((a ^ (unsigned)kap) & keep)];
-                s += (((unsigned)kap >> j) & 1u) ? (double)lut[kap] * w : -(double)lut[kap] * w;
-            }
-            acc += gy[((size_t)b * N + n) * O + d] * (float)((double)alpha * s);
-        }
-    }
-    gx[gid] = acc;
-}
-
-__global__ __launch_bounds__(256) void dwn_generic_bwd_luts(const float *__restrict__ x, const int *__restrict__ idx32,
-                                                             const float *__restrict__ gy, float *__restrict__ gluts,
-                                                             int B, int I, int N, int K, int O) {
-    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
-    const long long NO = (long long)N * O;
-    if (gid >= (long long)B * NO) return;
-    const int b = (int)(gid / NO);
-    const long long c = gid % NO;
-    const int n = (int)(c / O);
-    const unsigned a = dwn_addr_generic(x + (size_t)b * I, idx32 + (size_t)n * K, K);
-    atomicAdd(&gluts[(c << K) + a], gy[gid]);
-}
-
-// Eval: address = floor(sum_j x_j 2^j), no thresholding of x; table value binarised at 0.5.
-__global__ __launch_bounds__(256) void dwn_eval_fwd(const float *__restrict__ x, const int *__restrict__ idx32,
-                                                     const float *__restrict__ luts, float *__restrict__ y,
-                                                     int B, int I, int N, int K, int O) {
-    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
-    const long long NO = (long long)N * O;
-    if (gid >= (long long)B * NO) return;
-    const int b = (int)(gid / NO);
-    const long long c = gid % NO;
-    const int n = (int)(c / O);
-    const float *xrow = x + (size_t)b * I;
-    const int *ix = idx32 + (size_t)n * K;
-    float s = 0.0f;
-    for (int j = 0; j < K; ++j) s += xrow[ix[j]] * (float)(1 << j);
-    long long a = (long long)s;  // truncation, as tensor.long()
-    a = a < 0 ? 0 : (a > (1 << K) - 1 ? (1 << K) - 1 : a);
-    y[gid] = luts[(c << K) + a] >= 0.5f ? 1.0f : 0.0f;
 }
 
 // ---------------------------------------------------------------------------------
@@ -336,26 +402,34 @@ static int dwn_check(int B, int I, int N, int k, int O) {
     if ((long long)N * O * ((long long)1 << k) > 0x7fffffffLL) return DL_ERR_UNSUPPORTED;
     return DL_OK;
 }
+// the fast kernels pack a node number into 23 bits of an entry record
+static inline bool dwn_fast(int N, int k) { return k <= DL_MAX_FAST_K && N < (1 << 23); }
 
 extern "C" size_t dl_dwn_saved_bytes(int B, int I, int N, int k, int O) {
     (void)I; (void)O;
-    if (k > DL_MAX_FAST_K) return 256;  // nothing is kept; a token allocation keeps callers simple
+    if (!dwn_fast(N, k)) return 256;  // nothing is kept; a token allocation keeps callers simple
     return dl_align256((size_t)N * dwn_bt(B) * 64);
 }
 extern "C" size_t dl_dwn_fwd_workspace_bytes(int B, int I, int N, int k, int O) {
-    (void)N; (void)O;
-    return k > DL_MAX_FAST_K ? 256 : dwn_planes_bytes(B, I);
+    (void)O;
+    return dwn_fast(N, k) ? dwn_planes_bytes(B, I) : 256;
 }
 extern "C" size_t dl_dwn_bwd_workspace_bytes(int B, int I, int N, int k, int O) {
     (void)I;
-    return k > DL_MAX_FAST_K ? 256 : dwn_table_bytes(N, k, O) + dwn_gyT_bytes(B, N, O);
+    return dwn_fast(N, k) ? dwn_table_bytes(N, k, O) + dwn_gyT_bytes(B, N, O) : 256;
 }
 
 template <int K>
 static void dwn_launch_lookup(const u64 *planes, const int *idx32, const float *luts, float *y, uint8_t *addrT,
                               int B, int I, int N, int O, hipStream_t s) {
-    dim3 grid(dl_ceil_div((long long)N * O, DWN_TC), dwn_bt(B));
-    DL_TIMED("dwn_lookup_fwd", s, (dwn_lookup_fwd<K><<<grid, 256, 0, s>>>(planes, idx32, luts, y, addrT, B, I, N, O, dwn_bt(B) * 64)));
+    const int BT = dwn_bt(B);
+    const int grid = dl_xcd_grid(dl_ceil_div((long long)N * O, DWN_TC), BT);
+    if (O == 1)
+        DL_TIMED("dwn_lookup_fwd", s,
+                 (dwn_lookup_fwd<K, true><<<grid, 256, 0, s>>>(planes, idx32, luts, y, addrT, B, I, N, O, BT)));
+    else
+        DL_TIMED("dwn_lookup_fwd", s,
+                 (dwn_lookup_fwd<K, false><<<grid, 256, 0, s>>>(planes, idx32, luts, y, addrT, B, I, N, O, BT)));
 }
 
 extern "C" int dl_dwn_layer_fwd(const float *x, const int32_t *idx32, const float *luts, float *y, void *saved,
@@ -364,10 +438,7 @@ extern "C" int dl_dwn_layer_fwd(const float *x, const int32_t *idx32, const floa
     int rc = dwn_check(B, I, N, k, O);
     if (rc) return rc;
     hipStream_t s = (hipStream_t)stream;
-    if (k > DL_MAX_FAST_K) {
-        dwn_generic_fwd<<<dl_ceil_div((long long)B * N * O, 256), 256, 0, s>>>(x, idx32, luts, y, B, I, N, k, O);
-        return dl_launch_status();
-    }
+    if (!dwn_fast(N, k)) return dwn_generic_forward(x, idx32, luts, y, B, I, N, k, O, s);
     if (!saved || !ws) return DL_ERR_NULL;
     if (ws_bytes < dl_dwn_fwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
     u64 *planes = (u64 *)ws;
@@ -390,9 +461,13 @@ extern "C" int dl_dwn_layer_fwd(const float *x, const int32_t *idx32, const floa
 
 template <int K>
 static void dwn_launch_gx(const float *gyT, const uint8_t *addrT, const float *D, const int *inv_ptr, const int *inv_pos,
-                          float *gx, int B, int I, int O, hipStream_t s) {
-    dim3 grid(dl_ceil_div(I, DWN_IS), dwn_bt(B));
-    DL_TIMED("dwn_bwd_gx", s, (dwn_bwd_gx<K><<<grid, 256, 0, s>>>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, O, dwn_bt(B) * 64)));
+                          float *gx, int B, int I, int N, int O, hipStream_t s) {
+    const int BT = dwn_bt(B);
+    const int grid = dl_xcd_grid(dl_ceil_div(I, DWN_IS), BT);
+    if (O == 1)
+        DL_TIMED("dwn_bwd_gx", s, (dwn_bwd_gx<K, true><<<grid, 256, 0, s>>>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, BT)));
+    else
+        DL_TIMED("dwn_bwd_gx", s, (dwn_bwd_gx<K, false><<<grid, 256, 0, s>>>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, BT)));
 }
 
 extern "C" int dl_dwn_layer_bwd(const float *x, const void *saved, const int32_t *idx32, const int32_t *inv_ptr,
@@ -406,14 +481,9 @@ extern "C" int dl_dwn_layer_bwd(const float *x, const void *saved, const int32_t
     hipStream_t s = (hipStream_t)stream;
     const long long NO = (long long)N * O;
     const int L = 1 << k;
-    dl_fill_zero(gluts, NO * L, s);
-    if (k > DL_MAX_FAST_K) {
+    if (!dwn_fast(N, k)) {
         if (!x) return DL_ERR_NULL;
-        dwn_generic_bwd_luts<<<dl_ceil_div((long long)B * NO, 256), 256, 0, s>>>(x, idx32, gy, gluts, B, I, N, k, O);
-        if (gx)
-            dwn_generic_bwd_gx<<<dl_ceil_div((long long)B * I, 256), 256, 0, s>>>(x, idx32, inv_ptr, inv_pos, luts, gy,
-                                                                                alpha, beta, gx, B, I, N, k, O);
-        return dl_launch_status();
+        return dwn_generic_backward(x, idx32, inv_ptr, inv_pos, luts, gy, alpha, beta, gx, gluts, B, I, N, k, O, s);
     }
     if (!saved || !ws) return DL_ERR_NULL;
     if (ws_bytes < dl_dwn_bwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
@@ -423,35 +493,28 @@ extern "C" int dl_dwn_layer_bwd(const float *x, const void *saved, const int32_t
     const int BT = dwn_bt(B), BP = BT * 64;
     // enough blocks to fill 256 CUs several times over, few enough that the per-block
     // histogram flush (one atomic per bin) stays small next to the streaming work
-    const int col_tiles = dl_ceil_div(NO, DWN_TC);
+    const int col_tiles = dl_ceil_div(NO, DWN_HC);
     int chunks = dl_ceil_div(1024, col_tiles);
     if (chunks > BT) chunks = BT;
     const int tpc = dl_ceil_div(BT, chunks);
     chunks = dl_ceil_div(BT, tpc);
     if (gx) {
-        DL_TIMED("dwn_efd_table", s, (dwn_efd_table<<<dl_ceil_div(NO * k * (L / 2), 256), 256, 0, s>>>(luts, D, (int)NO, k, alpha, beta)));
+        DL_TIMED("dwn_efd_table", s,
+                 (dwn_efd_table<<<dl_ceil_div(NO, 4), 256, 0, s>>>(luts, D, gluts, (int)NO, k, alpha, beta)));
         DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<true><<<dim3(col_tiles, chunks), 256, 0, s>>>(
                                                   gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc)));
         switch (k) {
-            case 1: dwn_launch_gx<1>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, O, s); break;
-            case 2: dwn_launch_gx<2>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, O, s); break;
-            case 3: dwn_launch_gx<3>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, O, s); break;
-            case 4: dwn_launch_gx<4>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, O, s); break;
-            case 5: dwn_launch_gx<5>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, O, s); break;
-            default: dwn_launch_gx<6>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, O, s); break;
+            case 1: dwn_launch_gx<1>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, s); break;
+            case 2: dwn_launch_gx<2>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, s); break;
+            case 3: dwn_launch_gx<3>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, s); break;
+            case 4: dwn_launch_gx<4>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, s); break;
+            case 5: dwn_launch_gx<5>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, s); break;
+            default: dwn_launch_gx<6>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, s); break;
         }
     } else {
+        dl_fill_zero(gluts, NO * L, s);
         DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<false><<<dim3(col_tiles, chunks), 256, 0, s>>>(
                                                   gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc)));
     }
-    return dl_launch_status();
-}
-
-extern "C" int dl_dwn_layer_eval(const float *x, const int32_t *idx32, const float *luts, float *y, int B, int I, int N,
-                                 int k, int O, void *stream) {
-    if (!x || !idx32 || !luts || !y) return DL_ERR_NULL;
-    int rc = dwn_check(B, I, N, k, O);
-    if (rc) return rc;
-    dwn_eval_fwd<<<dl_ceil_div((long long)B * N * O, 256), 256, 0, (hipStream_t)stream>>>(x, idx32, luts, y, B, I, N, k, O);
     return dl_launch_status();
 }
