@@ -89,18 +89,25 @@ __global__ __launch_bounds__(256) void dwn_pack_planes(const float *__restrict__
 }
 
 // ---------------------------------------------------------------------------------
-// lookup_fwd: grid (ceil(N*O / 128), B/64), 256 threads = 4 wavefronts, lane = batch row.
-// A wavefront walks 32 consecutive columns (column = node*O + output) in groups of 4 so that the
-// two dependent scalar loads per input (index, then bit-plane word) of a whole group are in flight
-// together.  Per column: k add-with-carry steps build the address, one bpermute reads the table.
+// lookup_fwd: one block per (128-column tile, 64-row batch tile), 512 threads = 8 wavefronts,
+// lane = batch row, column = node*O + output.  A wavefront owns 16 consecutive columns.  Their
+// k*16 input indices are fetched once (one per lane) and handed out with readlane; the bit-plane
+// words and table rows of the next group of 4 columns are requested (plain vector loads with a
+// wave-uniform address, so the in-order vector-memory counter allows partial waits) while the
+// current group is evaluated: per input one 64-bit shift picks the lane's bit, one bpermute per
+// column reads the table.
 #define DWN_TC 128
-#define DWN_CG 4
+#define DWN_FW 8                      // wavefronts per block
+#define DWN_WC (DWN_TC / DWN_FW)      // columns per wavefront
+#define DWN_CG 4                      // columns per group
 template <int K, bool O1>
-__global__ __launch_bounds__(256) void dwn_lookup_fwd(const u64 *__restrict__ planes, const int *__restrict__ idx32,
-                                                       const float *__restrict__ luts, float *__restrict__ y,
-                                                       uint8_t *__restrict__ addrT, int B, int I, int N, int O, int BT) {
+__global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restrict__ planes, const int *__restrict__ idx32,
+                                                               const float *__restrict__ luts, float *__restrict__ y,
+                                                               uint8_t *__restrict__ addrT, int B, int I, int N, int O,
+                                                               int BT) {
     __shared__ float tile[DWN_TC][65];  // [column][row]
     constexpr int L = 1 << K;
+    constexpr int NIDX = (DWN_WC * K + 63) / 64;  // index registers per lane
     const int NO = N * O;
     int ctile, t;
     if (!dl_xcd_map((NO + DWN_TC - 1) / DWN_TC, BT, ctile, t)) return;
@@ -109,52 +116,85 @@ __global__ __launch_bounds__(256) void dwn_lookup_fwd(const u64 *__restrict__ pl
     const int wave = dl_uniform(threadIdx.x >> 6);
     const u64 *pl = planes + (size_t)t * I;
     const int cend = min(DWN_TC, NO - c0);
-    const int wbeg = wave * (DWN_TC / 4);
-    for (int g = 0; g < DWN_TC / 4; g += DWN_CG) {
-        if (wbeg + g >= cend) break;
-        int node[DWN_CG], src[DWN_CG][K];
+    const int wbeg = wave * DWN_WC;
+    // slot s = (column within my 16) * K + j  ->  lane s % 64 of register s / 64
+    int myidx[NIDX];
+#pragma unroll
+    for (int v = 0; v < NIDX; ++v) {
+        const int s = v * 64 + lane;
+        const int c = min(c0 + wbeg + min(s / K, DWN_WC - 1), NO - 1);
+        myidx[v] = idx32[(O1 ? c : c / O) * K + s % K];
+    }
+    struct Group {
         u64 w[DWN_CG][K];
         float entry[DWN_CG];
+    };
+    auto request = [&](int g, Group &G) {
 #pragma unroll
         for (int q = 0; q < DWN_CG; ++q) {
-            const int c = min(c0 + wbeg + g + q, NO - 1);  // clamp: loads of a ragged last group stay in range
-            node[q] = O1 ? c : c / O;
+            const int c = min(c0 + wbeg + g + q, NO - 1);
+            G.entry[q] = luts[(size_t)c * L + (lane & (L - 1))];
 #pragma unroll
-            for (int j = 0; j < K; ++j) src[q][j] = idx32[node[q] * K + j];
-            entry[q] = luts[(size_t)c * L + (lane & (L - 1))];
+            for (int j = 0; j < K; ++j) {
+                const int s = (g + q) * K + j;  // wave-uniform
+                int src = 0;
+#pragma unroll
+                for (int v = 0; v < NIDX; ++v)
+                    if (s / 64 == v) src = __builtin_amdgcn_readlane(myidx[v], s % 64);
+                G.w[q][j] = pl[src];
+            }
         }
-#pragma unroll
-        for (int q = 0; q < DWN_CG; ++q)
-#pragma unroll
-            for (int j = 0; j < K; ++j) w[q][j] = pl[src[q][j]];
+    };
+    auto evaluate = [&](int g, const Group &G) {
 #pragma unroll
         for (int q = 0; q < DWN_CG; ++q) {
             const int cc = wbeg + g + q;
             unsigned addr = 0;
 #pragma unroll
-            for (int j = K - 1; j >= 0; --j) addr = dwn_shift_in(addr, w[q][j]);
-            const float v = dl_lane_read(entry[q], (int)addr);
+            for (int j = K - 1; j >= 0; --j) addr = (addr << 1) | ((unsigned)(G.w[q][j] >> lane) & 1u);
+            const float v = dl_lane_read(G.entry[q], (int)addr);
             if (cc < cend) {
                 tile[cc][lane] = v;
-                if (O1 || (c0 + cc) - node[q] * O == 0) addrT[((size_t)t * N + node[q]) * 64 + lane] = (uint8_t)addr;
+                const int c = c0 + cc;
+                const int n = O1 ? c : c / O;
+                if (O1 || c - n * O == 0) addrT[((size_t)t * N + n) * 64 + lane] = (uint8_t)addr;
             }
+        }
+    };
+    Group A, Bq;
+    if (wbeg < cend) {
+        request(0, A);
+#pragma unroll
+        for (int g = 0; g < DWN_WC; g += 2 * DWN_CG) {
+            if (g + DWN_CG < DWN_WC) request(g + DWN_CG, Bq);
+            evaluate(g, A);
+            if (g + 2 * DWN_CG < DWN_WC) request(g + 2 * DWN_CG, A);
+            if (g + DWN_CG < DWN_WC) evaluate(g + DWN_CG, Bq);
         }
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < 64 * DWN_TC; e += 256) {
+    for (int e = threadIdx.x; e < 64 * DWN_TC; e += 64 * DWN_FW) {
         const int r = e / DWN_TC, cc = e % DWN_TC;
         const int b = t * 64 + r;
-        if (b < B && cc < cend) y[(size_t)b * NO + c0 + cc] = tile[cc][r];
+        if (b < B && cc < cend) __builtin_nontemporal_store(tile[cc][r], &y[(size_t)b * NO + c0 + cc]);
     }
 }
 
 // ---------------------------------------------------------------------------------
-// efd_table: one wavefront per table (column), lane = table entry.  For every input j the table is
-// smoothed along all other inputs (v <- v + beta * v[entry ^ bit]) and differenced along j; lanes
-// whose bit j is clear hold the coefficient.  Double precision, one rounding to float.  The same
-// wavefront clears the table's gradient row.
+// efd_table: one wavefront per table (column), lane = table entry; also clears the table's
+// gradient row.  Two forms of the EFD coefficients, both in double with one rounding to float:
+//   D form: for every input j the table is smoothed along all OTHER inputs
+//           (v <- v + beta * v[entry ^ bit]) and differenced along j; lanes whose bit j is clear
+//           hold D[c][j][a'] = alpha * (v[a | bit j] - v[a & ~bit j]).          192 floats/table
+//   S form: the table smoothed along ALL inputs, scaled by alpha / (1 - beta).    64 floats/table
+//           Smoothing along j maps (u0,u1) -> (u0 + beta u1, beta u0 + u1), so the difference of
+//           the fully smoothed table across bit j is (1 - beta) times the D-form value:
+//           D[c][j][a'] = S[c][a | bit j] - S[c][a & ~bit j].  Cheaper to build, a third of the
+//           memory, shared by the k slots of a node - but it amplifies rounding by
+//           (1+|beta|)^k / (1-beta), so it is only used for |beta| <= 1/2 (the default is 1/3).
 __global__ __launch_bounds__(256) void dwn_efd_table(const float *__restrict__ luts, float *__restrict__ D,
-                                                      float *__restrict__ gluts, int NO, int K, float alpha, float beta) {
+                                                      float *__restrict__ gluts, int NO, int K, float alpha, float beta,
+                                                      int sform) {
     const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int a = threadIdx.x & 63;
     if (c >= NO) return;
@@ -162,6 +202,12 @@ __global__ __launch_bounds__(256) void dwn_efd_table(const float *__restrict__ l
     const bool live = a < L;
     const double v0 = live ? (double)luts[(size_t)c * L + a] : 0.0;
     if (live) gluts[(size_t)c * L + a] = 0.0f;
+    if (sform) {
+        double v = v0;
+        for (int m = 0; m < K; ++m) v += (double)beta * __shfl_xor(v, 1 << m);
+        if (live) D[(size_t)c * L + a] = (float)((double)alpha / (1.0 - (double)beta) * v);
+        return;
+    }
     for (int j = 0; j < K; ++j) {
         double v = v0;
         for (int m = 0; m < K; ++m) {
@@ -186,8 +232,11 @@ __global__ __launch_bounds__(256) void dwn_efd_table(const float *__restrict__ l
 //     step are merged with quad permutes first and no two lanes of the block ever update the same
 //     word at once (float atomics in LDS are far slower than this).
 #define DWN_HC 64
-__device__ __forceinline__ float dwn_quad_read(float v, int src) {  // value of lane (quad base + src)
-    return __int_as_float(__builtin_amdgcn_ds_bpermute(((threadIdx.x & ~3) | src) << 2, __float_as_int(v)));
+// value held by lane (lane ^ X) of the same quad, X = 1..3: a DPP quad permute, no LDS traffic
+template <int X>
+__device__ __forceinline__ int dwn_quad_xor(int v) {
+    constexpr int ctrl = X == 1 ? 0xB1 : (X == 2 ? 0x4E : 0x1B);  // quad_perm [1,0,3,2] / [2,3,0,1] / [3,2,1,0]
+    return __builtin_amdgcn_update_dpp(0, v, ctrl, 0xf, 0xf, true);
 }
 template <bool WRITE_T>
 __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__restrict__ gy, const uint8_t *__restrict__ addrT,
@@ -259,16 +308,14 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
                 const unsigned a = atile[hc][r0 + hr];
                 float sum = v;
                 bool leader = true;
-#pragma unroll
-                for (int o = 1; o < 4; ++o) {  // the other three lanes of my quad
-                    const int other = hr ^ o;
-                    const unsigned ao = (unsigned)__float_as_int(dwn_quad_read(__int_as_float((int)a), other));
-                    const float vo = dwn_quad_read(v, other);
-                    if (ao == a) {
-                        sum += vo;
-                        if (other < hr) leader = false;
-                    }
-                }
+                const unsigned a1 = (unsigned)dwn_quad_xor<1>((int)a), a2 = (unsigned)dwn_quad_xor<2>((int)a),
+                               a3 = (unsigned)dwn_quad_xor<3>((int)a);
+                const float v1 = __int_as_float(dwn_quad_xor<1>(__float_as_int(v))),
+                            v2 = __int_as_float(dwn_quad_xor<2>(__float_as_int(v))),
+                            v3 = __int_as_float(dwn_quad_xor<3>(__float_as_int(v)));
+                if (a1 == a) { sum += v1; leader = leader && (hr ^ 1) > hr; }
+                if (a2 == a) { sum += v2; leader = leader && (hr ^ 2) > hr; }
+                if (a3 == a) { sum += v3; leader = leader && (hr ^ 3) > hr; }
                 if (leader) hist[hc][a] += sum;
             }
         }
@@ -278,14 +325,16 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
 }
 
 // ---------------------------------------------------------------------------------
-// bwd_gx: grid (ceil(I / 128), B/64), lane = batch row.  A wavefront owns 32 consecutive inputs, i.e.
-// one contiguous run of CSR entries.  The run is read 64 entries at a time into registers (one
-// entry per lane: node, slot, local input), then replayed 8 entries per step with wave-uniform
-// addressing so that the 8 x 3 vector loads of a step are in flight together.  The entries of one input are
-// consecutive, so its sum is kept in a register and written to the LDS tile once (fixed order).
-#define DWN_IS 128
+// bwd_gx: one block per (64-input slab, 64-row batch tile), 256 threads, lane = batch row.  A wavefront
+// owns 16 consecutive inputs, i.e. one contiguous run of CSR entries.  The run is read 64 entries
+// at a time into registers (one entry per lane: node, slot, local input), then replayed 8 entries
+// per step with wave-uniform addressing; the 8 x 3 vector loads of the next step are requested
+// before the current step is evaluated.  The entries of one input are consecutive, so its sum is
+// kept in a register and written to the LDS tile once, in CSR order (reproducible sums).
+#define DWN_IS 64
+#define DWN_WI (DWN_IS / 4)  // inputs per wavefront
 #define DWN_EG 8
-template <int K, bool O1>
+template <int K, bool O1, bool SFORM>
 __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT, const uint8_t *__restrict__ addrT,
                                                    const float *__restrict__ D, const int *__restrict__ inv_ptr,
                                                    const int *__restrict__ inv_pos, float *__restrict__ gx,
@@ -301,17 +350,20 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT,
     const int iend = min(DWN_IS, I - i0);
     const uint8_t *addr_t = addrT + (size_t)t * N * 64 + lane;
     const float *gy_t = gyT + (size_t)t * NO * 64 + lane;
-    const int wbeg = wave * 32;
+    const int wbeg = wave * DWN_WI;
+    // CSR pointers of my inputs: lane l (0..DWN_WI) holds inv_ptr[first + l], clamped at I
+    const int myptr = inv_ptr[min(i0 + wbeg + min(lane, DWN_WI), I)];
 #pragma unroll
-    for (int r = 0; r < 32; ++r) tile[wbeg + r][lane] = 0.0f;
-    if (lane == 0)
-#pragma unroll
-        for (int r = 0; r < 32; ++r) tile[wbeg + r][64] = 0.0f;
-    // CSR pointers of my 32 inputs: lane l (0..32) holds inv_ptr[first + l], clamped at I
-    const int myptr = inv_ptr[min(i0 + wbeg + min(lane, 32), I)];
+    for (int r = 0; r < DWN_WI; ++r) tile[wbeg + r][lane] = 0.0f;  // inputs nobody reads keep 0
     const int ebeg = __builtin_amdgcn_readlane(myptr, 0);
-    const int eend = __builtin_amdgcn_readlane(myptr, 32);
-    float acc = 0.0f;  // running sum of the input `cur` (entries of one input are consecutive)
+    const int eend = __builtin_amdgcn_readlane(myptr, DWN_WI);
+    struct Group {
+        int rj[DWN_EG], ri[DWN_EG];
+        bool live[DWN_EG];
+        unsigned a[DWN_EG];
+        float g[DWN_EG], coef[DWN_EG];
+    };
+    float acc = 0.0f;  // running sum of the input `cur`
     int cur = -1;
     for (int base = ebeg; base < eend; base += 64) {
         const int e = base + lane;
@@ -319,61 +371,74 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT,
         const int p = valid ? inv_pos[e] : 0;
         int ii = 0;  // local input of entry e = number of my inputs that end at or before e
 #pragma unroll
-        for (int l = 1; l <= 32; ++l) ii += (__builtin_amdgcn_readlane(myptr, l) <= e) ? 1 : 0;
+        for (int l = 1; l <= DWN_WI; ++l) ii += (__builtin_amdgcn_readlane(myptr, l) <= e) ? 1 : 0;
         const int n = p / K, j = p - n * K;
         const int rec = valid ? ((n << 8) | (j << 5) | ii) : -1;
         const int cnt = min(64, eend - base);
-        for (int s0 = 0; s0 < cnt; s0 += DWN_EG) {
-            int rn[DWN_EG], rj[DWN_EG], ri[DWN_EG];
-            bool live[DWN_EG];
-            unsigned a[DWN_EG];
+        auto request = [&](int s0, Group &G) {
 #pragma unroll
             for (int q = 0; q < DWN_EG; ++q) {
-                const int r = __builtin_amdgcn_readlane(rec, s0 + q);
-                live[q] = r >= 0;
-                const int rr = r >= 0 ? r : 0;
-                rn[q] = rr >> 8; rj[q] = (rr >> 5) & 7; ri[q] = rr & 31;
-                a[q] = addr_t[(size_t)rn[q] * 64];
+                const int r = __builtin_amdgcn_readlane(rec, min(s0 + q, 63));
+                G.live[q] = r >= 0 && s0 + q < 64;
+                const int rr = G.live[q] ? r : 0;
+                const int rn = rr >> 8;
+                G.rj[q] = (rr >> 5) & 7;
+                G.ri[q] = rr & 31;
+                G.a[q] = addr_t[(size_t)rn * 64];
+                if (O1) {
+                    G.g[q] = gy_t[(size_t)rn * 64];
+                    if (SFORM)
+                        G.coef[q] = D[(size_t)rn * (2 * Lh) + (lane & (2 * Lh - 1))];
+                    else
+                        G.coef[q] = __builtin_nontemporal_load(&D[((size_t)rn * K + G.rj[q]) * Lh + (lane & (Lh - 1))]);
+                } else {
+                    G.g[q] = __int_as_float(rn);  // node number; outputs are walked in evaluate()
+                }
             }
-            if (O1) {
-                float g[DWN_EG], coef[DWN_EG];
+        };
+        auto evaluate = [&](const Group &G) {
 #pragma unroll
-                for (int q = 0; q < DWN_EG; ++q) {
-                    g[q] = gy_t[(size_t)rn[q] * 64];
-                    coef[q] = __builtin_nontemporal_load(&D[((size_t)rn[q] * K + rj[q]) * Lh + (lane & (Lh - 1))]);
-                }
-#pragma unroll
-                for (int q = 0; q < DWN_EG; ++q) {
-                    const unsigned ap = (a[q] & ((1u << rj[q]) - 1u)) | ((a[q] >> (rj[q] + 1)) << rj[q]);
-                    if (live[q]) {  // wave-uniform
-                        if (ri[q] != cur) {
-                            if (cur >= 0) tile[wbeg + cur][lane] = acc;
-                            acc = 0.0f;
-                            cur = ri[q];
-                        }
-                        acc += g[q] * dl_lane_read(coef[q], (int)ap);
-                    }
-                }
-            } else {
-#pragma unroll
-                for (int q = 0; q < DWN_EG; ++q) {
-                    const unsigned ap = (a[q] & ((1u << rj[q]) - 1u)) | ((a[q] >> (rj[q] + 1)) << rj[q]);
-                    float term = 0.0f;
+            for (int q = 0; q < DWN_EG; ++q) {
+                if (!G.live[q]) continue;  // wave-uniform
+                const int j_ = G.rj[q];
+                const unsigned ap = (G.a[q] & ((1u << j_) - 1u)) | ((G.a[q] >> (j_ + 1)) << j_);
+                float term;
+                if (O1 && SFORM) {
+                    const float hi = dl_lane_read(G.coef[q], (int)(G.a[q] | (1u << j_)));
+                    const float lo = dl_lane_read(G.coef[q], (int)(G.a[q] & ~(1u << j_)));
+                    term = G.g[q] * (hi - lo);
+                } else if (O1) {
+                    term = G.g[q] * dl_lane_read(G.coef[q], (int)ap);
+                } else {
+                    const int rn = __float_as_int(G.g[q]);
+                    term = 0.0f;
                     for (int d = 0; d < O; ++d) {
-                        const size_t c = (size_t)rn[q] * O + d;
-                        const float coef = D[(c * K + rj[q]) * Lh + (lane & (Lh - 1))];
-                        term += gy_t[c * 64] * dl_lane_read(coef, (int)ap);
-                    }
-                    if (live[q]) {
-                        if (ri[q] != cur) {
-                            if (cur >= 0) tile[wbeg + cur][lane] = acc;
-                            acc = 0.0f;
-                            cur = ri[q];
+                        const size_t c = (size_t)rn * O + d;
+                        if (SFORM) {
+                            const float coef = D[c * (2 * Lh) + (lane & (2 * Lh - 1))];
+                            term += gy_t[c * 64] * (dl_lane_read(coef, (int)(G.a[q] | (1u << j_))) -
+                                                    dl_lane_read(coef, (int)(G.a[q] & ~(1u << j_))));
+                        } else {
+                            const float coef = D[(c * K + j_) * Lh + (lane & (Lh - 1))];
+                            term += gy_t[c * 64] * dl_lane_read(coef, (int)ap);
                         }
-                        acc += term;
                     }
                 }
+                if (G.ri[q] != cur) {
+                    if (cur >= 0) tile[wbeg + cur][lane] = acc;
+                    acc = 0.0f;
+                    cur = G.ri[q];
+                }
+                acc += term;
             }
+        };
+        Group A, Bq;
+        request(0, A);
+        for (int s0 = 0; s0 < cnt; s0 += 2 * DWN_EG) {
+            if (s0 + DWN_EG < cnt) request(s0 + DWN_EG, Bq);
+            evaluate(A);
+            if (s0 + 2 * DWN_EG < cnt) request(s0 + 2 * DWN_EG, A);
+            if (s0 + DWN_EG < cnt) evaluate(Bq);
         }
     }
     if (cur >= 0) tile[wbeg + cur][lane] = acc;
@@ -381,7 +446,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT,
     for (int e = threadIdx.x; e < 64 * DWN_IS; e += 256) {
         const int r = e / DWN_IS, ii = e % DWN_IS;
         const int b = t * 64 + r;
-        if (b < B && ii < iend) gx[(size_t)b * I + i0 + ii] = tile[ii][r];
+        if (b < B && ii < iend) __builtin_nontemporal_store(tile[ii][r], &gx[(size_t)b * I + i0 + ii]);
     }
 }
 
@@ -426,10 +491,10 @@ static void dwn_launch_lookup(const u64 *planes, const int *idx32, const float *
     const int grid = dl_xcd_grid(dl_ceil_div((long long)N * O, DWN_TC), BT);
     if (O == 1)
         DL_TIMED("dwn_lookup_fwd", s,
-                 (dwn_lookup_fwd<K, true><<<grid, 256, 0, s>>>(planes, idx32, luts, y, addrT, B, I, N, O, BT)));
+                 (dwn_lookup_fwd<K, true><<<grid, 64 * DWN_FW, 0, s>>>(planes, idx32, luts, y, addrT, B, I, N, O, BT)));
     else
         DL_TIMED("dwn_lookup_fwd", s,
-                 (dwn_lookup_fwd<K, false><<<grid, 256, 0, s>>>(planes, idx32, luts, y, addrT, B, I, N, O, BT)));
+                 (dwn_lookup_fwd<K, false><<<grid, 64 * DWN_FW, 0, s>>>(planes, idx32, luts, y, addrT, B, I, N, O, BT)));
 }
 
 extern "C" int dl_dwn_layer_fwd(const float *x, const int32_t *idx32, const float *luts, float *y, void *saved,
@@ -461,13 +526,16 @@ extern "C" int dl_dwn_layer_fwd(const float *x, const int32_t *idx32, const floa
 
 template <int K>
 static void dwn_launch_gx(const float *gyT, const uint8_t *addrT, const float *D, const int *inv_ptr, const int *inv_pos,
-                          float *gx, int B, int I, int N, int O, hipStream_t s) {
+                          float *gx, int B, int I, int N, int O, bool sform, hipStream_t s) {
     const int BT = dwn_bt(B);
     const int grid = dl_xcd_grid(dl_ceil_div(I, DWN_IS), BT);
-    if (O == 1)
-        DL_TIMED("dwn_bwd_gx", s, (dwn_bwd_gx<K, true><<<grid, 256, 0, s>>>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, BT)));
-    else
-        DL_TIMED("dwn_bwd_gx", s, (dwn_bwd_gx<K, false><<<grid, 256, 0, s>>>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, BT)));
+#define DWN_GX(O1_, S_) \
+    DL_TIMED("dwn_bwd_gx", s, (dwn_bwd_gx<K, O1_, S_><<<grid, 256, 0, s>>>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, BT)))
+    if (O == 1 && sform) DWN_GX(true, true);
+    else if (O == 1) DWN_GX(true, false);
+    else if (sform) DWN_GX(false, true);
+    else DWN_GX(false, false);
+#undef DWN_GX
 }
 
 extern "C" int dl_dwn_layer_bwd(const float *x, const void *saved, const int32_t *idx32, const int32_t *inv_ptr,
@@ -499,17 +567,18 @@ extern "C" int dl_dwn_layer_bwd(const float *x, const void *saved, const int32_t
     const int tpc = dl_ceil_div(BT, chunks);
     chunks = dl_ceil_div(BT, tpc);
     if (gx) {
+        const bool sform = beta >= -0.5f && beta <= 0.5f;
         DL_TIMED("dwn_efd_table", s,
-                 (dwn_efd_table<<<dl_ceil_div(NO, 4), 256, 0, s>>>(luts, D, gluts, (int)NO, k, alpha, beta)));
+                 (dwn_efd_table<<<dl_ceil_div(NO, 4), 256, 0, s>>>(luts, D, gluts, (int)NO, k, alpha, beta, sform ? 1 : 0)));
         DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<true><<<dim3(col_tiles, chunks), 256, 0, s>>>(
                                                   gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc)));
         switch (k) {
-            case 1: dwn_launch_gx<1>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, s); break;
-            case 2: dwn_launch_gx<2>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, s); break;
-            case 3: dwn_launch_gx<3>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, s); break;
-            case 4: dwn_launch_gx<4>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, s); break;
-            case 5: dwn_launch_gx<5>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, s); break;
-            default: dwn_launch_gx<6>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, s); break;
+            case 1: dwn_launch_gx<1>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, s); break;
+            case 2: dwn_launch_gx<2>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, s); break;
+            case 3: dwn_launch_gx<3>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, s); break;
+            case 4: dwn_launch_gx<4>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, s); break;
+            case 5: dwn_launch_gx<5>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, s); break;
+            default: dwn_launch_gx<6>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, s); break;
         }
     } else {
         dl_fill_zero(gluts, NO * L, s);
