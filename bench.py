@@ -30,8 +30,11 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 WORKLOADS = {
     # name: (B, I, N, k, O)
-    "dwn_k6_b4096_i16384_n8192": (4096, 16384, 8192, 6, 1),
+    "dwn_k6_b4096_i16384_n8192": (4096, 16384, 8192, 6, 1),   # the configuration the metric is quoted on
     "dwn_small": (256, 3136, 2000, 6, 1),
+    # secondary workloads of the same path, reported with their own metric names (see run_secondary)
+    "prob_k4_b1024_i4096_n4096": (1024, 4096, 4096, 4, 1),
+    "softmap_b512_i3136_m48000": (512, 3136, 8000, 6, 1),
 }
 
 
@@ -53,6 +56,96 @@ def algorithmic_bytes(B, I, N, k, O):
     return fwd, bwd, per_kernel
 
 
+def time_steps(step, steps, warmup):
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def kernel_times(step, reps):
+    from difflut_amd import _native as nat
+    nat.profile_enable(True)
+    per = {}
+    for _ in range(reps):
+        step()
+        for name, ms in nat.profile_read():
+            per.setdefault(name, []).append(ms)
+    nat.profile_enable(False)
+    return {name: float(np.mean(v)) for name, v in per.items()}
+
+
+def run_secondary(args):
+    """Probabilistic layer (BASELINE configs[1]) and soft connectivity (configs[3]) through the C ABI."""
+    from difflut_amd import _native as nat
+    from difflut_amd import ops
+    from oracle import difflut_oracle as orc
+
+    lib = nat.lib()
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    B, I, N, k, O = WORKLOADS[args.workload]
+    torch.manual_seed(0)
+    if args.workload.startswith("prob"):
+        dims = (B, I, N, k, O)
+        x = torch.sigmoid(torch.randn(B, I, device=dev))
+        plan = ops.MappingPlan(orc.random_mapping(I, N, k, seed=42).to(dev), I)
+        raw = torch.rand(N, 1 << k, O, device=dev)
+        gy = torch.randn(B, N * O, device=dev)
+        y = torch.empty(B, N * O, device=dev); gx = torch.empty(B, I, device=dev); graw = torch.empty_like(raw)
+        ws = torch.empty(max(lib.dl_prob_bwd_workspace_bytes(*dims), 256), dtype=torch.uint8, device=dev)
+
+        def step():
+            nat.check(lib.dl_prob_layer_fwd(x.data_ptr(), plan.idx32.data_ptr(), raw.data_ptr(), 1.0, y.data_ptr(), *dims,
+                                            stream))
+            nat.check(lib.dl_prob_layer_bwd(x.data_ptr(), plan.idx32.data_ptr(), plan.inv_ptr.data_ptr(),
+                                            plan.inv_pos.data_ptr(), raw.data_ptr(), 1.0, gy.data_ptr(), gx.data_ptr(),
+                                            graw.data_ptr(), ws.data_ptr(), ws.numel(), *dims, stream))
+
+        ms = time_steps(step, args.steps, args.warmup)
+        nbytes = 5 * B * I * 4 + 3 * N * (1 << k) * O * 4 + 2 * N * k * 2  # x, y, gy, x again, gx; tables r, r, grad
+        flops = 320 * B * N
+        out = {"metric": "LUT-node evals/sec fwd+bwd (Probabilistic k=4, B=1024, 4096 nodes)", "value": B * N / (ms * 1e-3),
+               "unit": "node-evals/s", "ms_per_step": ms, "dtype": "f32",
+               "roofline_step": {"bound": "hbm", "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
+                                 "unit": "GB/s", "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                 "algorithmic_bytes_per_step": nbytes},
+               "valu": {"achieved_tflops": flops / (ms * 1e-3) / 1e12, "peak_tflops": 157.3}}
+    else:
+        M = N * k
+        precision = args.precision
+        x = torch.rand(B, I, device=dev)
+        W = torch.randn(M, I, device=dev) * 0.01
+        gm = torch.randn(B, M, device=dev)
+        m = torch.empty(B, M, device=dev); stats = torch.empty(2 * M, device=dev)
+        gx = torch.empty_like(x); gW = torch.empty_like(W)
+        ws = torch.empty(max(lib.dl_soft_map_workspace_bytes(B, I, M, precision), 256), dtype=torch.uint8, device=dev)
+
+        def step():
+            nat.check(lib.dl_soft_map_fwd(x.data_ptr(), W.data_ptr(), 1.0, m.data_ptr(), stats.data_ptr(), ws.data_ptr(),
+                                          ws.numel(), B, I, M, precision, stream))
+            nat.check(lib.dl_soft_map_bwd(x.data_ptr(), W.data_ptr(), 1.0, m.data_ptr(), stats.data_ptr(), gm.data_ptr(),
+                                          gx.data_ptr(), gW.data_ptr(), ws.data_ptr(), ws.numel(), B, I, M, precision,
+                                          stream))
+
+        ms = time_steps(step, args.steps, args.warmup)
+        flops = 3 * 2.0 * B * I * M
+        peak = 157.3 if precision == 0 else 2500.0
+        out = {"metric": "soft-connectivity contraction fwd+bwd (x[512,3136] . softmax(W[48000,3136])^T)",
+               "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": ms,
+               "dtype": "f32" if precision == 0 else "bf16",
+               "roofline_step": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
+                                 "frac": flops / (ms * 1e-3) / 1e12 / peak, "algorithmic_flops_per_step": flops}}
+    out.update({"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+                "vs_baseline": None, "data": "synthetic", "config": {"workload": args.workload},
+                "kernel_ms": kernel_times(step, min(args.steps, 10))})
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -60,7 +153,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="dwn_k6_b4096_i16384_n8192", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-rows", type=int, default=512, help="batch rows of the workload the CPU baseline runs")
+    ap.add_argument("--cpu-rows", type=int, default=4096, help="batch rows of the workload the CPU baseline runs")
+    ap.add_argument("--precision", type=int, default=0, help="soft-connectivity workload: 0 fp32, 1 bf16 operands")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no collective); run with --gpus 1",
@@ -74,6 +168,8 @@ def main():
     lib = nat.lib()  # raises if the HIP library has not been built
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a ROCm device")
+    if not args.workload.startswith("dwn"):
+        return run_secondary(args)
     dev = torch.device("cuda:0")
     B, I, N, k, O = WORKLOADS[args.workload]
     dims = (B, I, N, k, O)

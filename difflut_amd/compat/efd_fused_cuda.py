@@ -1,0 +1,43 @@
+"""efd_fused_cuda.forward/backward (difflut/nodes/cuda/efd_fused_cuda.cpp:19-34): whole layer,
+int64 mapping [N,k], luts [N,O,L]; returns [B,N,O] and [grad_input, grad_luts]."""
+from _common import check_cuda_contiguous, nat, ops, plan_for, torch
+
+
+def _dims(input, mapping, luts):
+    B, I = input.shape
+    N, k = mapping.shape
+    return B, I, N, k, luts.shape[1]
+
+
+def forward(input, mapping, luts):
+    check_cuda_contiguous(input, mapping, luts)
+    plan = plan_for(mapping, input.shape[1])
+    dims = _dims(input, mapping, luts)
+    lib = nat.lib()
+    B, _, N, _, O = dims
+    y = torch.empty((B, N, O), dtype=torch.float32, device=input.device)
+    saved = torch.empty(lib.dl_dwn_saved_bytes(*dims), dtype=torch.uint8, device=input.device)
+    ws = torch.empty(lib.dl_dwn_fwd_workspace_bytes(*dims), dtype=torch.uint8, device=input.device)
+    nat.check(lib.dl_dwn_layer_fwd(input.data_ptr(), plan.idx32.data_ptr(), luts.data_ptr(), y.data_ptr(),
+                                   saved.data_ptr(), ws.data_ptr(), ws.numel(), *dims, nat.stream()))
+    plan.last_saved = (input.data_ptr(), saved)  # reused by backward when it is called on the same input
+    return y
+
+
+def backward(input, mapping, luts, grad_output, alpha, beta):
+    check_cuda_contiguous(input, mapping, luts, grad_output)
+    plan = plan_for(mapping, input.shape[1])
+    dims = _dims(input, mapping, luts)
+    lib = nat.lib()
+    cached = getattr(plan, "last_saved", None)
+    if cached is None or cached[0] != input.data_ptr():
+        forward(input, mapping, luts)  # the legacy signature hands over x, not the saved addresses
+        cached = plan.last_saved
+    gx = torch.empty_like(input)
+    gl = torch.empty_like(luts)
+    ws = torch.empty(lib.dl_dwn_bwd_workspace_bytes(*dims), dtype=torch.uint8, device=input.device)
+    nat.check(lib.dl_dwn_layer_bwd(input.data_ptr(), cached[1].data_ptr(), plan.idx32.data_ptr(),
+                                   plan.inv_ptr.data_ptr(), plan.inv_pos.data_ptr(), luts.data_ptr(),
+                                   grad_output.data_ptr(), float(alpha), float(beta), gx.data_ptr(), gl.data_ptr(),
+                                   ws.data_ptr(), ws.numel(), *dims, nat.stream()))
+    return [gx, gl]

@@ -92,10 +92,10 @@ __global__ __launch_bounds__(256) void dwn_pack_planes(const float *__restrict__
 // lookup_fwd: one block per (128-column tile, 64-row batch tile), 512 threads = 8 wavefronts,
 // lane = batch row, column = node*O + output.  A wavefront owns 16 consecutive columns.  Their
 // k*16 input indices are fetched once (one per lane) and handed out with readlane; the bit-plane
-// words and table rows of the next group of 4 columns are requested (plain vector loads with a
-// wave-uniform address, so the in-order vector-memory counter allows partial waits) while the
-// current group is evaluated: per input one 64-bit shift picks the lane's bit, one bpermute per
-// column reads the table.
+// word of (tile, input) is wave-uniform, so it comes through a scalar load and is used directly
+// as a lane mask: one add-with-carry per input shifts the lane's bit into its address
+// (addr <- 2*addr + bit), one bpermute per column reads the table entry.  Columns are taken four
+// at a time so that the 4*k scalar loads of a group are in flight together.
 #define DWN_TC 128
 #define DWN_FW 8                      // wavefronts per block
 #define DWN_WC (DWN_TC / DWN_FW)      // columns per wavefront
@@ -125,51 +125,38 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
         const int c = min(c0 + wbeg + min(s / K, DWN_WC - 1), NO - 1);
         myidx[v] = idx32[(O1 ? c : c / O) * K + s % K];
     }
-    struct Group {
-        u64 w[DWN_CG][K];
-        float entry[DWN_CG];
-    };
-    auto request = [&](int g, Group &G) {
-#pragma unroll
-        for (int q = 0; q < DWN_CG; ++q) {
-            const int c = min(c0 + wbeg + g + q, NO - 1);
-            G.entry[q] = luts[(size_t)c * L + (lane & (L - 1))];
-#pragma unroll
-            for (int j = 0; j < K; ++j) {
-                const int s = (g + q) * K + j;  // wave-uniform
-                int src = 0;
-#pragma unroll
-                for (int v = 0; v < NIDX; ++v)
-                    if (s / 64 == v) src = __builtin_amdgcn_readlane(myidx[v], s % 64);
-                G.w[q][j] = pl[src];
-            }
-        }
-    };
-    auto evaluate = [&](int g, const Group &G) {
-#pragma unroll
-        for (int q = 0; q < DWN_CG; ++q) {
-            const int cc = wbeg + g + q;
-            unsigned addr = 0;
-#pragma unroll
-            for (int j = K - 1; j >= 0; --j) addr = (addr << 1) | ((unsigned)(G.w[q][j] >> lane) & 1u);
-            const float v = dl_lane_read(G.entry[q], (int)addr);
-            if (cc < cend) {
-                tile[cc][lane] = v;
-                const int c = c0 + cc;
-                const int n = O1 ? c : c / O;
-                if (O1 || c - n * O == 0) addrT[((size_t)t * N + n) * 64 + lane] = (uint8_t)addr;
-            }
-        }
-    };
-    Group A, Bq;
     if (wbeg < cend) {
-        request(0, A);
 #pragma unroll
-        for (int g = 0; g < DWN_WC; g += 2 * DWN_CG) {
-            if (g + DWN_CG < DWN_WC) request(g + DWN_CG, Bq);
-            evaluate(g, A);
-            if (g + 2 * DWN_CG < DWN_WC) request(g + 2 * DWN_CG, A);
-            if (g + DWN_CG < DWN_WC) evaluate(g + DWN_CG, Bq);
+        for (int g = 0; g < DWN_WC; g += DWN_CG) {
+            u64 w[DWN_CG][K];
+            float entry[DWN_CG];
+#pragma unroll
+            for (int q = 0; q < DWN_CG; ++q) {
+                const int c = min(c0 + wbeg + g + q, NO - 1);
+                entry[q] = luts[(size_t)c * L + (lane & (L - 1))];
+#pragma unroll
+                for (int j = 0; j < K; ++j) {
+                    constexpr int dummy = 0;
+                    (void)dummy;
+                    const int s = (g + q) * K + j;  // compile-time after unrolling
+                    const int src = __builtin_amdgcn_readlane(myidx[s / 64], s % 64);
+                    w[q][j] = pl[src];  // wave-uniform address: scalar load
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < DWN_CG; ++q) {
+                const int cc = wbeg + g + q;
+                unsigned addr = 0;
+#pragma unroll
+                for (int j = K - 1; j >= 0; --j) addr = dwn_shift_in(addr, w[q][j]);
+                const float v = dl_lane_read(entry[q], (int)addr);
+                if (cc < cend) {
+                    tile[cc][lane] = v;
+                    const int c = c0 + cc;
+                    const int n = O1 ? c : c / O;
+                    if (O1 || c - n * O == 0) addrT[((size_t)t * N + n) * 64 + lane] = (uint8_t)addr;
+                }
+            }
         }
     }
     __syncthreads();

@@ -270,12 +270,13 @@ extern "C" int dl_prob_layer_fwd(const float *x, const int32_t *idx32, const flo
     hipStream_t s = (hipStream_t)stream;
     const float inv_t = prob_inv_t(temperature);
     if (!prob_fast(I, k)) {
-        prob_generic_fwd<<<dl_ceil_div((long long)B * N * O, 256), 256, 0, s>>>(x, idx32, raw_w, inv_t, y, B, I, N, k, O);
+        DL_TIMED("prob_generic_fwd", s, (prob_generic_fwd<<<dl_ceil_div((long long)B * N * O, 256), 256, 0, s>>>(x, idx32, raw_w, inv_t, y, B, I, N, k, O)));
         return dl_launch_status();
     }
     dim3 grid(dl_ceil_div(N, PROB_NODES), dl_ceil_div(B, PROB_ROWS));
     const size_t lds = (size_t)I * sizeof(float);
-#define CALL(KK) prob_fwd_kernel<KK><<<grid, PROB_NODES, lds, s>>>(x, idx32, raw_w, inv_t, y, B, I, N, O, PROB_ROWS)
+#define CALL(KK) \
+    DL_TIMED("prob_fwd_kernel", s, (prob_fwd_kernel<KK><<<grid, PROB_NODES, lds, s>>>(x, idx32, raw_w, inv_t, y, B, I, N, O, PROB_ROWS)))
     PROB_DISPATCH(k, CALL)
 #undef CALL
     return dl_launch_status();
@@ -292,10 +293,10 @@ extern "C" int dl_prob_layer_bwd(const float *x, const int32_t *idx32, const int
     const float inv_t = prob_inv_t(temperature);
     const long long WT = (long long)N * ((long long)1 << k) * O;
     if (!prob_fast(I, k)) {
-        prob_fill_zero<<<dl_ceil_div(WT, 256), 256, 0, s>>>(graw, WT);
+        DL_TIMED("prob_fill_zero", s, (prob_fill_zero<<<dl_ceil_div(WT, 256), 256, 0, s>>>(graw, WT)));
         if (gx) prob_fill_zero<<<dl_ceil_div((long long)B * I, 256), 256, 0, s>>>(gx, (long long)B * I);
-        prob_generic_bwd<<<dl_ceil_div((long long)B * N, 256), 256, 0, s>>>(x, idx32, raw_w, inv_t, gy, gx, graw, B, I, N,
-                                                                          k, O);
+        DL_TIMED("prob_generic_bwd", s, (prob_generic_bwd<<<dl_ceil_div((long long)B * N, 256), 256, 0, s>>>(x, idx32, raw_w, inv_t, gy, gx, graw, B, I, N,
+                                                                          k, O)));
         return dl_launch_status();
     }
     if (!ws) return DL_ERR_NULL;
@@ -306,12 +307,17 @@ extern "C" int dl_prob_layer_bwd(const float *x, const int32_t *idx32, const int
     float *gpart = (float *)((char *)ws + dl_align256((size_t)B * N * k * sizeof(float)));
     dim3 grid(dl_ceil_div(N, PROB_NODES), chunks);
     const size_t lds = (size_t)I * sizeof(float);
-#define CALL(KK) \
-    prob_bwd_kernel<KK><<<grid, PROB_NODES, lds, s>>>(x, idx32, raw_w, inv_t, gy, gm, gpart, B, I, N, O, rows, gx != nullptr)
+#define CALL(KK)                                                                                                     \
+    DL_TIMED("prob_bwd_kernel", s,                                                                                   \
+             (prob_bwd_kernel<KK><<<grid, PROB_NODES, lds, s>>>(x, idx32, raw_w, inv_t, gy, gm, gpart, B, I, N, O, rows, \
+                                                                gx != nullptr)))
     PROB_DISPATCH(k, CALL)
 #undef CALL
-    prob_reduce_weights<<<dl_ceil_div(WT, 256), 256, 0, s>>>(gpart, raw_w, inv_t, graw, WT, chunks);
-    if (gx) prob_gather_bwd<<<dim3(dl_ceil_div(I, 256), B), 256, 0, s>>>(gm, inv_ptr, inv_pos, gx, I, (long long)N * k);
+    DL_TIMED("prob_reduce_weights", s,
+             (prob_reduce_weights<<<dl_ceil_div(WT, 256), 256, 0, s>>>(gpart, raw_w, inv_t, graw, WT, chunks)));
+    if (gx)
+        DL_TIMED("prob_gather_bwd", s,
+                 (prob_gather_bwd<<<dim3(dl_ceil_div(I, 256), B), 256, 0, s>>>(gm, inv_ptr, inv_pos, gx, I, (long long)N * k)));
     return dl_launch_status();
 }
 
@@ -320,7 +326,7 @@ extern "C" int dl_prob_layer_eval(const float *x, const int32_t *idx32, const fl
     if (!x || !idx32 || !raw_w || !y) return DL_ERR_NULL;
     int rc = prob_check(B, I, N, k, O);
     if (rc) return rc;
-    prob_eval_kernel<<<dl_ceil_div((long long)B * N * O, 256), 256, 0, (hipStream_t)stream>>>(
-        x, idx32, raw_w, prob_inv_t(temperature), y, B, I, N, k, O);
+    DL_TIMED("prob_eval_kernel", (hipStream_t)stream, (prob_eval_kernel<<<dl_ceil_div((long long)B * N * O, 256), 256, 0, (hipStream_t)stream>>>(
+        x, idx32, raw_w, prob_inv_t(temperature), y, B, I, N, k, O)));
     return dl_launch_status();
 }

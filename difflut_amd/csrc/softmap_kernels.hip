@@ -172,9 +172,9 @@ extern "C" int dl_soft_map_fwd(const float *x, const float *W, float tau, float 
     if (!(tau > 0.0f)) return DL_ERR_SHAPE;
     hipStream_t s = (hipStream_t)stream;
     const float inv_tau = 1.0f / tau;
-    softmap_rowstats<<<dl_ceil_div(M, 4), 256, 0, s>>>(W, inv_tau, stats, M, I);
-    softmap_gemm<0><<<dim3(dl_ceil_div(M, SM_T), dl_ceil_div(B, SM_T)), 256, 0, s>>>(x, W, stats, nullptr, nullptr, inv_tau,
-                                                                                   m, B, I, M);
+    DL_TIMED("softmap_rowstats", s, (softmap_rowstats<<<dl_ceil_div(M, 4), 256, 0, s>>>(W, inv_tau, stats, M, I)));
+    DL_TIMED("softmap_gemm_fwd", s, (softmap_gemm<0><<<dim3(dl_ceil_div(M, SM_T), dl_ceil_div(B, SM_T)), 256, 0, s>>>(x, W, stats, nullptr, nullptr, inv_tau,
+                                                                                   m, B, I, M)));
     return dl_launch_status();
 }
 
@@ -189,10 +189,10 @@ extern "C" int dl_soft_map_bwd(const float *x, const float *W, float tau, const 
     hipStream_t s = (hipStream_t)stream;
     const float inv_tau = 1.0f / tau;
     float *r = (float *)ws;
-    softmap_rowdot<<<dl_ceil_div(M, 256), 256, 0, s>>>(gm, m, r, B, M);
-    softmap_gemm<1><<<dim3(dl_ceil_div(I, SM_T), dl_ceil_div(B, SM_T)), 256, 0, s>>>(x, W, stats, gm, nullptr, inv_tau, gx,
-                                                                                   B, I, M);
-    softmap_gemm<2><<<dim3(dl_ceil_div(I, SM_T), dl_ceil_div(M, SM_T)), 256, 0, s>>>(x, W, stats, gm, r, inv_tau, gW, B, I,
-                                                                                   M);
+    DL_TIMED("softmap_rowdot", s, (softmap_rowdot<<<dl_ceil_div(M, 256), 256, 0, s>>>(gm, m, r, B, M)));
+    DL_TIMED("softmap_gemm_gx", s, (softmap_gemm<1><<<dim3(dl_ceil_div(I, SM_T), dl_ceil_div(B, SM_T)), 256, 0, s>>>(x, W, stats, gm, nullptr, inv_tau, gx,
+                                                                                   B, I, M)));
+    DL_TIMED("softmap_gemm_gw", s, (softmap_gemm<2><<<dim3(dl_ceil_div(I, SM_T), dl_ceil_div(M, SM_T)), 256, 0, s>>>(x, W, stats, gm, r, inv_tau, gW, B, I,
+                                                                                   M)));
     return dl_launch_status();
 }

@@ -245,3 +245,48 @@ def test_full_size_properties_dwn_k6_b4096_n8192():
     want = torch.zeros(N, 64, device="cuda", dtype=torch.float64)
     want.scatter_add_(1, addr.t().contiguous(), gy.t().double().contiguous())
     torch.testing.assert_close(gl1[:, 0, :].double(), want, rtol=1e-5, atol=1e-4)
+
+
+def test_legacy_extension_names_and_signatures(golden):
+    """tests/test_layers/test_fused_kernels.py:159-179 imports efd_cuda / efd_fused_cuda by bare name;
+    the shims answer with the reference's signatures."""
+    import difflut_amd.compat as compat
+    compat.install()
+    import efd_cuda
+    import efd_fused_cuda
+    import learnable_mapping_cuda
+    import mapping_cuda
+    import probabilistic_cuda
+
+    g = golden
+    dev = "cuda"
+    x = torch.tensor(g["dwn_k6o2_x"], device=dev); luts = torch.tensor(g["dwn_k6o2_luts"], device=dev)
+    gy = torch.tensor(g["dwn_k6o2_gy"], device=dev)
+    a, b = (float(v) for v in g["dwn_k6o2_ab"])
+    assert np.array_equal(efd_cuda.forward(x, luts).cpu().numpy(), g["dwn_k6o2_y"])
+    gx, gl = efd_cuda.backward(x, luts, gy, a, b)
+    np.testing.assert_allclose(gx.cpu().numpy(), g["dwn_k6o2_gx"], rtol=1e-5, atol=2e-6)
+    np.testing.assert_allclose(gl.cpu().numpy(), g["dwn_k6o2_gl"], rtol=1e-5, atol=1e-6)
+    rng = np.random.default_rng(0)
+    xin = torch.tensor(rng.random((50, 30)).astype(np.float32), device=dev)
+    mapping = orc.random_mapping(30, 12, 4, seed=3).to(dev).long()
+    l3 = torch.tensor(rng.uniform(-1, 1, (12, 2, 16)).astype(np.float32), device=dev)
+    y = efd_fused_cuda.forward(xin, mapping, l3)
+    assert y.shape == (50, 12, 2)
+    assert np.array_equal(y.cpu().numpy(), orc.dwn_layer_forward(xin.cpu().numpy(), mapping.cpu().numpy(), l3.cpu().numpy()))
+    m = mapping_cuda.forward(xin, mapping.to(torch.int16))
+    assert np.array_equal(m.cpu().numpy(), orc.gather_forward(xin.cpu().numpy(), mapping.cpu().numpy()))
+    gm = torch.randn_like(m)
+    np.testing.assert_allclose(mapping_cuda.backward(gm, mapping.to(torch.int16), 30).cpu().numpy(),
+                               orc.gather_backward(gm.cpu().numpy(), mapping.cpu().numpy(), 30), rtol=1e-6, atol=1e-6)
+    T = torch.tensor(float(g["prob_k4o2_T"][0]), device=dev)
+    px = torch.tensor(g["prob_k4o2_x"], device=dev); pw = torch.tensor(g["prob_k4o2_w"], device=dev)
+    np.testing.assert_allclose(probabilistic_cuda.forward(px, pw, T).cpu().numpy(), g["prob_k4o2_y"], rtol=1e-5, atol=1e-6)
+    pgx, pgw = probabilistic_cuda.backward(px, pw, T, torch.tensor(g["prob_k4o2_gy"], device=dev))
+    np.testing.assert_allclose(pgx.cpu().numpy(), g["prob_k4o2_gx"], rtol=1e-5, atol=2e-6)
+    np.testing.assert_allclose(pgw.cpu().numpy(), g["prob_k4o2_gw"], rtol=1e-5, atol=2e-6)
+    sx = torch.tensor(g["soft_x"], device=dev); sW = torch.tensor(g["soft_W"], device=dev)
+    np.testing.assert_allclose(learnable_mapping_cuda.soft_forward(sx, sW, 1.0).cpu().numpy(), g["soft_m"].reshape(5, -1),
+                               rtol=1e-5, atol=1e-6)
+    sel = torch.tensor(g["hard_idx"].reshape(-1), device=dev, dtype=torch.int32)
+    assert np.array_equal(learnable_mapping_cuda.forward(sx, sel).cpu().numpy(), g["hard_m"].reshape(5, -1))
