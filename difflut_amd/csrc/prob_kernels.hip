@@ -19,13 +19,46 @@ __device__ __forceinline__ float dl_sigmoid(float v) { return 1.0f / (1.0f + exp
 #define PROB_NODES 256  // nodes (= threads) per block
 #define PROB_ROWS 16    // batch rows per block in the forward
 
+
+// Row staging shared by the forward and backward kernels: the block's next row of x is fetched
+// into registers (up to PROB_PRE float4 per thread, i.e. rows of up to 4096 floats) while the
+// current one is being used from LDS, so only one barrier pair per row sits on the critical path.
+// Wider or unaligned rows are staged directly.
+#define PROB_PRE 4
+struct ProbRowStage {
+    float4 pre[PROB_PRE];
+    bool vec;
+    __device__ void init(const float *x, int I) { vec = (I % 4 == 0) && I <= 4 * PROB_NODES * PROB_PRE && (((size_t)x & 15) == 0); }
+    __device__ void fetch(const float *x, int I, int b) {
+        if (!vec) return;
+        const float4 *row = reinterpret_cast<const float4 *>(x + (size_t)b * I);
+#pragma unroll
+        for (int u = 0; u < PROB_PRE; ++u) {
+            const int q = u * PROB_NODES + threadIdx.x;
+            if (q * 4 < I) pre[u] = row[q];
+        }
+    }
+    // call between two __syncthreads(): the first guards the previous row's readers
+    __device__ void commit(float *xrow, const float *x, int I, int b) {
+        if (vec) {
+#pragma unroll
+            for (int u = 0; u < PROB_PRE; ++u) {
+                const int q = u * PROB_NODES + threadIdx.x;
+                if (q * 4 < I) reinterpret_cast<float4 *>(xrow)[q] = pre[u];
+            }
+        } else {
+            for (int i = threadIdx.x; i < I; i += PROB_NODES) xrow[i] = x[(size_t)b * I + i];
+        }
+    }
+};
+
 // ---------------------------------------------------------------------------------
 template <int K>
 __global__ __launch_bounds__(PROB_NODES) void prob_fwd_kernel(const float *__restrict__ x, const int *__restrict__ idx32,
                                                                const float *__restrict__ raw, float inv_t,
                                                                float *__restrict__ y, int B, int I, int N, int O,
                                                                int rows_per_block) {
-    extern __shared__ float xrow[];  // I floats
+    extern __shared__ __align__(16) float xrow[];  // I floats
     constexpr int L = 1 << K;
     const int n = blockIdx.x * PROB_NODES + threadIdx.x;
     const bool live = n < N;
@@ -38,10 +71,14 @@ __global__ __launch_bounds__(PROB_NODES) void prob_fwd_kernel(const float *__res
         float tab[L];
 #pragma unroll
         for (int a = 0; a < L; ++a) tab[a] = live ? dl_sigmoid(raw[((size_t)n * L + a) * O + d] * inv_t) : 0.0f;
+        ProbRowStage stage;
+        stage.init(x, I);
+        if (b0 < b1) stage.fetch(x, I, b0);
         for (int b = b0; b < b1; ++b) {
             __syncthreads();
-            for (int i = threadIdx.x; i < I; i += PROB_NODES) xrow[i] = x[(size_t)b * I + i];
+            stage.commit(xrow, x, I, b);
             __syncthreads();
+            if (b + 1 < b1) stage.fetch(x, I, b + 1);
             float v[L];
 #pragma unroll
             for (int a = 0; a < L; ++a) v[a] = tab[a];
@@ -65,7 +102,7 @@ __global__ __launch_bounds__(PROB_NODES) void prob_bwd_kernel(const float *__res
                                                                const float *__restrict__ gy, float *__restrict__ gm,
                                                                float *__restrict__ gpart, int B, int I, int N, int O,
                                                                int rows_per_block, int want_gm) {
-    extern __shared__ float xrow[];
+    extern __shared__ __align__(16) float xrow[];
     constexpr int L = 1 << K;
     const int n = blockIdx.x * PROB_NODES + threadIdx.x;
     const bool live = n < N;
@@ -81,10 +118,14 @@ __global__ __launch_bounds__(PROB_NODES) void prob_bwd_kernel(const float *__res
             tab[a] = live ? dl_sigmoid(raw[((size_t)n * L + a) * O + d] * inv_t) : 0.0f;
             gt[a] = 0.0f;
         }
+        ProbRowStage stage;
+        stage.init(x, I);
+        if (b0 < b1) stage.fetch(x, I, b0);
         for (int b = b0; b < b1; ++b) {
             __syncthreads();
-            for (int i = threadIdx.x; i < I; i += PROB_NODES) xrow[i] = x[(size_t)b * I + i];
+            stage.commit(xrow, x, I, b);
             __syncthreads();
+            if (b + 1 < b1) stage.fetch(x, I, b + 1);
             float xs[K];
 #pragma unroll
             for (int j = 0; j < K; ++j) xs[j] = xrow[src[j]];
@@ -223,17 +264,23 @@ __global__ __launch_bounds__(256) void prob_fill_zero(float *p, long long n) {
     if (i < n) p[i] = 0.0f;
 }
 
-// gather of the mapping adjoint (same kernel shape as the RandomLayer gather backward)
+// gather of the mapping adjoint: one block per batch row; the row of gm [N*k] is staged in LDS when it
+// fits (coalesced read), then every input sums its CSR entries from LDS in fixed order.
 __global__ __launch_bounds__(256) void prob_gather_bwd(const float *__restrict__ gm, const int *__restrict__ inv_ptr,
                                                         const int *__restrict__ inv_pos, float *__restrict__ gx, int I,
-                                                        long long NK) {
-    const int b = blockIdx.y;
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= I) return;
+                                                        long long NK, int staged) {
+    extern __shared__ __align__(16) float grow[];
+    const int b = blockIdx.x;
     const float *row = gm + (size_t)b * NK;
-    float acc = 0.0f;
-    for (int e = inv_ptr[i]; e < inv_ptr[i + 1]; ++e) acc += row[inv_pos[e]];
-    gx[(size_t)b * I + i] = acc;
+    if (staged) {
+        for (long long p = threadIdx.x; p < NK; p += 256) grow[p] = row[p];
+        __syncthreads();
+    }
+    for (int i = threadIdx.x; i < I; i += 256) {
+        float acc = 0.0f;
+        for (int e = inv_ptr[i]; e < inv_ptr[i + 1]; ++e) acc += staged ? grow[inv_pos[e]] : row[inv_pos[e]];
+        gx[(size_t)b * I + i] = acc;
+    }
 }
 
 // ---------------------------------------------------------------------------------
@@ -315,9 +362,11 @@ extern "C" int dl_prob_layer_bwd(const float *x, const int32_t *idx32, const int
 #undef CALL
     DL_TIMED("prob_reduce_weights", s,
              (prob_reduce_weights<<<dl_ceil_div(WT, 256), 256, 0, s>>>(gpart, raw_w, inv_t, graw, WT, chunks)));
+    const int staged = (size_t)N * k * sizeof(float) <= 64 * 1024;
+    const size_t gbytes = staged ? (size_t)N * k * sizeof(float) : 0;
     if (gx)
         DL_TIMED("prob_gather_bwd", s,
-                 (prob_gather_bwd<<<dim3(dl_ceil_div(I, 256), B), 256, 0, s>>>(gm, inv_ptr, inv_pos, gx, I, (long long)N * k)));
+                 (prob_gather_bwd<<<B, 256, gbytes, s>>>(gm, inv_ptr, inv_pos, gx, I, (long long)N * k, staged)));
     return dl_launch_status();
 }
 

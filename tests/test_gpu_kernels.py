@@ -199,7 +199,8 @@ def test_prob_node_against_reference_vectors(golden, tag):
 
 # ------------------------------------------------------------------------------ learnable mapping
 @pytest.mark.parametrize("shape,tau", [((5, 20, 21), 1.0), ((70, 130, 200), 0.3), ((64, 64, 64), 1.0),
-                                       ((33, 257, 18), 0.05)])
+                                       ((33, 257, 18), 0.05), ((256, 384, 1000), 1.0),
+                                       ((130, 260, 516), 0.5), ((129, 132, 4100), 2.0)])
 def test_soft_mapping_forward_backward_fp32(shape, tau):
     ops = _ops()
     B, I, M = shape
