@@ -12,42 +12,103 @@
 //              matrix G never needs a second pass)
 //
 // One product kernel, three operand modes.  Block = 256 threads = 2x2 wavefronts, output tile
-// 128 x 128, each wavefront 64 x 64 = 2x2 MFMA tiles (4 x 16 accumulator registers), reduction
-// staged through LDS 32 deep as As[k][row], Bs[k][col] (k-major, so an MFMA operand read is 64
-// consecutive floats).  The next stage's global loads are issued before the current stage's
-// MFMAs.
+// 128 x 128, each wavefront 64 x 64 = 2x2 MFMA tiles (4 x 16 accumulator registers).  The
+// reduction is staged through LDS SM_K deep as As[k][row], Bs[k][col] (k-major, so an MFMA operand
+// read is 64 consecutive floats), two stages resident: while the MFMAs read one, the next is
+// written piecewise between MFMA groups and the one after that is on its way from memory.
+#include <type_traits>
+
 #include "dl_common.h"
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-#define SM_T 128   // output tile edge
-#define SM_K 32    // reduction depth per LDS stage
-#define SM_LD 132  // LDS row stride in floats (multiple of 4: float4 stores stay aligned)
+#define SM_T 128     // output tile edge
+#ifndef SM_K0
+#define SM_K0 16     // reduction depth per LDS stage: forward,
+#endif
+#ifndef SM_K1
+#define SM_K1 16     // input gradient,
+#endif
+#ifndef SM_K2
+#define SM_K2 16     // weight gradient
+#endif
+#ifndef SM_BAR_MASK
+#define SM_BAR_MASK 7
+#endif
+#define SM_LD_V 132  // LDS row stride (floats) of a stage written with float4 stores: multiple of 4
+#define SM_LD_T 133  // ... of a stage written transposed, one float at a time: odd, spreads the banks
+#define SM_LOG2E 1.4426950408889634f
 
-// one wavefront per row of W
-__global__ __launch_bounds__(256) void softmap_rowstats(const float *__restrict__ W, float inv_tau, float *__restrict__ stats,
+// exp((w - mx)/tau) / sum, with scale = log2(e)/tau: one subtract, one multiply, the hardware
+// exp2 and the normalisation.  Relative error about |w - mx|/tau * 6e-8 plus one ulp of exp2.
+// The row sums are built with the same function, so rows of S sum to one to rounding.
+__device__ __forceinline__ float softmap_e(float w, float mx, float scale) {
+    return __builtin_amdgcn_exp2f((w - mx) * scale);
+}
+__device__ __forceinline__ float softmap_s(float w, float mx, float rs, float scale) {
+    return softmap_e(w, mx, scale) * rs;
+}
+
+// one wavefront per row of W; the second sweep of the row comes from cache
+__global__ __launch_bounds__(256) void softmap_rowstats(const float *__restrict__ W, float scale, float *__restrict__ stats,
                                                          int M, int I) {
     const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     if (row >= M) return;
     const float *w = W + (size_t)row * I;
-    float mx = -INFINITY;
-    for (int i = lane; i < I; i += 64) mx = fmaxf(mx, w[i]);
-    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-    float sum = 0.0f;
-    for (int i = lane; i < I; i += 64) sum += expf((w[i] - mx) * inv_tau);
+    float mx = -INFINITY, sum = 0.0f;
+    if (I % 4 == 0) {
+        const float4 *w4 = reinterpret_cast<const float4 *>(w);
+        const int n4 = I >> 2;
+        float m0 = -INFINITY, m1 = -INFINITY;
+        int i = lane;
+        for (; i + 64 < n4; i += 128) {
+            const float4 a = w4[i], b = w4[i + 64];
+            m0 = fmaxf(m0, fmaxf(fmaxf(a.x, a.y), fmaxf(a.z, a.w)));
+            m1 = fmaxf(m1, fmaxf(fmaxf(b.x, b.y), fmaxf(b.z, b.w)));
+        }
+        if (i < n4) { const float4 a = w4[i]; m0 = fmaxf(m0, fmaxf(fmaxf(a.x, a.y), fmaxf(a.z, a.w))); }
+        mx = fmaxf(m0, m1);
+        for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+        for (i = lane; i < n4; i += 64) {
+            const float4 a = w4[i];
+            sum += (softmap_e(a.x, mx, scale) + softmap_e(a.y, mx, scale)) +
+                   (softmap_e(a.z, mx, scale) + softmap_e(a.w, mx, scale));
+        }
+    } else {
+        for (int i = lane; i < I; i += 64) mx = fmaxf(mx, w[i]);
+        for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+        for (int i = lane; i < I; i += 64) sum += softmap_e(w[i], mx, scale);
+    }
     for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
     if (lane == 0) { stats[2 * row] = mx; stats[2 * row + 1] = 1.0f / sum; }
 }
 
-// r[o] = sum_b gm[b,o] m[b,o]
+// r[o] = sum_b gm[b,o] m[b,o]; block = 32 columns x 8 row groups, partial sums joined in LDS in fixed order
 __global__ __launch_bounds__(256) void softmap_rowdot(const float *__restrict__ gm, const float *__restrict__ m,
                                                        float *__restrict__ r, int B, int M) {
-    const int o = blockIdx.x * 256 + threadIdx.x;
-    if (o >= M) return;
+    __shared__ float part[8][33];
+    const int c = threadIdx.x & 31, g = threadIdx.x >> 5;
+    const int o = blockIdx.x * 32 + c;
     float acc = 0.0f;
-    for (int b = 0; b < B; ++b) acc += gm[(size_t)b * M + o] * m[(size_t)b * M + o];
-    r[o] = acc;
+    if (o < M) {
+        int b = g;
+        for (; b + 24 < B; b += 32) {
+            const size_t e = (size_t)b * M + o;
+            const float g0 = gm[e], g1 = gm[e + 8 * (size_t)M], g2 = gm[e + 16 * (size_t)M], g3 = gm[e + 24 * (size_t)M];
+            const float m0 = m[e], m1 = m[e + 8 * (size_t)M], m2 = m[e + 16 * (size_t)M], m3 = m[e + 24 * (size_t)M];
+            acc += g0 * m0; acc += g1 * m1; acc += g2 * m2; acc += g3 * m3;
+        }
+        for (; b < B; b += 8) acc += gm[(size_t)b * M + o] * m[(size_t)b * M + o];
+    }
+    part[g][c] = acc;
+    __syncthreads();
+    if (g == 0 && o < M) {
+        float t = part[0][c];
+#pragma unroll
+        for (int q = 1; q < 8; ++q) t += part[q][c];
+        r[o] = t;
+    }
 }
 
 // out[e] = sum over chunks of part[chunk][e], fixed order
@@ -60,38 +121,54 @@ __global__ __launch_bounds__(256) void softmap_reduce_chunks(const float *__rest
     out[e] = acc;
 }
 
-__device__ __forceinline__ float softmap_s(float w, float mx, float rs, float inv_tau) {
-    return expf((w - mx) * inv_tau) * rs;
-}
+struct SoftmapArgs {
+    const float *x, *W, *stats, *gm, *r;
+    float scale, inv_tau;
+    float *out;
+    int B, I, M;
+    int inner_count, outer_count, col_tiles, red_chunk;
+};
 
 // MODE 0: forward   rows=b cols=o red=i   A = x[b,i]  (red contiguous)   B = S[o,i] (red contiguous)
 // MODE 1: gx        rows=b cols=i red=o   A = gm[b,o] (red contiguous)   B = S[o,i] (col contiguous)
 // MODE 2: gW        rows=o cols=i red=b   A = gm[b,o] (row contiguous)   B = x[b,i] (col contiguous)
 //                   epilogue S[o,i] (C - r[o]) / tau
-// blockIdx.z selects a chunk of the reduction (MODE 1); out then points at [chunks][R][C] partials.
-template <int MODE>
-__global__ __launch_bounds__(256) void softmap_mfma(const float *__restrict__ x, const float *__restrict__ W,
-                                                     const float *__restrict__ stats, const float *__restrict__ gm,
-                                                     const float *__restrict__ r, float inv_tau, float *__restrict__ out,
-                                                     int B, int I, int M, int red_chunk) {
-    __shared__ __align__(16) float As[SM_K][SM_LD];
-    __shared__ __align__(16) float Bs[SM_K][SM_LD];
+// EDGE false: the tile lies inside the matrices, the reduction range is a whole number of stages
+// and every float4 is aligned, so the loop body is straight-line code and the compiler can count
+// outstanding loads exactly.  EDGE true: every access is predicated (ragged shapes).
+template <int MODE, int KC, bool EDGE>
+__device__ __forceinline__ void softmap_tile(const SoftmapArgs &g, float *sm_lds, int rt, int ct, int zc) {
+    constexpr bool A_RED_CONTIG = MODE != 2;
+    constexpr bool B_RED_CONTIG = MODE == 0;
+    constexpr int LDA = A_RED_CONTIG ? SM_LD_T : SM_LD_V;
+    constexpr int LDB = B_RED_CONTIG ? SM_LD_T : SM_LD_V;
+    constexpr int P = KC / 8;  // float4 pieces per operand per thread per stage
+    float *const As = sm_lds;                  // [2][KC][LDA]
+    float *const Bs = sm_lds + 2 * KC * LDA;   // [2][KC][LDB]
+    const float *__restrict__ x = g.x, *__restrict__ W = g.W, *__restrict__ stats = g.stats, *__restrict__ gm = g.gm;
+    const int B = g.B, I = g.I, M = g.M;
+    const float scale = g.scale;
+
     const int R = MODE == 2 ? M : B;                      // rows of the output
     const int C = MODE == 0 ? M : I;                      // columns of the output
     const int KD = MODE == 0 ? I : (MODE == 1 ? M : B);   // reduction length
-    const int r0 = blockIdx.y * SM_T, c0 = blockIdx.x * SM_T;
-    const int k_begin = blockIdx.z * red_chunk;
-    const int k_end = min(KD, k_begin + red_chunk);
+    const int r0 = rt * SM_T, c0 = ct * SM_T;
+    const int k_begin = zc * g.red_chunk;
+    const int k_end = min(KD, k_begin + g.red_chunk);
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;  // wavefront's corner inside the tile
-    constexpr bool A_RED_CONTIG = MODE != 2;
-    constexpr bool B_RED_CONTIG = MODE == 0;
-    // staging registers: 4 float4 per operand per thread (128 x 32 floats / 256 threads)
-    float4 pa[4], pb[4];
-    float bmx[4], brs[4];  // row statistics that go with pb (B operand built from W)
+    float4 pa[P], pb[P];
+    float bmx[P], brs[P];  // row statistics that go with pb (B operand built from W)
 
-    auto in_a = [&](int row, int k) -> float {  // scalar fallback for ragged edges
+    // thread -> piece of the tile.  red-contiguous operand: float4 runs along k (KC/4 per row),
+    // 1024/KC rows per pass; row/col-contiguous operand: float4 runs along the row/col axis (32 per k), 8 k per pass
+    constexpr int QR = KC / 4, RP = 1024 / KC;
+    const int a_q = A_RED_CONTIG ? (tid % QR) : (tid & 31), a_o = A_RED_CONTIG ? (tid / QR) : (tid >> 5);
+    const int b_q = B_RED_CONTIG ? (tid % QR) : (tid & 31), b_o = B_RED_CONTIG ? (tid / QR) : (tid >> 5);
+    const int lda = MODE == 0 ? I : M;
+
+    auto in_a = [&](int row, int k) -> float {  // predicated scalar access
         if (row >= R || k >= k_end) return 0.0f;
         if (MODE == 0) return x[(size_t)row * I + k];
         if (MODE == 1) return gm[(size_t)row * M + k];
@@ -99,72 +176,70 @@ __global__ __launch_bounds__(256) void softmap_mfma(const float *__restrict__ x,
     };
     auto in_b = [&](int k, int col) -> float {
         if (col >= C || k >= k_end) return 0.0f;
-        if (MODE == 0) return softmap_s(W[(size_t)col * I + k], stats[2 * col], stats[2 * col + 1], inv_tau);
-        if (MODE == 1) return softmap_s(W[(size_t)k * I + col], stats[2 * k], stats[2 * k + 1], inv_tau);
+        if (MODE == 0) return softmap_s(W[(size_t)col * I + k], stats[2 * col], stats[2 * col + 1], scale);
+        if (MODE == 1) return softmap_s(W[(size_t)k * I + col], stats[2 * k], stats[2 * k + 1], scale);
         return x[(size_t)k * I + col];
     };
-    // thread -> piece of the tile.  red-contiguous operand: float4 runs along k (8 per 32-deep row),
-    // 32 rows per pass; row/col-contiguous operand: float4 runs along the row/col axis (32 per k), 8 k per pass
-    const int a_q = A_RED_CONTIG ? (tid & 7) : (tid & 31), a_o = A_RED_CONTIG ? (tid >> 3) : (tid >> 5);
-    const int b_q = B_RED_CONTIG ? (tid & 7) : (tid & 31), b_o = B_RED_CONTIG ? (tid >> 3) : (tid >> 5);
-    const int lda = MODE == 0 ? I : M;
-    const bool a_vec = (lda % 4 == 0), b_vec = (I % 4 == 0);
 
-    auto fetch = [&](int k0) {
+    if (!EDGE && MODE == 0) {  // the W rows a thread stages do not change from stage to stage
 #pragma unroll
-        for (int p = 0; p < 4; ++p) {
+        for (int p = 0; p < P; ++p) {
+            const int col = c0 + b_o + RP * p;
+            bmx[p] = stats[2 * col]; brs[p] = stats[2 * col + 1];
+        }
+    }
+    auto fetch = [&](int p, int k0) {
+        if (EDGE) {
             if (A_RED_CONTIG) {
-                const int row = r0 + a_o + 32 * p, k = k0 + a_q * 4;
-                const float *A = MODE == 0 ? x : gm;
-                if (a_vec && row < R && k + 3 < k_end) pa[p] = *reinterpret_cast<const float4 *>(A + (size_t)row * lda + k);
-                else pa[p] = make_float4(in_a(row, k), in_a(row, k + 1), in_a(row, k + 2), in_a(row, k + 3));
+                const int row = r0 + a_o + RP * p, k = k0 + a_q * 4;
+                pa[p] = make_float4(in_a(row, k), in_a(row, k + 1), in_a(row, k + 2), in_a(row, k + 3));
             } else {
                 const int k = k0 + a_o + 8 * p, row = r0 + a_q * 4;
-                if (a_vec && k < k_end && row + 3 < R) pa[p] = *reinterpret_cast<const float4 *>(gm + (size_t)k * M + row);
-                else pa[p] = make_float4(in_a(row, k), in_a(row + 1, k), in_a(row + 2, k), in_a(row + 3, k));
+                pa[p] = make_float4(in_a(row, k), in_a(row + 1, k), in_a(row + 2, k), in_a(row + 3, k));
             }
             if (B_RED_CONTIG) {
-                const int col = c0 + b_o + 32 * p, k = k0 + b_q * 4;
-                if (b_vec && col < C && k + 3 < k_end) {
-                    pb[p] = *reinterpret_cast<const float4 *>(W + (size_t)col * I + k);
-                    bmx[p] = stats[2 * col]; brs[p] = stats[2 * col + 1];
-                } else {
-                    pb[p] = make_float4(in_b(k, col), in_b(k + 1, col), in_b(k + 2, col), in_b(k + 3, col));
-                    bmx[p] = 0.0f; brs[p] = -1.0f;  // already transformed
-                }
+                const int col = c0 + b_o + RP * p, k = k0 + b_q * 4;
+                pb[p] = make_float4(in_b(k, col), in_b(k + 1, col), in_b(k + 2, col), in_b(k + 3, col));
             } else {
                 const int k = k0 + b_o + 8 * p, col = c0 + b_q * 4;
-                const float *Bsrc = MODE == 1 ? W : x;
-                if (b_vec && k < k_end && col + 3 < C) {
-                    pb[p] = *reinterpret_cast<const float4 *>(Bsrc + (size_t)k * I + col);
-                    if (MODE == 1) { bmx[p] = stats[2 * k]; brs[p] = stats[2 * k + 1]; }
-                } else {
-                    pb[p] = make_float4(in_b(k, col), in_b(k, col + 1), in_b(k, col + 2), in_b(k, col + 3));
-                    bmx[p] = 0.0f; brs[p] = -1.0f;
-                }
+                pb[p] = make_float4(in_b(k, col), in_b(k, col + 1), in_b(k, col + 2), in_b(k, col + 3));
+            }
+        } else {
+            if (A_RED_CONTIG) {
+                const int row = r0 + a_o + RP * p, k = k0 + a_q * 4;
+                pa[p] = *reinterpret_cast<const float4 *>((MODE == 0 ? x : gm) + (size_t)row * lda + k);
+            } else {
+                const int k = k0 + a_o + 8 * p, row = r0 + a_q * 4;
+                pa[p] = *reinterpret_cast<const float4 *>(gm + (size_t)k * M + row);
+            }
+            if (B_RED_CONTIG) {
+                const int col = c0 + b_o + RP * p, k = k0 + b_q * 4;
+                pb[p] = *reinterpret_cast<const float4 *>(W + (size_t)col * I + k);
+            } else {
+                const int k = k0 + b_o + 8 * p, col = c0 + b_q * 4;
+                pb[p] = *reinterpret_cast<const float4 *>((MODE == 1 ? W : x) + (size_t)k * I + col);
+                if (MODE == 1) { bmx[p] = stats[2 * k]; brs[p] = stats[2 * k + 1]; }
             }
         }
     };
-    auto commit = [&]() {
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            if (A_RED_CONTIG) {
-                const int rr = a_o + 32 * p, kk = a_q * 4;
-                As[kk][rr] = pa[p].x; As[kk + 1][rr] = pa[p].y; As[kk + 2][rr] = pa[p].z; As[kk + 3][rr] = pa[p].w;
-            } else {
-                *reinterpret_cast<float4 *>(&As[a_o + 8 * p][a_q * 4]) = pa[p];
-            }
-            float4 v = pb[p];
-            if (MODE != 2 && brs[p] >= 0.0f) {  // W values -> softmax entries
-                v.x = softmap_s(v.x, bmx[p], brs[p], inv_tau); v.y = softmap_s(v.y, bmx[p], brs[p], inv_tau);
-                v.z = softmap_s(v.z, bmx[p], brs[p], inv_tau); v.w = softmap_s(v.w, bmx[p], brs[p], inv_tau);
-            }
-            if (B_RED_CONTIG) {
-                const int cc = b_o + 32 * p, kk = b_q * 4;
-                Bs[kk][cc] = v.x; Bs[kk + 1][cc] = v.y; Bs[kk + 2][cc] = v.z; Bs[kk + 3][cc] = v.w;
-            } else {
-                *reinterpret_cast<float4 *>(&Bs[b_o + 8 * p][b_q * 4]) = v;
-            }
+    auto commit = [&](int p, int buf) {
+        float *Ab = As + buf * KC * LDA, *Bb = Bs + buf * KC * LDB;
+        if (A_RED_CONTIG) {
+            float *d = Ab + (a_q * 4) * LDA + a_o + RP * p;
+            d[0] = pa[p].x; d[LDA] = pa[p].y; d[2 * LDA] = pa[p].z; d[3 * LDA] = pa[p].w;
+        } else {
+            *reinterpret_cast<float4 *>(Ab + (a_o + 8 * p) * LDA + a_q * 4) = pa[p];
+        }
+        float4 v = pb[p];
+        if (!EDGE && MODE != 2) {  // W values -> softmax entries (the predicated path did it on load)
+            v.x = softmap_s(v.x, bmx[p], brs[p], scale); v.y = softmap_s(v.y, bmx[p], brs[p], scale);
+            v.z = softmap_s(v.z, bmx[p], brs[p], scale); v.w = softmap_s(v.w, bmx[p], brs[p], scale);
+        }
+        if (B_RED_CONTIG) {
+            float *d = Bb + (b_q * 4) * LDB + b_o + RP * p;
+            d[0] = v.x; d[LDB] = v.y; d[2 * LDB] = v.z; d[3 * LDB] = v.w;
+        } else {
+            *reinterpret_cast<float4 *>(Bb + (b_o + 8 * p) * LDB + b_q * 4) = v;
         }
     };
 
@@ -176,25 +251,60 @@ __global__ __launch_bounds__(256) void softmap_mfma(const float *__restrict__ x,
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    if (k_begin < k_end) fetch(k_begin);
-    for (int k0 = k_begin; k0 < k_end; k0 += SM_K) {
-        __syncthreads();  // previous stage fully consumed
-        commit();
-        __syncthreads();
-        if (k0 + SM_K < k_end) fetch(k0 + SM_K);
-        const int kh = lane >> 5, l32 = lane & 31;
+    const int nst = (k_end - k_begin + KC - 1) / KC;
+    if (nst > 0) {
 #pragma unroll
-        for (int k2 = 0; k2 < SM_K; k2 += 2) {
-            const float a0 = As[k2 + kh][wm + l32], a1 = As[k2 + kh][wm + 32 + l32];
-            const float b0 = Bs[k2 + kh][wn + l32], b1 = Bs[k2 + kh][wn + 32 + l32];
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+        for (int p = 0; p < P; ++p) fetch(p, k_begin);
+#pragma unroll
+        for (int p = 0; p < P; ++p) commit(p, 0);
+        if (nst > 1) {
+#pragma unroll
+            for (int p = 0; p < P; ++p) fetch(p, k_begin + KC);
         }
     }
+    __syncthreads();
+    const int kh = lane >> 5, l32 = lane & 31;
+    // one stage: MFMAs over buffer s&1; between MFMA groups, piece p of stage s+1 goes from
+    // registers to the other buffer and piece p of stage s+2 is requested from memory
+    auto stage = [&](int s, auto do_commit, auto do_fetch) {
+        const int cur = s & 1;
+        const float *Ab = As + cur * KC * LDA + kh * LDA + wm + l32;
+        const float *Bb = Bs + cur * KC * LDB + kh * LDB + wn + l32;
+        float a0 = Ab[0], a1 = Ab[32], b0 = Bb[0], b1 = Bb[32];
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+#pragma unroll
+            for (int k2 = p * 8; k2 < p * 8 + 8; k2 += 2) {
+                float na0 = 0.0f, na1 = 0.0f, nb0 = 0.0f, nb1 = 0.0f;
+                if (k2 + 2 < KC) {  // operands of the next step are on their way while this step's MFMAs issue
+                    na0 = Ab[(k2 + 2) * LDA]; na1 = Ab[(k2 + 2) * LDA + 32];
+                    nb0 = Bb[(k2 + 2) * LDB]; nb1 = Bb[(k2 + 2) * LDB + 32];
+                }
+                acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+                acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+                acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+                acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+                a0 = na0; a1 = na1; b0 = nb0; b1 = nb1;
+            }
+            // keep the scheduler from sinking the loads to the end of the stage (their data is
+            // needed one stage later, not sooner) or hoisting the staging work above the MFMAs
+            if (SM_BAR_MASK & (1 << MODE)) __builtin_amdgcn_sched_barrier(0);
+            if constexpr (decltype(do_commit)::value) commit(p, cur ^ 1);
+            if constexpr (decltype(do_fetch)::value) fetch(p, k_begin + (s + 2) * KC);
+            if (SM_BAR_MASK & (1 << MODE)) __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();
+    };
+    {
+        using T = std::true_type;
+        using F = std::false_type;
+        int s = 0;
+        for (; s + 2 < nst; ++s) stage(s, T{}, T{});
+        if (s + 1 < nst) { stage(s, T{}, F{}); ++s; }
+        if (s < nst) stage(s, F{}, F{});
+    }
     // accumulator layout of a 32x32 tile: register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4, column l%32
-    float *dst = out + (size_t)blockIdx.z * R * C;
+    float *dst = g.out + (size_t)zc * R * C;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -203,11 +313,11 @@ __global__ __launch_bounds__(256) void softmap_mfma(const float *__restrict__ x,
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int row = r0 + wm + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                if (row < R && col < C) {
+                if (!EDGE || (row < R && col < C)) {
                     float val = acc[i][j][v];
                     if (MODE == 2) {
-                        const float sv = softmap_s(W[(size_t)row * I + col], stats[2 * row], stats[2 * row + 1], inv_tau);
-                        val = sv * (val - r[row]) * inv_tau;
+                        const float sv = softmap_s(W[(size_t)row * I + col], stats[2 * row], stats[2 * row + 1], scale);
+                        val = sv * (val - g.r[row]) * g.inv_tau;
                     }
                     dst[(size_t)row * C + col] = val;
                 }
@@ -215,20 +325,275 @@ __global__ __launch_bounds__(256) void softmap_mfma(const float *__restrict__ x,
         }
 }
 
+// 1-D grid decoded so that blocks which share the large operand tile (W, or the gm column slab in
+// MODE 2) sit next to each other on one XCD and find it in that XCD's L2.  MODE 1 also carries a
+// chunk of the reduction in the block index; out then points at [chunks][R][C] partial products.
+template <int MODE, int KC>
+__global__ __launch_bounds__(256) void softmap_mfma(SoftmapArgs g) {
+    extern __shared__ __align__(16) float sm_lds[];
+    int inner, outer;
+    if (!dl_xcd_map(g.inner_count, g.outer_count, inner, outer)) return;
+    const int rt = MODE == 2 ? outer : inner;
+    const int ct = MODE == 2 ? inner : (MODE == 1 ? outer % g.col_tiles : outer);
+    const int zc = MODE == 1 ? outer / g.col_tiles : 0;
+    const int R = MODE == 2 ? g.M : g.B, C = MODE == 0 ? g.M : g.I;
+    const int KD = MODE == 0 ? g.I : (MODE == 1 ? g.M : g.B);
+    const int k_begin = zc * g.red_chunk, k_end = min(KD, k_begin + g.red_chunk);
+    const bool inside = (rt + 1) * SM_T <= R && (ct + 1) * SM_T <= C && (k_end - k_begin) % KC == 0 &&
+                        g.red_chunk % 4 == 0 && g.I % 4 == 0 && g.M % 4 == 0;
+    if (inside) softmap_tile<MODE, KC, false>(g, sm_lds, rt, ct, zc);
+    else softmap_tile<MODE, KC, true>(g, sm_lds, rt, ct, zc);
+}
+
+template <int MODE, int KC>
+static void softmap_launch(const SoftmapArgs &g, hipStream_t s) {
+    constexpr int LDA = MODE != 2 ? SM_LD_T : SM_LD_V, LDB = MODE == 0 ? SM_LD_T : SM_LD_V;
+    constexpr int lds_bytes = 2 * KC * (LDA + LDB) * (int)sizeof(float);
+    if (lds_bytes > 65536)
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&softmap_mfma<MODE, KC>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    softmap_mfma<MODE, KC><<<dl_xcd_grid(g.inner_count, g.outer_count), 256, lds_bytes, s>>>(g);
+}
+
+// ---------------------------------------------------------------------------------
+// bf16 operands, fp32 accumulation (v_mfma_f32_32x32x16_bf16).  Same tiling and operand modes as
+// the fp32 kernel; operands are rounded to bf16 (nearest even) while they are staged, the row
+// statistics, r and the gW epilogue stay fp32.  A lane feeds the MFMA eight consecutive k of one
+// row, so LDS holds a stage row-major, As[row][32 k] with 16 bytes of padding per row.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+#define SB_K 32   // reduction depth per stage
+#define SB_LD 80  // bytes per LDS row
+
+__device__ __forceinline__ unsigned softmap_pk_bf16(float lo, float hi) {
+    const floatx2 v = {lo, hi};
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2));
+}
+
+template <int MODE, bool EDGE>
+__device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *lds, int rt, int ct, int zc) {
+    constexpr int KC = SB_K, P = 4;
+    constexpr bool A_RED_CONTIG = MODE != 2;
+    constexpr bool B_RED_CONTIG = MODE == 0;
+    constexpr int STAGE = SM_T * SB_LD;  // bytes of one operand stage
+    char *const As = lds;                // [2][128][SB_LD]
+    char *const Bs = lds + 2 * STAGE;
+    const float *__restrict__ x = g.x, *__restrict__ W = g.W, *__restrict__ stats = g.stats, *__restrict__ gm = g.gm;
+    const int B = g.B, I = g.I, M = g.M;
+    const float scale = g.scale;
+    const int R = MODE == 2 ? M : B, C = MODE == 0 ? M : I;
+    const int KD = MODE == 0 ? I : (MODE == 1 ? M : B);
+    const int r0 = rt * SM_T, c0 = ct * SM_T;
+    const int k_begin = zc * g.red_chunk;
+    const int k_end = min(KD, k_begin + g.red_chunk);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    float4 pa[P], pb[P];
+    float bmx[P], brs[P];
+
+    // red-contiguous operand: float4 along k, 8 per row, rows q_o + 32 p.
+    // row/col-contiguous operand: float4 along the row/col axis for one k; piece p holds
+    // k = 2 q_o + (p & 1) + 16 (p >> 1), so pieces 2j and 2j+1 are neighbours in k and go to LDS
+    // as packed pairs.
+    const int a_q = A_RED_CONTIG ? (tid & 7) : (tid & 31), a_o = A_RED_CONTIG ? (tid >> 3) : (tid >> 5);
+    const int b_q = B_RED_CONTIG ? (tid & 7) : (tid & 31), b_o = B_RED_CONTIG ? (tid >> 3) : (tid >> 5);
+    const int lda = MODE == 0 ? I : M;
+    auto k_of = [](int o, int p) { return 2 * o + (p & 1) + 16 * (p >> 1); };
+
+    auto in_a = [&](int row, int k) -> float {
+        if (row >= R || k >= k_end) return 0.0f;
+        if (MODE == 0) return x[(size_t)row * I + k];
+        if (MODE == 1) return gm[(size_t)row * M + k];
+        return gm[(size_t)k * M + row];
+    };
+    auto in_b = [&](int k, int col) -> float {
+        if (col >= C || k >= k_end) return 0.0f;
+        if (MODE == 0) return softmap_s(W[(size_t)col * I + k], stats[2 * col], stats[2 * col + 1], scale);
+        if (MODE == 1) return softmap_s(W[(size_t)k * I + col], stats[2 * k], stats[2 * k + 1], scale);
+        return x[(size_t)k * I + col];
+    };
+    if (!EDGE && MODE == 0) {
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const int col = c0 + b_o + 32 * p;
+            bmx[p] = stats[2 * col]; brs[p] = stats[2 * col + 1];
+        }
+    }
+    auto fetch = [&](int p, int k0) {
+        if (A_RED_CONTIG) {
+            const int row = r0 + a_o + 32 * p, k = k0 + a_q * 4;
+            if (EDGE) pa[p] = make_float4(in_a(row, k), in_a(row, k + 1), in_a(row, k + 2), in_a(row, k + 3));
+            else pa[p] = *reinterpret_cast<const float4 *>((MODE == 0 ? x : gm) + (size_t)row * lda + k);
+        } else {
+            const int k = k0 + k_of(a_o, p), row = r0 + a_q * 4;
+            if (EDGE) pa[p] = make_float4(in_a(row, k), in_a(row + 1, k), in_a(row + 2, k), in_a(row + 3, k));
+            else pa[p] = *reinterpret_cast<const float4 *>(gm + (size_t)k * M + row);
+        }
+        if (B_RED_CONTIG) {
+            const int col = c0 + b_o + 32 * p, k = k0 + b_q * 4;
+            if (EDGE) pb[p] = make_float4(in_b(k, col), in_b(k + 1, col), in_b(k + 2, col), in_b(k + 3, col));
+            else pb[p] = *reinterpret_cast<const float4 *>(W + (size_t)col * I + k);
+        } else {
+            const int k = k0 + k_of(b_o, p), col = c0 + b_q * 4;
+            if (EDGE) pb[p] = make_float4(in_b(k, col), in_b(k, col + 1), in_b(k, col + 2), in_b(k, col + 3));
+            else {
+                pb[p] = *reinterpret_cast<const float4 *>((MODE == 1 ? W : x) + (size_t)k * I + col);
+                if (MODE == 1) { bmx[p] = stats[2 * k]; brs[p] = stats[2 * k + 1]; }
+            }
+        }
+    };
+    auto soft = [&](int p) -> float4 {
+        float4 v = pb[p];
+        if (!EDGE && MODE != 2) {
+            v.x = softmap_s(v.x, bmx[p], brs[p], scale); v.y = softmap_s(v.y, bmx[p], brs[p], scale);
+            v.z = softmap_s(v.z, bmx[p], brs[p], scale); v.w = softmap_s(v.w, bmx[p], brs[p], scale);
+        }
+        return v;
+    };
+    auto commit = [&](int p, int buf) {
+        char *Ab = As + buf * STAGE, *Bb = Bs + buf * STAGE;
+        if (A_RED_CONTIG) {
+            *reinterpret_cast<uint2 *>(Ab + (a_o + 32 * p) * SB_LD + a_q * 8) =
+                make_uint2(softmap_pk_bf16(pa[p].x, pa[p].y), softmap_pk_bf16(pa[p].z, pa[p].w));
+        } else if (p & 1) {
+            char *d = Ab + (a_q * 4) * SB_LD + k_of(a_o, p - 1) * 2;
+            *reinterpret_cast<unsigned *>(d) = softmap_pk_bf16(pa[p - 1].x, pa[p].x);
+            *reinterpret_cast<unsigned *>(d + SB_LD) = softmap_pk_bf16(pa[p - 1].y, pa[p].y);
+            *reinterpret_cast<unsigned *>(d + 2 * SB_LD) = softmap_pk_bf16(pa[p - 1].z, pa[p].z);
+            *reinterpret_cast<unsigned *>(d + 3 * SB_LD) = softmap_pk_bf16(pa[p - 1].w, pa[p].w);
+        }
+        if (B_RED_CONTIG) {
+            const float4 v = soft(p);
+            *reinterpret_cast<uint2 *>(Bb + (b_o + 32 * p) * SB_LD + b_q * 8) =
+                make_uint2(softmap_pk_bf16(v.x, v.y), softmap_pk_bf16(v.z, v.w));
+        } else if (p & 1) {
+            const float4 u = soft(p - 1), v = soft(p);
+            char *d = Bb + (b_q * 4) * SB_LD + k_of(b_o, p - 1) * 2;
+            *reinterpret_cast<unsigned *>(d) = softmap_pk_bf16(u.x, v.x);
+            *reinterpret_cast<unsigned *>(d + SB_LD) = softmap_pk_bf16(u.y, v.y);
+            *reinterpret_cast<unsigned *>(d + 2 * SB_LD) = softmap_pk_bf16(u.z, v.z);
+            *reinterpret_cast<unsigned *>(d + 3 * SB_LD) = softmap_pk_bf16(u.w, v.w);
+        }
+    };
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    const int nst = (k_end - k_begin + KC - 1) / KC;
+    if (nst > 0) {
+#pragma unroll
+        for (int p = 0; p < P; ++p) fetch(p, k_begin);
+#pragma unroll
+        for (int p = 0; p < P; ++p) commit(p, 0);
+        if (nst > 1) {
+#pragma unroll
+            for (int p = 0; p < P; ++p) fetch(p, k_begin + KC);
+        }
+    }
+    __syncthreads();
+    const int kh = lane >> 5, l32 = lane & 31;
+    auto stage = [&](int s, auto do_commit, auto do_fetch) {
+        const int cur = s & 1;
+        const char *Ab = As + cur * STAGE + (wm + l32) * SB_LD + kh * 16;
+        const char *Bb = Bs + cur * STAGE + (wn + l32) * SB_LD + kh * 16;
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+            const bf16x8 a0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(Ab + kk * 32));
+            const bf16x8 a1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(Ab + 32 * SB_LD + kk * 32));
+            const bf16x8 b0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(Bb + kk * 32));
+            const bf16x8 b1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(Bb + 32 * SB_LD + kk * 32));
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b0, acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b1, acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b0, acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b1, acc[1][1], 0, 0, 0);
+            if constexpr (decltype(do_commit)::value) { commit(2 * kk, cur ^ 1); commit(2 * kk + 1, cur ^ 1); }
+            if constexpr (decltype(do_fetch)::value) {
+                fetch(2 * kk, k_begin + (s + 2) * KC);
+                fetch(2 * kk + 1, k_begin + (s + 2) * KC);
+            }
+        }
+        __syncthreads();
+    };
+    {
+        using T = std::true_type;
+        using F = std::false_type;
+        int s = 0;
+        for (; s + 2 < nst; ++s) stage(s, T{}, T{});
+        if (s + 1 < nst) { stage(s, T{}, F{}); ++s; }
+        if (s < nst) stage(s, F{}, F{});
+    }
+    float *dst = g.out + (size_t)zc * R * C;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int col = c0 + wn + j * 32 + (lane & 31);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = r0 + wm + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                if (!EDGE || (row < R && col < C)) {
+                    float val = acc[i][j][v];
+                    if (MODE == 2) {
+                        const float sv = softmap_s(W[(size_t)row * I + col], stats[2 * row], stats[2 * row + 1], scale);
+                        val = sv * (val - g.r[row]) * g.inv_tau;
+                    }
+                    dst[(size_t)row * C + col] = val;
+                }
+            }
+        }
+}
+
+template <int MODE>
+__global__ __launch_bounds__(256) void softmap_mfma_bf16(SoftmapArgs g) {
+    __shared__ __align__(16) char lds[4 * SM_T * SB_LD];
+    int inner, outer;
+    if (!dl_xcd_map(g.inner_count, g.outer_count, inner, outer)) return;
+    const int rt = MODE == 2 ? outer : inner;
+    const int ct = MODE == 2 ? inner : (MODE == 1 ? outer % g.col_tiles : outer);
+    const int zc = MODE == 1 ? outer / g.col_tiles : 0;
+    const int R = MODE == 2 ? g.M : g.B, C = MODE == 0 ? g.M : g.I;
+    const int KD = MODE == 0 ? g.I : (MODE == 1 ? g.M : g.B);
+    const int k_begin = zc * g.red_chunk, k_end = min(KD, k_begin + g.red_chunk);
+    const bool inside = (rt + 1) * SM_T <= R && (ct + 1) * SM_T <= C && (k_end - k_begin) % SB_K == 0 &&
+                        g.red_chunk % 4 == 0 && g.I % 4 == 0 && g.M % 4 == 0;
+    if (inside) softmap_tile_bf16<MODE, false>(g, lds, rt, ct, zc);
+    else softmap_tile_bf16<MODE, true>(g, lds, rt, ct, zc);
+}
+
+template <int MODE>
+static void softmap_launch_bf16(const SoftmapArgs &g, hipStream_t s) {
+    softmap_mfma_bf16<MODE><<<dl_xcd_grid(g.inner_count, g.outer_count), 256, 0, s>>>(g);
+}
+
 // ---------------------------------------------------------------------------------
 static int softmap_check(int B, int I, int M, int precision) {
     if (B <= 0 || I <= 0 || M <= 0) return DL_ERR_SHAPE;
-    if (precision != 0) return DL_ERR_UNSUPPORTED;  // bf16 operands: not built yet
+    if (precision != 0 && precision != 1) return DL_ERR_UNSUPPORTED;
     return DL_OK;
 }
 
-// the gx product reduces over M; it is cut into chunks so that the grid fills the chip
+// The gx product reduces over M.  It is cut into chunks so that the grid fills the chip: the chunk
+// count is the one whose block count comes closest to whole rounds of the 768 resident blocks
+// (256 CUs x 3 blocks), smallest count first on ties.
 static inline int softmap_gx_chunks(int B, int I, int M) {
-    const int tiles = dl_ceil_div(I, SM_T) * dl_ceil_div(B, SM_T);
-    int chunks = dl_ceil_div(1024, tiles);
-    const int max_chunks = dl_ceil_div(M, 4 * SM_K);
-    if (chunks > max_chunks) chunks = max_chunks;
-    return chunks < 1 ? 1 : chunks;
+    const long long tiles = (long long)dl_ceil_div(I, SM_T) * dl_ceil_div(B, SM_T);
+    const int max_chunks = dl_ceil_div(M, 256);
+    const int lo = dl_ceil_div(512, tiles), hi = dl_ceil_div(2304, tiles);
+    int best = 1;
+    double best_fill = 0.0;
+    for (int c = lo < 1 ? 1 : lo; c <= hi && c <= max_chunks; ++c) {
+        const long long blocks = tiles * c;
+        const double fill = (double)blocks / (double)(((blocks + 767) / 768) * 768);
+        if (fill > best_fill + 1e-9) { best_fill = fill; best = c; }
+    }
+    return best;
 }
 
 extern "C" size_t dl_soft_map_workspace_bytes(int B, int I, int M, int precision) {
@@ -246,11 +611,12 @@ extern "C" int dl_soft_map_fwd(const float *x, const float *W, float tau, float 
     if (rc) return rc;
     if (!(tau > 0.0f)) return DL_ERR_SHAPE;
     hipStream_t s = (hipStream_t)stream;
-    const float inv_tau = 1.0f / tau;
-    DL_TIMED("softmap_rowstats", s, (softmap_rowstats<<<dl_ceil_div(M, 4), 256, 0, s>>>(W, inv_tau, stats, M, I)));
-    DL_TIMED("softmap_mfma_fwd", s,
-             (softmap_mfma<0><<<dim3(dl_ceil_div(M, SM_T), dl_ceil_div(B, SM_T), 1), 256, 0, s>>>(
-                 x, W, stats, nullptr, nullptr, inv_tau, m, B, I, M, I)));
+    const float inv_tau = 1.0f / tau, scale = SM_LOG2E / tau;
+    DL_TIMED("softmap_rowstats", s, (softmap_rowstats<<<dl_ceil_div(M, 4), 256, 0, s>>>(W, scale, stats, M, I)));
+    const SoftmapArgs g{x, W, stats, nullptr, nullptr, scale, inv_tau, m, B, I, M,
+                        dl_ceil_div(B, SM_T), dl_ceil_div(M, SM_T), 1, dl_ceil_div(I, 4) * 4};
+    if (precision == 1) DL_TIMED("softmap_bf16_fwd", s, (softmap_launch_bf16<0>(g, s)));
+    else DL_TIMED("softmap_mfma_fwd", s, (softmap_launch<0, SM_K0>(g, s)));
     return dl_launch_status();
 }
 
@@ -263,22 +629,25 @@ extern "C" int dl_soft_map_bwd(const float *x, const float *W, float tau, const 
     if (!(tau > 0.0f)) return DL_ERR_SHAPE;
     if (ws_bytes < dl_soft_map_workspace_bytes(B, I, M, precision)) return DL_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
-    const float inv_tau = 1.0f / tau;
+    const float inv_tau = 1.0f / tau, scale = SM_LOG2E / tau;
     float *r = (float *)ws;
     float *part = (float *)((char *)ws + dl_align256((size_t)M * sizeof(float)));
     const int chunks = softmap_gx_chunks(B, I, M);
     int red_chunk = dl_ceil_div(M, chunks);
-    red_chunk = dl_ceil_div(red_chunk, SM_K) * SM_K;  // whole stages, so float4 loads stay aligned
-    DL_TIMED("softmap_rowdot", s, (softmap_rowdot<<<dl_ceil_div(M, 256), 256, 0, s>>>(gm, m, r, B, M)));
-    DL_TIMED("softmap_mfma_gx", s,
-             (softmap_mfma<1><<<dim3(dl_ceil_div(I, SM_T), dl_ceil_div(B, SM_T), dl_ceil_div(M, red_chunk)), 256, 0, s>>>(
-                 x, W, stats, gm, nullptr, inv_tau, chunks > 1 ? part : gx, B, I, M, red_chunk)));
-    if (chunks > 1)
+    red_chunk = dl_ceil_div(red_chunk, 32) * 32;  // whole stages, so float4 loads stay aligned
+    const int col_tiles = dl_ceil_div(I, SM_T), used_chunks = dl_ceil_div(M, red_chunk);
+    DL_TIMED("softmap_rowdot", s, (softmap_rowdot<<<dl_ceil_div(M, 32), 256, 0, s>>>(gm, m, r, B, M)));
+    const SoftmapArgs ggx{x, W, stats, gm, nullptr, scale, inv_tau, used_chunks > 1 ? part : gx, B, I, M,
+                          dl_ceil_div(B, SM_T), col_tiles * used_chunks, col_tiles, red_chunk};
+    if (precision == 1) DL_TIMED("softmap_bf16_gx", s, (softmap_launch_bf16<1>(ggx, s)));
+    else DL_TIMED("softmap_mfma_gx", s, (softmap_launch<1, SM_K1>(ggx, s)));
+    if (used_chunks > 1)
         DL_TIMED("softmap_reduce_chunks", s,
                  (softmap_reduce_chunks<<<dl_ceil_div((long long)B * I, 256), 256, 0, s>>>(part, gx, (long long)B * I,
-                                                                                         dl_ceil_div(M, red_chunk))));
-    DL_TIMED("softmap_mfma_gw", s,
-             (softmap_mfma<2><<<dim3(dl_ceil_div(I, SM_T), dl_ceil_div(M, SM_T), 1), 256, 0, s>>>(
-                 x, W, stats, gm, r, inv_tau, gW, B, I, M, B)));
+                                                                                         used_chunks)));
+    const SoftmapArgs ggw{x, W, stats, gm, r, scale, inv_tau, gW, B, I, M,
+                          col_tiles, dl_ceil_div(M, SM_T), 1, dl_ceil_div(B, 4) * 4};
+    if (precision == 1) DL_TIMED("softmap_bf16_gw", s, (softmap_launch_bf16<2>(ggw, s)));
+    else DL_TIMED("softmap_mfma_gw", s, (softmap_launch<2, SM_K2>(ggw, s)));
     return dl_launch_status();
 }

@@ -218,6 +218,30 @@ def test_soft_mapping_forward_backward_fp32(shape, tau):
     np.testing.assert_allclose(Wt.grad.cpu().numpy(), gW, rtol=1e-4, atol=1e-5 / tau)
 
 
+@pytest.mark.parametrize("shape,tau", [((5, 20, 21), 1.0), ((256, 384, 1000), 1.0), ((130, 260, 516), 0.5),
+                                       ((129, 132, 4100), 2.0), ((128, 256, 384), 1.0)])
+def test_soft_mapping_bf16_operands(shape, tau):
+    """precision=1 rounds x, S and gm to bf16 (8 significant bits, relative step 2^-8) before the
+    MFMA and accumulates in fp32.  Tolerance: 1e-2 of the largest reference magnitude per tensor
+    (rounding errors of the summands are independent, so the sums do better than 2^-8)."""
+    ops = _ops()
+    B, I, M = shape
+    rng = np.random.default_rng(sum(shape) + 1)
+    x = rng.random((B, I)).astype(np.float32)
+    W = (rng.standard_normal((M, I)) * 0.5).astype(np.float32)
+    gm = rng.standard_normal((B, M)).astype(np.float32)
+    xt = dev(x).requires_grad_(); Wt = dev(W).requires_grad_()
+    m = ops.SoftMapFunction.apply(xt, Wt, tau, 1)
+    want_m = orc.soft_mapping_forward(x, W, tau, torch.float64)
+    got_m = m.detach().cpu().numpy()
+    assert np.abs(got_m - want_m).max() <= 1e-2 * np.abs(want_m).max()
+    assert np.abs(got_m - want_m).max() > 0  # the bf16 path ran, not the fp32 one
+    m.backward(dev(gm))
+    gx, gW = orc.soft_mapping_backward(x, W, gm, tau)
+    assert np.abs(xt.grad.cpu().numpy() - gx).max() <= 1e-2 * np.abs(gx).max()
+    assert np.abs(Wt.grad.cpu().numpy() - gW).max() <= 1e-2 * np.abs(gW).max()
+
+
 def test_soft_and_hard_mapping_against_reference_vectors(golden):
     ops = _ops()
     g = golden
