@@ -329,7 +329,7 @@ __device__ __forceinline__ void softmap_tile(const SoftmapArgs &g, float *sm_lds
 // MODE 2) sit next to each other on one XCD and find it in that XCD's L2.  MODE 1 also carries a
 // chunk of the reduction in the block index; out then points at [chunks][R][C] partial products.
 template <int MODE, int KC>
-__global__ __launch_bounds__(256) void softmap_mfma(SoftmapArgs g) {
+__global__ __launch_bounds__(256, 3) void softmap_mfma(SoftmapArgs g) {
     extern __shared__ __align__(16) float sm_lds[];
     int inner, outer;
     if (!dl_xcd_map(g.inner_count, g.outer_count, inner, outer)) return;
@@ -551,7 +551,7 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
 }
 
 template <int MODE>
-__global__ __launch_bounds__(256) void softmap_mfma_bf16(SoftmapArgs g) {
+__global__ __launch_bounds__(256, 3) void softmap_mfma_bf16(SoftmapArgs g) {
     __shared__ __align__(16) char lds[4 * SM_T * SB_LD];
     int inner, outer;
     if (!dl_xcd_map(g.inner_count, g.outer_count, inner, outer)) return;
