@@ -115,6 +115,10 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
     const int lane = threadIdx.x & 63;
     const int wave = dl_uniform(threadIdx.x >> 6);
     const u64 *pl = planes + (size_t)t * I;
+    const __amdgpu_buffer_rsrc_t rs_luts = __builtin_amdgcn_make_buffer_rsrc((void *)luts, 0, NO * L * 4, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_addr =
+        __builtin_amdgcn_make_buffer_rsrc((void *)(addrT + (size_t)t * N * 64), 0, N * 64, 0x00020000);
+    const int lane4s = (lane & (L - 1)) * 4;
     const int cend = min(DWN_TC, NO - c0);
     const int wbeg = wave * DWN_WC;
     // slot s = (column within my 16) * K + j  ->  lane s % 64 of register s / 64
@@ -123,7 +127,7 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
     for (int v = 0; v < NIDX; ++v) {
         const int s = v * 64 + lane;
         const int c = min(c0 + wbeg + min(s / K, DWN_WC - 1), NO - 1);
-        myidx[v] = idx32[(O1 ? c : c / O) * K + s % K];
+        myidx[v] = idx32[(O1 ? c : c / O) * K + s % K] * 8;  // byte offset of the input's plane word
     }
     if (wbeg < cend) {
 #pragma unroll
@@ -133,14 +137,17 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
 #pragma unroll
             for (int q = 0; q < DWN_CG; ++q) {
                 const int c = min(c0 + wbeg + g + q, NO - 1);
-                entry[q] = luts[(size_t)c * L + (lane & (L - 1))];
+                // table row of column c, one entry per lane; the row offset travels in an SGPR
+                entry[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_luts, lane4s, c * (L * 4), 0));
 #pragma unroll
                 for (int j = 0; j < K; ++j) {
                     constexpr int dummy = 0;
                     (void)dummy;
                     const int s = (g + q) * K + j;  // compile-time after unrolling
-                    const int src = __builtin_amdgcn_readlane(myidx[s / 64], s % 64);
-                    w[q][j] = pl[src];  // wave-uniform address: scalar load
+                    // wave-uniform unsigned byte offset: a scalar load with the offset in an SGPR,
+                    // no scalar address arithmetic
+                    const unsigned src = (unsigned)__builtin_amdgcn_readlane(myidx[s / 64], s % 64);
+                    w[q][j] = *reinterpret_cast<const u64 *>(reinterpret_cast<const char *>(pl) + src);
                 }
             }
 #pragma unroll
@@ -154,7 +161,7 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
                     tile[cc][lane] = v;
                     const int c = c0 + cc;
                     const int n = O1 ? c : c / O;
-                    if (O1 || c - n * O == 0) addrT[((size_t)t * N + n) * 64 + lane] = (uint8_t)addr;
+                    if (O1 || c - n * O == 0) __builtin_amdgcn_raw_buffer_store_b8((uint8_t)addr, rs_addr, lane, n * 64, 0);
                 }
             }
         }
@@ -451,6 +458,7 @@ static inline size_t dwn_gyT_bytes(int B, int N, int O) {
 static int dwn_check(int B, int I, int N, int k, int O) {
     if (B <= 0 || I <= 0 || N <= 0 || k <= 0 || O <= 0) return DL_ERR_SHAPE;
     if (k > DL_MAX_K) return DL_ERR_UNSUPPORTED;
+    if (I > (1 << 28)) return DL_ERR_UNSUPPORTED;  // byte offsets into one batch tile's bit-planes are 32-bit
     if ((long long)N * O * ((long long)1 << k) > 0x7fffffffLL) return DL_ERR_UNSUPPORTED;
     return DL_OK;
 }
