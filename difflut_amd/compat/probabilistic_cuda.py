@@ -18,8 +18,11 @@ def forward(input, raw_weights, temperature):
     L, O = raw_weights.shape
     y = torch.empty((B, O), dtype=torch.float32, device=input.device)
     plan = _plan(k, input.device)
-    nat.check(nat.lib().dl_prob_layer_fwd(input.data_ptr(), plan.idx32.data_ptr(), raw_weights.data_ptr(),
-                                          float(temperature), y.data_ptr(), B, k, 1, k, O, nat.stream()))
+    lib = nat.lib()
+    ws = torch.empty(max(lib.dl_prob_fwd_workspace_bytes(B, k, 1, k, O), 256), dtype=torch.uint8, device=input.device)
+    nat.check(lib.dl_prob_layer_fwd(input.data_ptr(), plan.idx32.data_ptr(), raw_weights.data_ptr(),
+                                    float(temperature), y.data_ptr(), ws.data_ptr(), ws.numel(), B, k, 1, k, O,
+                                    nat.stream()))
     return y
 
 

@@ -2,191 +2,268 @@
 //   y[b,n,d] = sum_a sigmoid(w[n,a,d]/T) * prod_j (x_j a_j + (1-x_j)(1-a_j)),  x_j = x[b, idx[n,j]]
 // i.e. the multilinear interpolation of the node's sigmoid table at the point x.
 //
-// k <= 6: a thread owns one node; its 2^k table entries live in registers (all of them are
-// touched by every evaluation, in a fixed order, so no dynamic indexing is needed), the rows of
-// x are staged in LDS and shared by the block's 256 nodes, writes of y are coalesced.
-//   forward : folds the table along x_0, x_1, ... (2^k - 1 lerps)
-//   backward: the same fold run backwards gives dy/dx_j and dy/dtable in O(2^k):
-//             table-gradient partials are kept in registers over the block's rows and written
-//             once per block to a partial buffer that a second kernel reduces in fixed order
-//             (and scales by sigmoid'(w/T)/T); input-gradient terms go to a [B,N,k] buffer
-//             that the CSR gather of the mapping sums in fixed order.
-// k > 6: one-thread-per-element kernels with atomics.
+// k <= 6: tiled kernels with lanes = batch rows (see below); k > 6: one-thread-per-element kernels
+// with atomics.
 #include "dl_common.h"
 
 __device__ __forceinline__ float dl_sigmoid(float v) { return 1.0f / (1.0f + expf(-v)); }
 
-#define PROB_NODES 256  // nodes (= threads) per block
-#define PROB_ROWS 16    // batch rows per block in the forward
-
-
-// Row staging shared by the forward and backward kernels: the block's next row of x is fetched
-// into registers (up to PROB_PRE float4 per thread, i.e. rows of up to 4096 floats) while the
-// current one is being used from LDS, so only one barrier pair per row sits on the critical path.
-// Wider or unaligned rows are staged directly.
-#define PROB_PRE 4
-struct ProbRowStage {
-    float4 pre[PROB_PRE];
-    bool vec;
-    __device__ void init(const float *x, int I) { vec = (I % 4 == 0) && I <= 4 * PROB_NODES * PROB_PRE && (((size_t)x & 15) == 0); }
-    __device__ void fetch(const float *x, int I, int b) {
-        if (!vec) return;
-        const float4 *row = reinterpret_cast<const float4 *>(x + (size_t)b * I);
-#pragma unroll
-        for (int u = 0; u < PROB_PRE; ++u) {
-            const int q = u * PROB_NODES + threadIdx.x;
-            if (q * 4 < I) pre[u] = row[q];
-        }
-    }
-    // call between two __syncthreads(): the first guards the previous row's readers
-    __device__ void commit(float *xrow, const float *x, int I, int b) {
-        if (vec) {
-#pragma unroll
-            for (int u = 0; u < PROB_PRE; ++u) {
-                const int q = u * PROB_NODES + threadIdx.x;
-                if (q * 4 < I) reinterpret_cast<float4 *>(xrow)[q] = pre[u];
-            }
-        } else {
-            for (int i = threadIdx.x; i < I; i += PROB_NODES) xrow[i] = x[(size_t)b * I + i];
-        }
-    }
-};
+typedef float prob_f4 __attribute__((ext_vector_type(4)));
+#define PROB_RSRC 0x00020000
 
 // ---------------------------------------------------------------------------------
+// k <= 6 path.  As for the DWN nodes, a wavefront's 64 lanes are 64 batch rows and everything
+// that belongs to a node is wave-uniform: its input indices are scalar byte offsets, its sigmoid
+// table is read through scalar loads.  Tensors that cross the [batch, feature] boundary are
+// re-tiled once: xT [B/64][I][64], gyT [B/64][N*O][64], gmT [B/64][N*O*k][64], so the row of an
+// input (or a column's gradient) for a batch tile is 256 contiguous bytes, whatever the mapping.
+//   sig_table   : sig[c][a] = sigmoid(raw[n,a,d] / T), c = n*O + d                (tiny)
+//   to_tiles    : [B][C] -> [B/64][C][64], rows past B are zero                    (x, gy)
+//   fwd_t       : per (column, batch tile): fold the table along x_0, x_1, ... ; y leaves through
+//                 an LDS transpose as whole rows
+//   bwd_t       : one wavefront per column over a chunk of batch tiles.  The fold is run forward
+//                 keeping the differences of every level, then backward: that gives dy/dx_j for
+//                 all j and, at the bottom, p_a = dy/dtable_a (the product weights) in about
+//                 5 * 2^k operations.  Table-gradient partials stay in registers over the chunk,
+//                 are summed across lanes once and written per chunk; gm_j goes to gmT.
+//   reduce      : fixed-order sum of the chunk partials, times sigmoid'(w/T)/T
+//   gather_t    : gx[b,i] = sum over the CSR entries (n,j) of input i (and d) of gmT: a wavefront
+//                 owns 16 inputs, sums each in CSR order in a register, rows leave through LDS.
+__global__ __launch_bounds__(256) void prob_sig_table(const float *__restrict__ raw, float inv_t, float *__restrict__ sig,
+                                                       int N, int L, int O) {
+    const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (e >= (long long)N * L * O) return;
+    const int a = (int)(e % L);
+    const long long c = e / L;
+    const int n = (int)(c / O), d = (int)(c % O);
+    sig[e] = dl_sigmoid(raw[((size_t)n * L + a) * O + d] * inv_t);
+}
+
+// grid (ceil(C / 64), B/64 rounded up), 256 threads
+__global__ __launch_bounds__(256) void prob_to_tiles(const float *__restrict__ src, float *__restrict__ dst, int B, int C) {
+    __shared__ float tile[64][65];  // [column][row]
+    const int t = blockIdx.y, c0 = blockIdx.x * 64;
+    for (int e = threadIdx.x; e < 4096; e += 256) {
+        const int r = e >> 6, c = e & 63;
+        const int b = t * 64 + r;
+        tile[c][r] = (b < B && c0 + c < C) ? src[(size_t)b * C + c0 + c] : 0.0f;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < 4096; e += 256) {
+        const int c = e >> 6, r = e & 63;
+        if (c0 + c < C) dst[((size_t)t * C + c0 + c) * 64 + r] = tile[c][r];
+    }
+}
+
+// table of one column as wave-uniform values
 template <int K>
-__global__ __launch_bounds__(PROB_NODES) void prob_fwd_kernel(const float *__restrict__ x, const int *__restrict__ idx32,
-                                                               const float *__restrict__ raw, float inv_t,
-                                                               float *__restrict__ y, int B, int I, int N, int O,
-                                                               int rows_per_block) {
-    extern __shared__ __align__(16) float xrow[];  // I floats
-    constexpr int L = 1 << K;
-    const int n = blockIdx.x * PROB_NODES + threadIdx.x;
-    const bool live = n < N;
-    int src[K];
+__device__ __forceinline__ void prob_load_table(const float *__restrict__ sig, int c, float (&tab)[1 << K]) {
+    const float *row = sig + (size_t)c * (1 << K);
 #pragma unroll
-    for (int j = 0; j < K; ++j) src[j] = live ? idx32[(size_t)n * K + j] : 0;
-    const int b0 = blockIdx.y * rows_per_block;
-    const int b1 = min(B, b0 + rows_per_block);
-    for (int d = 0; d < O; ++d) {
+    for (int a = 0; a < (1 << K); ++a) tab[a] = row[a];
+}
+
+#define PROB_TC 128                    // columns per block
+#define PROB_FW 8                      // wavefronts per block
+#define PROB_WC (PROB_TC / PROB_FW)    // columns per wavefront
+template <int K>
+__global__ __launch_bounds__(64 * PROB_FW) void prob_fwd_t(const float *__restrict__ xT, const int *__restrict__ idx32,
+                                                            const float *__restrict__ sig, float *__restrict__ y,
+                                                            int B, int I, int N, int O, int BT) {
+    __shared__ float tile[PROB_TC][65];  // [column][row]
+    constexpr int L = 1 << K;
+    const int NO = N * O;
+    int ctile, t;
+    if (!dl_xcd_map((NO + PROB_TC - 1) / PROB_TC, BT, ctile, t)) return;
+    const int c0 = ctile * PROB_TC;
+    const int lane = threadIdx.x & 63;
+    const int wave = dl_uniform(threadIdx.x >> 6);
+    const int cend = min(PROB_TC, NO - c0);
+    const int wbeg = wave * PROB_WC;
+    const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc((void *)(xT + (size_t)t * I * 64), 0, I * 256, PROB_RSRC);
+    const int lane4 = lane * 4;
+    for (int q = 0; q < PROB_WC; ++q) {
+        const int cc = wbeg + q;
+        if (cc >= cend) break;  // wave-uniform
+        const int c = c0 + cc;
+        const int n = c / O;
+        float xs[K];
+#pragma unroll
+        for (int j = 0; j < K; ++j)
+            xs[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_x, lane4, idx32[(size_t)n * K + j] * 256, 0));
         float tab[L];
+        prob_load_table<K>(sig, c, tab);
+        float v[L / 2 > 0 ? L / 2 : 1];
+        {
+            const float om = 1.0f - xs[0];
 #pragma unroll
-        for (int a = 0; a < L; ++a) tab[a] = live ? dl_sigmoid(raw[((size_t)n * L + a) * O + d] * inv_t) : 0.0f;
-        ProbRowStage stage;
-        stage.init(x, I);
-        if (b0 < b1) stage.fetch(x, I, b0);
-        for (int b = b0; b < b1; ++b) {
-            __syncthreads();
-            stage.commit(xrow, x, I, b);
-            __syncthreads();
-            if (b + 1 < b1) stage.fetch(x, I, b + 1);
-            float v[L];
-#pragma unroll
-            for (int a = 0; a < L; ++a) v[a] = tab[a];
-#pragma unroll
-            for (int j = 0; j < K; ++j) {  // fold bit j: entries a and a + 2^j with bit j clear
-                const float xj = xrow[src[j]];
-#pragma unroll
-                for (int a = 0; a < (L >> (j + 1)); ++a) v[a] = v[2 * a] + xj * (v[2 * a + 1] - v[2 * a]);
-            }
-            if (live) y[((size_t)b * N + n) * O + d] = v[0];
+            for (int a = 0; a < L / 2; ++a) v[a] = fmaf(tab[2 * a + 1], xs[0], tab[2 * a] * om);
         }
+#pragma unroll
+        for (int j = 1; j < K; ++j) {
+#pragma unroll
+            for (int a = 0; a < (L >> (j + 1)); ++a) v[a] = v[2 * a] + xs[j] * (v[2 * a + 1] - v[2 * a]);
+        }
+        tile[cc][lane] = v[0];
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < 64 * PROB_TC; e += 64 * PROB_FW) {
+        const int r = e / PROB_TC, cc = e % PROB_TC;
+        const int b = t * 64 + r;
+        if (b < B && cc < cend) __builtin_nontemporal_store(tile[cc][r], &y[(size_t)b * NO + c0 + cc]);
     }
 }
 
-// ---------------------------------------------------------------------------------
-// Backward main kernel.  gm [B,N,k] receives dL/d(mapped input); gpart [chunks][N*L*O] the
-// per-block sums of gy * p_a (before the sigmoid-derivative factor).
+// one wavefront per (column, chunk of batch tiles); 4 wavefronts per block
 template <int K>
-__global__ __launch_bounds__(PROB_NODES) void prob_bwd_kernel(const float *__restrict__ x, const int *__restrict__ idx32,
-                                                               const float *__restrict__ raw, float inv_t,
-                                                               const float *__restrict__ gy, float *__restrict__ gm,
-                                                               float *__restrict__ gpart, int B, int I, int N, int O,
-                                                               int rows_per_block, int want_gm) {
-    extern __shared__ __align__(16) float xrow[];
+__global__ __launch_bounds__(256) void prob_bwd_t(const float *__restrict__ xT, const float *__restrict__ gyT,
+                                                   const int *__restrict__ idx32, const float *__restrict__ sig,
+                                                   float *__restrict__ gmT, float *__restrict__ gpart, int I, int N,
+                                                   int O, int BT, int tiles_per_chunk, int want_gm) {
     constexpr int L = 1 << K;
-    const int n = blockIdx.x * PROB_NODES + threadIdx.x;
-    const bool live = n < N;
-    int src[K];
+    const int NO = N * O;
+    const int lane = threadIdx.x & 63;
+    const int c = blockIdx.x * 4 + dl_uniform(threadIdx.x >> 6);
+    if (c >= NO) return;
+    const int chunk = blockIdx.y;
+    const int n = c / O;
+    const int lane4 = lane * 4;
+    int off[K];
 #pragma unroll
-    for (int j = 0; j < K; ++j) src[j] = live ? idx32[(size_t)n * K + j] : 0;
-    const int b0 = blockIdx.y * rows_per_block;
-    const int b1 = min(B, b0 + rows_per_block);
-    for (int d = 0; d < O; ++d) {
-        float tab[L], gt[L];
+    for (int j = 0; j < K; ++j) off[j] = idx32[(size_t)n * K + j] * 256;
+    float tab[L];
+    prob_load_table<K>(sig, c, tab);
+    float acc[L];
 #pragma unroll
-        for (int a = 0; a < L; ++a) {
-            tab[a] = live ? dl_sigmoid(raw[((size_t)n * L + a) * O + d] * inv_t) : 0.0f;
-            gt[a] = 0.0f;
+    for (int a = 0; a < L; ++a) acc[a] = 0.0f;
+    const int t0 = chunk * tiles_per_chunk, t1 = min(BT, t0 + tiles_per_chunk);
+    for (int t = t0; t < t1; ++t) {
+        const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc((void *)(xT + (size_t)t * I * 64), 0, I * 256, PROB_RSRC);
+        float xs[K];
+#pragma unroll
+        for (int j = 0; j < K; ++j) xs[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_x, lane4, off[j], 0));
+        const float g = gyT[((size_t)t * NO + c) * 64 + lane];
+        // forward fold, keeping the differences d_j[a] = lvl_j[2a+1] - lvl_j[2a] of every level
+        float diff[L > 1 ? L - 1 : 1];  // level j occupies [L - (L >> j), L - (L >> (j+1)))
+        float v[L / 2 > 0 ? L / 2 : 1];
+#pragma unroll
+        for (int a = 0; a < L / 2; ++a) {
+            diff[a] = tab[2 * a + 1] - tab[2 * a];
+            v[a] = fmaf(xs[0], diff[a], tab[2 * a]);
         }
-        ProbRowStage stage;
-        stage.init(x, I);
-        if (b0 < b1) stage.fetch(x, I, b0);
-        for (int b = b0; b < b1; ++b) {
-            __syncthreads();
-            stage.commit(xrow, x, I, b);
-            __syncthreads();
-            if (b + 1 < b1) stage.fetch(x, I, b + 1);
-            float xs[K];
+        int base = L / 2;
 #pragma unroll
-            for (int j = 0; j < K; ++j) xs[j] = xrow[src[j]];
-            const float g = live ? gy[((size_t)b * N + n) * O + d] : 0.0f;
-            // p[a] = prod_j (a_j ? x_j : 1 - x_j), built by doubling: after step j, p[0 .. 2^(j+1)) is
-            // the product over inputs 0..j
-            float p[L];
-            p[0] = 1.0f;
+        for (int j = 1; j < K; ++j) {
 #pragma unroll
-            for (int j = 0; j < K; ++j) {
-#pragma unroll
-                for (int a = (1 << j) - 1; a >= 0; --a) {
-                    p[a + (1 << j)] = p[a] * xs[j];
-                    p[a] = p[a] * (1.0f - xs[j]);
-                }
+            for (int a = 0; a < (L >> (j + 1)); ++a) {
+                diff[base + a] = v[2 * a + 1] - v[2 * a];
+                v[a] = fmaf(xs[j], diff[base + a], v[2 * a]);
             }
+            base += L >> (j + 1);
+        }
+        // backward: bar_K[0] = 1; dx_j = sum_a bar_{j+1}[a] d_j[a]; bar_j[2a] = bar_{j+1}[a] (1 - x_j), bar_j[2a+1] = bar_{j+1}[a] x_j
+        float bar[L];
+        bar[0] = 1.0f;
+        float dx[K];
 #pragma unroll
-            for (int a = 0; a < L; ++a) gt[a] += g * p[a];
-            if (want_gm) {
-                // dy/dx_j = sum_a tab[a] (2 a_j - 1) prod_{m != j} q_m: fold the table along every input but j
+        for (int j = K - 1; j >= 0; --j) {
+            base -= L >> (j + 1);
+            const int cnt = L >> (j + 1);
+            float sum = 0.0f;
 #pragma unroll
-                for (int j = 0; j < K; ++j) {
-                    float v[L / 2 > 0 ? L / 2 : 1];
+            for (int a = 0; a < cnt; ++a) sum = fmaf(bar[a], diff[base + a], sum);
+            dx[j] = sum;
+            const float om = 1.0f - xs[j];
 #pragma unroll
-                    for (int a = 0; a < L / 2; ++a) {
-                        const int lo = (a & ((1 << j) - 1)) | ((a >> j) << (j + 1));
-                        v[a] = tab[lo | (1 << j)] - tab[lo];
-                    }
-                    int m = 0;
-#pragma unroll
-                    for (int jj = 0; jj < K; ++jj) {
-                        if (jj == j) continue;
-#pragma unroll
-                        for (int a = 0; a < (L >> (m + 2)); ++a) v[a] = v[2 * a] + xs[jj] * (v[2 * a + 1] - v[2 * a]);
-                        ++m;
-                    }
-                    if (live) {
-                        float *dst = gm + ((size_t)b * N + n) * K + j;
-                        if (d == 0) *dst = g * v[0]; else *dst += g * v[0];
-                    }
-                }
+            for (int a = cnt - 1; a >= 0; --a) {
+                const float w = bar[a];
+                bar[2 * a + 1] = w * xs[j];
+                bar[2 * a] = w * om;
             }
         }
-        if (live) {
-            float *dst = gpart + (size_t)blockIdx.y * N * L * O + (size_t)n * L * O + d;
 #pragma unroll
-            for (int a = 0; a < L; ++a) dst[(size_t)a * O] = gt[a];
+        for (int a = 0; a < L; ++a) acc[a] = fmaf(g, bar[a], acc[a]);
+        if (want_gm) {
+#pragma unroll
+            for (int j = 0; j < K; ++j) gmT[(((size_t)t * NO + c) * K + j) * 64 + lane] = g * dx[j];
         }
     }
+    // sum the 64 per-row partials of every table entry, lane a keeps entry a
+    float mine = 0.0f;
+#pragma unroll
+    for (int a = 0; a < L; ++a) {
+        float r = acc[a];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) r += __shfl_xor(r, o);
+        if (lane == a) mine = r;
+    }
+    if (lane < L) gpart[((size_t)chunk * NO + c) * L + lane] = mine;
 }
 
-// graw[e] = sigmoid'(w/T)/T * sum over chunks of gpart[chunk][e]
-__global__ __launch_bounds__(256) void prob_reduce_weights(const float *__restrict__ gpart, const float *__restrict__ raw,
-                                                            float inv_t, float *__restrict__ graw, long long total,
+// graw[n,a,d] = sigmoid'(w/T)/T * sum over chunks of gpart[chunk][c][a]
+__global__ __launch_bounds__(256) void prob_reduce_weights(const float *__restrict__ gpart, const float *__restrict__ sig,
+                                                            float inv_t, float *__restrict__ graw, int N, int L, int O,
                                                             int chunks) {
     const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long total = (long long)N * L * O;
     if (e >= total) return;
     float acc = 0.0f;
-    for (int c = 0; c < chunks; ++c) acc += gpart[(size_t)c * total + e];
-    const float s = dl_sigmoid(raw[e] * inv_t);
-    graw[e] = acc * s * (1.0f - s) * inv_t;
+    for (int ch = 0; ch < chunks; ++ch) acc += gpart[(size_t)ch * total + e];
+    const int a = (int)(e % L);
+    const long long c = e / L;
+    const int n = (int)(c / O), d = (int)(c % O);
+    const float s = sig[e];
+    graw[((size_t)n * L + a) * O + d] = acc * s * (1.0f - s) * inv_t;
+}
+
+#define PROB_IS 64  // inputs per block of the gather
+#define PROB_WI 16  // inputs per wavefront
+__global__ __launch_bounds__(256) void prob_gather_t(const float *__restrict__ gmT, const int *__restrict__ inv_ptr,
+                                                      const int *__restrict__ inv_pos, float *__restrict__ gx, int B,
+                                                      int I, int N, int K, int O, int BT) {
+    __shared__ float tile[PROB_IS][65];  // [input][row]
+    int slab, t;
+    if (!dl_xcd_map((I + PROB_IS - 1) / PROB_IS, BT, slab, t)) return;
+    const int i0 = slab * PROB_IS;
+    const int lane = threadIdx.x & 63;
+    const int wave = dl_uniform(threadIdx.x >> 6);
+    const int iend = min(PROB_IS, I - i0);
+    const int wbeg = wave * PROB_WI;
+    const float *slabT = gmT + (size_t)t * N * O * K * 64 + lane;
+    for (int r = 0; r < PROB_WI; ++r) {
+        const int i = i0 + wbeg + r;
+        float acc = 0.0f;
+        if (i < I) {
+            const int e0 = inv_ptr[i], e1 = inv_ptr[i + 1];  // wave-uniform
+            for (int e = e0; e < e1; ++e) {
+                const int p = inv_pos[e];
+                if (O == 1) {
+                    acc += slabT[(size_t)p * 64];
+                } else {
+                    const int n = p / K, j = p - n * K;
+                    for (int d = 0; d < O; ++d) acc += slabT[(((size_t)n * O + d) * K + j) * 64];
+                }
+            }
+        }
+        tile[wbeg + r][lane] = acc;
+    }
+    __syncthreads();
+    if (iend == PROB_IS && (I & 3) == 0 && ((uintptr_t)gx & 15) == 0) {
+#pragma unroll
+        for (int pass = 0; pass < 4; ++pass) {
+            const int e = pass * 256 + threadIdx.x;
+            const int r = e / (PROB_IS / 4), i4 = (e % (PROB_IS / 4)) * 4;
+            const int b = t * 64 + r;
+            const prob_f4 v = {tile[i4][r], tile[i4 + 1][r], tile[i4 + 2][r], tile[i4 + 3][r]};
+            if (b < B) *reinterpret_cast<prob_f4 *>(&gx[(size_t)b * I + i0 + i4]) = v;
+        }
+    } else {
+        for (int e = threadIdx.x; e < 64 * PROB_IS; e += 256) {
+            const int r = e / PROB_IS, ii = e % PROB_IS;
+            const int b = t * 64 + r;
+            if (b < B && ii < iend) gx[(size_t)b * I + i0 + ii] = tile[ii][r];
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------------
@@ -264,43 +341,39 @@ __global__ __launch_bounds__(256) void prob_fill_zero(float *p, long long n) {
     if (i < n) p[i] = 0.0f;
 }
 
-// gather of the mapping adjoint: one block per batch row; the row of gm [N*k] is staged in LDS when it
-// fits (coalesced read), then every input sums its CSR entries from LDS in fixed order.
-__global__ __launch_bounds__(256) void prob_gather_bwd(const float *__restrict__ gm, const int *__restrict__ inv_ptr,
-                                                        const int *__restrict__ inv_pos, float *__restrict__ gx, int I,
-                                                        long long NK, int staged) {
-    extern __shared__ __align__(16) float grow[];
-    const int b = blockIdx.x;
-    const float *row = gm + (size_t)b * NK;
-    if (staged) {
-        for (long long p = threadIdx.x; p < NK; p += 256) grow[p] = row[p];
-        __syncthreads();
-    }
-    for (int i = threadIdx.x; i < I; i += 256) {
-        float acc = 0.0f;
-        for (int e = inv_ptr[i]; e < inv_ptr[i + 1]; ++e) acc += staged ? grow[inv_pos[e]] : row[inv_pos[e]];
-        gx[(size_t)b * I + i] = acc;
-    }
-}
-
 // ---------------------------------------------------------------------------------
 static int prob_check(int B, int I, int N, int k, int O) {
     if (B <= 0 || I <= 0 || N <= 0 || k <= 0 || O <= 0) return DL_ERR_SHAPE;
     if (k > DL_MAX_K) return DL_ERR_UNSUPPORTED;
     return DL_OK;
 }
-static inline bool prob_fast(int I, int k) { return k <= DL_MAX_FAST_K && (size_t)I * sizeof(float) <= 64 * 1024; }
-static inline float prob_inv_t(float t) { return 1.0f / (t > 1e-6f ? t : 1e-6f); }  // temperature.clamp(min=1e-6)
-static inline int prob_bwd_rows(int B) {  // rows per block: at most 64 partial buffers
-    int r = (B + 63) / 64;
-    return r < 16 ? 16 : r;
+// the tiled path addresses a batch tile of xT with 32-bit byte offsets (input * 256)
+static inline bool prob_fast(int I, int N, int k, int O) {
+    return k <= DL_MAX_FAST_K && I < (1 << 23) && (long long)N * O * k < (1 << 23);
 }
+static inline float prob_inv_t(float t) { return 1.0f / (t > 1e-6f ? t : 1e-6f); }  // temperature.clamp(min=1e-6)
+static inline int prob_bt(int B) { return (B + 63) / 64; }
+// batch tiles per wavefront of prob_bwd_t: enough (column, chunk) wavefronts to fill the chip
+static inline int prob_tiles_per_chunk(int B, int N, int O) {
+    const int BT = prob_bt(B);
+    int chunks = dl_ceil_div(8192, (long long)N * O);
+    if (chunks > BT) chunks = BT;
+    if (chunks < 1) chunks = 1;
+    return dl_ceil_div(BT, chunks);
+}
+static inline size_t prob_sig_bytes(int N, int k, int O) { return dl_align256((size_t)N * O * ((size_t)1 << k) * sizeof(float)); }
+static inline size_t prob_xT_bytes(int B, int I) { return dl_align256((size_t)prob_bt(B) * I * 64 * sizeof(float)); }
 
+extern "C" size_t dl_prob_fwd_workspace_bytes(int B, int I, int N, int k, int O) {
+    if (B <= 0 || I <= 0 || N <= 0 || k <= 0 || O <= 0 || !prob_fast(I, N, k, O)) return 256;
+    return prob_sig_bytes(N, k, O) + prob_xT_bytes(B, I);
+}
 extern "C" size_t dl_prob_bwd_workspace_bytes(int B, int I, int N, int k, int O) {
-    if (!prob_fast(I, k)) return 256;
-    const int chunks = dl_ceil_div(B, prob_bwd_rows(B));
-    return dl_align256((size_t)B * N * k * sizeof(float)) +
-           dl_align256((size_t)chunks * N * ((size_t)1 << k) * O * sizeof(float));
+    if (B <= 0 || I <= 0 || N <= 0 || k <= 0 || O <= 0 || !prob_fast(I, N, k, O)) return 256;
+    const size_t BT = prob_bt(B);
+    const int chunks = dl_ceil_div(prob_bt(B), prob_tiles_per_chunk(B, N, O));
+    return prob_sig_bytes(N, k, O) + prob_xT_bytes(B, I) + dl_align256(BT * N * O * 64 * sizeof(float)) +
+           dl_align256(BT * N * O * k * 64 * sizeof(float)) + dl_align256((size_t)chunks * N * O * ((size_t)1 << k) * sizeof(float));
 }
 
 #define PROB_DISPATCH(K, CALL) \
@@ -310,20 +383,25 @@ extern "C" size_t dl_prob_bwd_workspace_bytes(int B, int I, int N, int k, int O)
     }
 
 extern "C" int dl_prob_layer_fwd(const float *x, const int32_t *idx32, const float *raw_w, float temperature, float *y,
-                                 int B, int I, int N, int k, int O, void *stream) {
+                                 void *ws, size_t ws_bytes, int B, int I, int N, int k, int O, void *stream) {
     if (!x || !idx32 || !raw_w || !y) return DL_ERR_NULL;
     int rc = prob_check(B, I, N, k, O);
     if (rc) return rc;
     hipStream_t s = (hipStream_t)stream;
     const float inv_t = prob_inv_t(temperature);
-    if (!prob_fast(I, k)) {
+    if (!prob_fast(I, N, k, O)) {
         DL_TIMED("prob_generic_fwd", s, (prob_generic_fwd<<<dl_ceil_div((long long)B * N * O, 256), 256, 0, s>>>(x, idx32, raw_w, inv_t, y, B, I, N, k, O)));
         return dl_launch_status();
     }
-    dim3 grid(dl_ceil_div(N, PROB_NODES), dl_ceil_div(B, PROB_ROWS));
-    const size_t lds = (size_t)I * sizeof(float);
-#define CALL(KK) \
-    DL_TIMED("prob_fwd_kernel", s, (prob_fwd_kernel<KK><<<grid, PROB_NODES, lds, s>>>(x, idx32, raw_w, inv_t, y, B, I, N, O, PROB_ROWS)))
+    if (!ws) return DL_ERR_NULL;
+    if (ws_bytes < dl_prob_fwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
+    const int BT = prob_bt(B), L = 1 << k;
+    float *sig = (float *)ws;
+    float *xT = (float *)((char *)ws + prob_sig_bytes(N, k, O));
+    DL_TIMED("prob_sig_table", s, (prob_sig_table<<<dl_ceil_div((long long)N * L * O, 256), 256, 0, s>>>(raw_w, inv_t, sig, N, L, O)));
+    DL_TIMED("prob_to_tiles_x", s, (prob_to_tiles<<<dim3(dl_ceil_div(I, 64), BT), 256, 0, s>>>(x, xT, B, I)));
+    const int grid = dl_xcd_grid(dl_ceil_div((long long)N * O, PROB_TC), BT);
+#define CALL(KK) DL_TIMED("prob_fwd_t", s, (prob_fwd_t<KK><<<grid, 64 * PROB_FW, 0, s>>>(xT, idx32, sig, y, B, I, N, O, BT)))
     PROB_DISPATCH(k, CALL)
 #undef CALL
     return dl_launch_status();
@@ -339,7 +417,7 @@ extern "C" int dl_prob_layer_bwd(const float *x, const int32_t *idx32, const int
     hipStream_t s = (hipStream_t)stream;
     const float inv_t = prob_inv_t(temperature);
     const long long WT = (long long)N * ((long long)1 << k) * O;
-    if (!prob_fast(I, k)) {
+    if (!prob_fast(I, N, k, O)) {
         DL_TIMED("prob_fill_zero", s, (prob_fill_zero<<<dl_ceil_div(WT, 256), 256, 0, s>>>(graw, WT)));
         if (gx) prob_fill_zero<<<dl_ceil_div((long long)B * I, 256), 256, 0, s>>>(gx, (long long)B * I);
         DL_TIMED("prob_generic_bwd", s, (prob_generic_bwd<<<dl_ceil_div((long long)B * N, 256), 256, 0, s>>>(x, idx32, raw_w, inv_t, gy, gx, graw, B, I, N,
@@ -348,25 +426,30 @@ extern "C" int dl_prob_layer_bwd(const float *x, const int32_t *idx32, const int
     }
     if (!ws) return DL_ERR_NULL;
     if (ws_bytes < dl_prob_bwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
-    const int rows = prob_bwd_rows(B);
-    const int chunks = dl_ceil_div(B, rows);
-    float *gm = (float *)ws;
-    float *gpart = (float *)((char *)ws + dl_align256((size_t)B * N * k * sizeof(float)));
-    dim3 grid(dl_ceil_div(N, PROB_NODES), chunks);
-    const size_t lds = (size_t)I * sizeof(float);
-#define CALL(KK)                                                                                                     \
-    DL_TIMED("prob_bwd_kernel", s,                                                                                   \
-             (prob_bwd_kernel<KK><<<grid, PROB_NODES, lds, s>>>(x, idx32, raw_w, inv_t, gy, gm, gpart, B, I, N, O, rows, \
-                                                                gx != nullptr)))
+    const int BT = prob_bt(B), L = 1 << k, NO = N * O;
+    const int tpc = prob_tiles_per_chunk(B, N, O);
+    const int chunks = dl_ceil_div(BT, tpc);
+    char *w = (char *)ws;
+    float *sig = (float *)w; w += prob_sig_bytes(N, k, O);
+    float *xT = (float *)w; w += prob_xT_bytes(B, I);
+    float *gyT = (float *)w; w += dl_align256((size_t)BT * NO * 64 * sizeof(float));
+    float *gmT = (float *)w; w += dl_align256((size_t)BT * NO * k * 64 * sizeof(float));
+    float *gpart = (float *)w;
+    DL_TIMED("prob_sig_table", s, (prob_sig_table<<<dl_ceil_div(WT, 256), 256, 0, s>>>(raw_w, inv_t, sig, N, L, O)));
+    DL_TIMED("prob_to_tiles_x", s, (prob_to_tiles<<<dim3(dl_ceil_div(I, 64), BT), 256, 0, s>>>(x, xT, B, I)));
+    DL_TIMED("prob_to_tiles_gy", s, (prob_to_tiles<<<dim3(dl_ceil_div(NO, 64), BT), 256, 0, s>>>(gy, gyT, B, NO)));
+#define CALL(KK)                                                                                                    \
+    DL_TIMED("prob_bwd_t", s,                                                                                       \
+             (prob_bwd_t<KK><<<dim3(dl_ceil_div(NO, 4), chunks), 256, 0, s>>>(xT, gyT, idx32, sig, gmT, gpart, I, N, O, BT, \
+                                                                           tpc, gx != nullptr)))
     PROB_DISPATCH(k, CALL)
 #undef CALL
     DL_TIMED("prob_reduce_weights", s,
-             (prob_reduce_weights<<<dl_ceil_div(WT, 256), 256, 0, s>>>(gpart, raw_w, inv_t, graw, WT, chunks)));
-    const int staged = (size_t)N * k * sizeof(float) <= 64 * 1024;
-    const size_t gbytes = staged ? (size_t)N * k * sizeof(float) : 0;
+             (prob_reduce_weights<<<dl_ceil_div(WT, 256), 256, 0, s>>>(gpart, sig, inv_t, graw, N, L, O, chunks)));
     if (gx)
-        DL_TIMED("prob_gather_bwd", s,
-                 (prob_gather_bwd<<<B, 256, gbytes, s>>>(gm, inv_ptr, inv_pos, gx, I, (long long)N * k, staged)));
+        DL_TIMED("prob_gather_t", s,
+                 (prob_gather_t<<<dl_xcd_grid(dl_ceil_div(I, PROB_IS), BT), 256, 0, s>>>(gmT, inv_ptr, inv_pos, gx, B, I, N, k, O,
+                                                                                       BT)));
     return dl_launch_status();
 }
 

@@ -159,8 +159,9 @@ class ProbLayerFunction(torch.autograd.Function):
                                f"[{plan.N},{k}] over {plan.I} inputs")
         y = torch.empty((B, N * O), dtype=torch.float32, device=x.device)
         dims = (B, I, N, k, O)
+        ws = _bytes(nat.lib().dl_prob_fwd_workspace_bytes(*dims), x.device)
         nat.check(nat.lib().dl_prob_layer_fwd(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(raw), float(temperature),
-                                              nat.ptr(y), *dims, nat.stream()))
+                                              nat.ptr(y), nat.ptr(ws), ws.numel(), *dims, nat.stream()))
         ctx.save_for_backward(x, raw)
         ctx.plan, ctx.T, ctx.dims = plan, float(temperature), dims
         return y

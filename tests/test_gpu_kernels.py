@@ -153,7 +153,8 @@ def test_gather_forward_backward(dtype):
 
 # ------------------------------------------------------------------------------ probabilistic
 PROB_SHAPES = [(32, 40, 24, 4, 2), (64, 128, 300, 4, 1), (17, 30, 9, 6, 1), (20, 9, 5, 1, 1), (10, 50, 7, 2, 3),
-               (6, 40, 5, 7, 2)]
+               (6, 40, 5, 7, 2), (200, 300, 260, 4, 1), (130, 70, 33, 5, 2), (65, 1000, 515, 3, 1),
+               (300, 20, 3, 4, 1)]   # last: few nodes, many batch tiles -> several table-gradient chunks
 
 
 @pytest.mark.parametrize("shape", PROB_SHAPES)
@@ -303,7 +304,7 @@ def test_argument_errors_are_reported_not_launched():
     assert lib.dl_dwn_layer_fwd(p, p, p, p, p, p, 0, 4, 4, 4, 2, 1, None) == -4   # workspace too small
     assert lib.dl_dwn_layer_fwd(p, p, p, p, p, p, 1 << 20, 4, 4, 4, 17, 1, None) == -3  # k beyond DL_MAX_K
     assert lib.dl_gather_fwd(p, p, 8, p, 1, 1, 1, 1, None) == -3
-    assert lib.dl_prob_layer_fwd(p, p, p, 1.0, p, 0, 1, 1, 1, 1, None) == -2
+    assert lib.dl_prob_layer_fwd(p, p, p, 1.0, p, p, 256, 0, 1, 1, 1, 1, None) == -2
     with pytest.raises(RuntimeError, match="ROCm devices only"):
         _ops().DWNLayerFunction.apply(torch.zeros(2, 2), torch.zeros(1, 1, 4), None, 0.1, 0.1)
     with pytest.raises(IndexError):
