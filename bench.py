@@ -98,11 +98,12 @@ def run_secondary(args):
         gy = torch.randn(B, N * O, device=dev)
         y = torch.empty(B, N * O, device=dev); gx = torch.empty(B, I, device=dev); graw = torch.empty_like(raw)
         ws = torch.empty(max(lib.dl_prob_bwd_workspace_bytes(*dims), 256), dtype=torch.uint8, device=dev)
+        saved = torch.empty(max(lib.dl_prob_saved_bytes(*dims), 256), dtype=torch.uint8, device=dev)
 
         def step():
             nat.check(lib.dl_prob_layer_fwd(x.data_ptr(), plan.idx32.data_ptr(), raw.data_ptr(), 1.0, y.data_ptr(),
-                                            ws.data_ptr(), ws.numel(), *dims, stream))
-            nat.check(lib.dl_prob_layer_bwd(x.data_ptr(), plan.idx32.data_ptr(), plan.inv_ptr.data_ptr(),
+                                            saved.data_ptr(), saved.numel(), *dims, stream))
+            nat.check(lib.dl_prob_layer_bwd(x.data_ptr(), saved.data_ptr(), plan.idx32.data_ptr(), plan.inv_ptr.data_ptr(),
                                             plan.inv_pos.data_ptr(), raw.data_ptr(), 1.0, gy.data_ptr(), gx.data_ptr(),
                                             graw.data_ptr(), ws.data_ptr(), ws.numel(), *dims, stream))
 

@@ -28,10 +28,10 @@ SIGNATURES = {
     "dl_dwn_layer_fwd": (_I, [_P, _P, _P, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
     "dl_dwn_layer_bwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _F, _F, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
     "dl_dwn_layer_eval": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
-    "dl_prob_fwd_workspace_bytes": (_Z, [_I] * 5),
+    "dl_prob_saved_bytes": (_Z, [_I] * 5),
     "dl_prob_bwd_workspace_bytes": (_Z, [_I] * 5),
     "dl_prob_layer_fwd": (_I, [_P, _P, _P, _F, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
-    "dl_prob_layer_bwd": (_I, [_P, _P, _P, _P, _P, _F, _P, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
+    "dl_prob_layer_bwd": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
     "dl_prob_layer_eval": (_I, [_P, _P, _P, _F, _P, _I, _I, _I, _I, _I, _P]),
     "dl_soft_map_workspace_bytes": (_Z, [_I] * 4),
     "dl_soft_map_fwd": (_I, [_P, _P, _F, _P, _P, _P, _Z, _I, _I, _I, _I, _P]),

@@ -19,7 +19,7 @@ def forward(input, raw_weights, temperature):
     y = torch.empty((B, O), dtype=torch.float32, device=input.device)
     plan = _plan(k, input.device)
     lib = nat.lib()
-    ws = torch.empty(max(lib.dl_prob_fwd_workspace_bytes(B, k, 1, k, O), 256), dtype=torch.uint8, device=input.device)
+    ws = torch.empty(max(lib.dl_prob_saved_bytes(B, k, 1, k, O), 256), dtype=torch.uint8, device=input.device)
     nat.check(lib.dl_prob_layer_fwd(input.data_ptr(), plan.idx32.data_ptr(), raw_weights.data_ptr(),
                                     float(temperature), y.data_ptr(), ws.data_ptr(), ws.numel(), B, k, 1, k, O,
                                     nat.stream()))
@@ -35,7 +35,7 @@ def backward(input, raw_weights, temperature, grad_output):
     gx = torch.empty_like(input)
     gw = torch.empty_like(raw_weights)
     ws = torch.empty(max(lib.dl_prob_bwd_workspace_bytes(B, k, 1, k, O), 256), dtype=torch.uint8, device=input.device)
-    nat.check(lib.dl_prob_layer_bwd(input.data_ptr(), plan.idx32.data_ptr(), plan.inv_ptr.data_ptr(),
+    nat.check(lib.dl_prob_layer_bwd(input.data_ptr(), None, plan.idx32.data_ptr(), plan.inv_ptr.data_ptr(),
                                     plan.inv_pos.data_ptr(), raw_weights.data_ptr(), float(temperature),
                                     grad_output.data_ptr(), gx.data_ptr(), gw.data_ptr(), ws.data_ptr(), ws.numel(),
                                     B, k, 1, k, O, nat.stream()))

@@ -43,15 +43,30 @@ __global__ __launch_bounds__(256) void prob_sig_table(const float *__restrict__ 
 __global__ __launch_bounds__(256) void prob_to_tiles(const float *__restrict__ src, float *__restrict__ dst, int B, int C) {
     __shared__ float tile[64][65];  // [column][row]
     const int t = blockIdx.y, c0 = blockIdx.x * 64;
-    for (int e = threadIdx.x; e < 4096; e += 256) {
-        const int r = e >> 6, c = e & 63;
-        const int b = t * 64 + r;
-        tile[c][r] = (b < B && c0 + c < C) ? src[(size_t)b * C + c0 + c] : 0.0f;
+    if ((C & 3) == 0 && c0 + 64 <= C && (((uintptr_t)src) & 15) == 0) {
+#pragma unroll
+        for (int pass = 0; pass < 4; ++pass) {
+            const int e = pass * 256 + threadIdx.x;
+            const int r = e >> 4, c = (e & 15) * 4;
+            const int b = t * 64 + r;
+            prob_f4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (b < B) v = *reinterpret_cast<const prob_f4 *>(src + (size_t)b * C + c0 + c);
+            tile[c][r] = v.x; tile[c + 1][r] = v.y; tile[c + 2][r] = v.z; tile[c + 3][r] = v.w;
+        }
+    } else {
+        for (int e = threadIdx.x; e < 4096; e += 256) {
+            const int r = e >> 6, c = e & 63;
+            const int b = t * 64 + r;
+            tile[c][r] = (b < B && c0 + c < C) ? src[(size_t)b * C + c0 + c] : 0.0f;
+        }
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < 4096; e += 256) {
-        const int c = e >> 6, r = e & 63;
-        if (c0 + c < C) dst[((size_t)t * C + c0 + c) * 64 + r] = tile[c][r];
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        const int e = pass * 256 + threadIdx.x;
+        const int c = e >> 4, r = (e & 15) * 4;
+        const prob_f4 v = {tile[c][r], tile[c][r + 1], tile[c][r + 2], tile[c][r + 3]};
+        if (c0 + c < C) *reinterpret_cast<prob_f4 *>(dst + ((size_t)t * C + c0 + c) * 64 + r) = v;
     }
 }
 
@@ -218,6 +233,11 @@ __global__ __launch_bounds__(256) void prob_reduce_weights(const float *__restri
 
 #define PROB_IS 64  // inputs per block of the gather
 #define PROB_WI 16  // inputs per wavefront
+#define PROB_EG 8   // entries requested together
+// FAST (one output per node): the CSR entries of a wavefront's 16 inputs are held one per lane
+// (row offset, local input) and replayed eight at a time with buffer loads whose offset travels
+// in an SGPR, the next eight requested before the current ones are summed.
+template <bool FAST>
 __global__ __launch_bounds__(256) void prob_gather_t(const float *__restrict__ gmT, const int *__restrict__ inv_ptr,
                                                       const int *__restrict__ inv_pos, float *__restrict__ gx, int B,
                                                       int I, int N, int K, int O, int BT) {
@@ -229,23 +249,82 @@ __global__ __launch_bounds__(256) void prob_gather_t(const float *__restrict__ g
     const int wave = dl_uniform(threadIdx.x >> 6);
     const int iend = min(PROB_IS, I - i0);
     const int wbeg = wave * PROB_WI;
-    const float *slabT = gmT + (size_t)t * N * O * K * 64 + lane;
-    for (int r = 0; r < PROB_WI; ++r) {
-        const int i = i0 + wbeg + r;
+    if (FAST) {
+        const __amdgpu_buffer_rsrc_t rs =
+            __builtin_amdgcn_make_buffer_rsrc((void *)(gmT + (size_t)t * N * K * 64), 0, N * K * 256, PROB_RSRC);
+        const int lane4 = lane * 4;
+        const int myptr = inv_ptr[min(i0 + wbeg + min(lane, PROB_WI), I)];
+#pragma unroll
+        for (int r = 0; r < PROB_WI; ++r) tile[wbeg + r][lane] = 0.0f;  // inputs nobody reads keep 0
+        const int ebeg = __builtin_amdgcn_readlane(myptr, 0);
+        const int eend = __builtin_amdgcn_readlane(myptr, PROB_WI);
         float acc = 0.0f;
-        if (i < I) {
-            const int e0 = inv_ptr[i], e1 = inv_ptr[i + 1];  // wave-uniform
-            for (int e = e0; e < e1; ++e) {
-                const int p = inv_pos[e];
-                if (O == 1) {
-                    acc += slabT[(size_t)p * 64];
-                } else {
+        int cur = -1;
+        for (int base = ebeg; base < eend; base += 64) {
+            const int e = base + lane;
+            const bool valid = e < eend;
+            const int p = valid ? inv_pos[e] : 0;
+            int ii = 0;  // local input of entry e
+#pragma unroll
+            for (int l = 1; l <= PROB_WI; ++l) ii += (__builtin_amdgcn_readlane(myptr, l) <= e) ? 1 : 0;
+            const int rec = valid ? ((p << 8) | ii) : 0;  // row offset p * 256 in the upper bits
+            const int cnt = min(64, eend - base);
+            struct Group { int r[PROB_EG]; float g[PROB_EG]; };
+            auto request = [&](int s0, Group &G) {
+#pragma unroll
+                for (int q = 0; q < PROB_EG; ++q) {
+                    const int r = __builtin_amdgcn_readlane(rec, s0 + q);
+                    G.r[q] = r;
+                    G.g[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, lane4, r & ~255, 0));
+                }
+            };
+            auto sum_up = [&](const Group &G, int s0) {
+#pragma unroll
+                for (int q = 0; q < PROB_EG; ++q) {
+                    if (s0 + q >= cnt) break;  // wave-uniform
+                    const int ri = G.r[q] & 31;
+                    if (ri != cur) {
+                        if (cur >= 0) tile[wbeg + cur][lane] = acc;
+                        acc = 0.0f;
+                        cur = ri;
+                    }
+                    acc += G.g[q];
+                }
+            };
+            const int m = (cnt + PROB_EG - 1) / PROB_EG;
+            Group A, Bq;
+            request(0, A);
+            int gi = 0;
+            for (; gi + 2 < m; gi += 2) {
+                request((gi + 1) * PROB_EG, Bq);
+                sum_up(A, gi * PROB_EG);
+                request((gi + 2) * PROB_EG, A);
+                sum_up(Bq, (gi + 1) * PROB_EG);
+            }
+            if (gi + 1 < m) {
+                request((gi + 1) * PROB_EG, Bq);
+                sum_up(A, gi * PROB_EG);
+                sum_up(Bq, (gi + 1) * PROB_EG);
+            } else {
+                sum_up(A, gi * PROB_EG);
+            }
+        }
+        if (cur >= 0) tile[wbeg + cur][lane] = acc;
+    } else {
+        const float *slabT = gmT + (size_t)t * N * O * K * 64 + lane;
+        for (int r = 0; r < PROB_WI; ++r) {
+            const int i = i0 + wbeg + r;
+            float acc = 0.0f;
+            if (i < I) {
+                const int e0 = inv_ptr[i], e1 = inv_ptr[i + 1];  // wave-uniform
+                for (int e = e0; e < e1; ++e) {
+                    const int p = inv_pos[e];
                     const int n = p / K, j = p - n * K;
                     for (int d = 0; d < O; ++d) acc += slabT[(((size_t)n * O + d) * K + j) * 64];
                 }
             }
+            tile[wbeg + r][lane] = acc;
         }
-        tile[wbeg + r][lane] = acc;
     }
     __syncthreads();
     if (iend == PROB_IS && (I & 3) == 0 && ((uintptr_t)gx & 15) == 0) {
@@ -364,7 +443,8 @@ static inline int prob_tiles_per_chunk(int B, int N, int O) {
 static inline size_t prob_sig_bytes(int N, int k, int O) { return dl_align256((size_t)N * O * ((size_t)1 << k) * sizeof(float)); }
 static inline size_t prob_xT_bytes(int B, int I) { return dl_align256((size_t)prob_bt(B) * I * 64 * sizeof(float)); }
 
-extern "C" size_t dl_prob_fwd_workspace_bytes(int B, int I, int N, int k, int O) {
+// what the forward leaves for the backward: the sigmoid table and the re-tiled input
+extern "C" size_t dl_prob_saved_bytes(int B, int I, int N, int k, int O) {
     if (B <= 0 || I <= 0 || N <= 0 || k <= 0 || O <= 0 || !prob_fast(I, N, k, O)) return 256;
     return prob_sig_bytes(N, k, O) + prob_xT_bytes(B, I);
 }
@@ -383,7 +463,7 @@ extern "C" size_t dl_prob_bwd_workspace_bytes(int B, int I, int N, int k, int O)
     }
 
 extern "C" int dl_prob_layer_fwd(const float *x, const int32_t *idx32, const float *raw_w, float temperature, float *y,
-                                 void *ws, size_t ws_bytes, int B, int I, int N, int k, int O, void *stream) {
+                                 void *saved, size_t saved_bytes, int B, int I, int N, int k, int O, void *stream) {
     if (!x || !idx32 || !raw_w || !y) return DL_ERR_NULL;
     int rc = prob_check(B, I, N, k, O);
     if (rc) return rc;
@@ -393,11 +473,11 @@ extern "C" int dl_prob_layer_fwd(const float *x, const int32_t *idx32, const flo
         DL_TIMED("prob_generic_fwd", s, (prob_generic_fwd<<<dl_ceil_div((long long)B * N * O, 256), 256, 0, s>>>(x, idx32, raw_w, inv_t, y, B, I, N, k, O)));
         return dl_launch_status();
     }
-    if (!ws) return DL_ERR_NULL;
-    if (ws_bytes < dl_prob_fwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
+    if (!saved) return DL_ERR_NULL;
+    if (saved_bytes < dl_prob_saved_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
     const int BT = prob_bt(B), L = 1 << k;
-    float *sig = (float *)ws;
-    float *xT = (float *)((char *)ws + prob_sig_bytes(N, k, O));
+    float *sig = (float *)saved;
+    float *xT = (float *)((char *)saved + prob_sig_bytes(N, k, O));
     DL_TIMED("prob_sig_table", s, (prob_sig_table<<<dl_ceil_div((long long)N * L * O, 256), 256, 0, s>>>(raw_w, inv_t, sig, N, L, O)));
     DL_TIMED("prob_to_tiles_x", s, (prob_to_tiles<<<dim3(dl_ceil_div(I, 64), BT), 256, 0, s>>>(x, xT, B, I)));
     const int grid = dl_xcd_grid(dl_ceil_div((long long)N * O, PROB_TC), BT);
@@ -407,7 +487,8 @@ extern "C" int dl_prob_layer_fwd(const float *x, const int32_t *idx32, const flo
     return dl_launch_status();
 }
 
-extern "C" int dl_prob_layer_bwd(const float *x, const int32_t *idx32, const int32_t *inv_ptr, const int32_t *inv_pos,
+extern "C" int dl_prob_layer_bwd(const float *x, const void *saved, const int32_t *idx32, const int32_t *inv_ptr,
+                                 const int32_t *inv_pos,
                                  const float *raw_w, float temperature, const float *gy, float *gx, float *graw,
                                  void *ws, size_t ws_bytes, int B, int I, int N, int k, int O, void *stream) {
     if (!x || !idx32 || !raw_w || !gy || !graw) return DL_ERR_NULL;
@@ -435,8 +516,13 @@ extern "C" int dl_prob_layer_bwd(const float *x, const int32_t *idx32, const int
     float *gyT = (float *)w; w += dl_align256((size_t)BT * NO * 64 * sizeof(float));
     float *gmT = (float *)w; w += dl_align256((size_t)BT * NO * k * 64 * sizeof(float));
     float *gpart = (float *)w;
-    DL_TIMED("prob_sig_table", s, (prob_sig_table<<<dl_ceil_div(WT, 256), 256, 0, s>>>(raw_w, inv_t, sig, N, L, O)));
-    DL_TIMED("prob_to_tiles_x", s, (prob_to_tiles<<<dim3(dl_ceil_div(I, 64), BT), 256, 0, s>>>(x, xT, B, I)));
+    if (saved) {  // what the forward of the same x, raw_w and temperature left
+        sig = (float *)saved;
+        xT = (float *)((char *)saved + prob_sig_bytes(N, k, O));
+    } else {
+        DL_TIMED("prob_sig_table", s, (prob_sig_table<<<dl_ceil_div(WT, 256), 256, 0, s>>>(raw_w, inv_t, sig, N, L, O)));
+        DL_TIMED("prob_to_tiles_x", s, (prob_to_tiles<<<dim3(dl_ceil_div(I, 64), BT), 256, 0, s>>>(x, xT, B, I)));
+    }
     DL_TIMED("prob_to_tiles_gy", s, (prob_to_tiles<<<dim3(dl_ceil_div(NO, 64), BT), 256, 0, s>>>(gy, gyT, B, NO)));
 #define CALL(KK)                                                                                                    \
     DL_TIMED("prob_bwd_t", s,                                                                                       \
@@ -446,10 +532,14 @@ extern "C" int dl_prob_layer_bwd(const float *x, const int32_t *idx32, const int
 #undef CALL
     DL_TIMED("prob_reduce_weights", s,
              (prob_reduce_weights<<<dl_ceil_div(WT, 256), 256, 0, s>>>(gpart, sig, inv_t, graw, N, L, O, chunks)));
-    if (gx)
+    if (gx && O == 1)
         DL_TIMED("prob_gather_t", s,
-                 (prob_gather_t<<<dl_xcd_grid(dl_ceil_div(I, PROB_IS), BT), 256, 0, s>>>(gmT, inv_ptr, inv_pos, gx, B, I, N, k, O,
-                                                                                       BT)));
+                 (prob_gather_t<true><<<dl_xcd_grid(dl_ceil_div(I, PROB_IS), BT), 256, 0, s>>>(gmT, inv_ptr, inv_pos, gx, B, I,
+                                                                                             N, k, O, BT)));
+    else if (gx)
+        DL_TIMED("prob_gather_t", s,
+                 (prob_gather_t<false><<<dl_xcd_grid(dl_ceil_div(I, PROB_IS), BT), 256, 0, s>>>(gmT, inv_ptr, inv_pos, gx, B, I,
+                                                                                              N, k, O, BT)));
     return dl_launch_status();
 }
 

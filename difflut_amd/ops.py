@@ -159,16 +159,16 @@ class ProbLayerFunction(torch.autograd.Function):
                                f"[{plan.N},{k}] over {plan.I} inputs")
         y = torch.empty((B, N * O), dtype=torch.float32, device=x.device)
         dims = (B, I, N, k, O)
-        ws = _bytes(nat.lib().dl_prob_fwd_workspace_bytes(*dims), x.device)
+        saved = _bytes(nat.lib().dl_prob_saved_bytes(*dims), x.device)
         nat.check(nat.lib().dl_prob_layer_fwd(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(raw), float(temperature),
-                                              nat.ptr(y), nat.ptr(ws), ws.numel(), *dims, nat.stream()))
-        ctx.save_for_backward(x, raw)
+                                              nat.ptr(y), nat.ptr(saved), saved.numel(), *dims, nat.stream()))
+        ctx.save_for_backward(x, raw, saved)
         ctx.plan, ctx.T, ctx.dims = plan, float(temperature), dims
         return y
 
     @staticmethod
     def backward(ctx, gy):
-        x, raw = ctx.saved_tensors
+        x, raw, saved = ctx.saved_tensors
         plan = ctx.plan
         gy = _f32(gy)
         lib = nat.lib()
@@ -176,7 +176,8 @@ class ProbLayerFunction(torch.autograd.Function):
         gx = torch.empty((B, I), dtype=torch.float32, device=gy.device) if ctx.needs_input_grad[0] else None
         graw = torch.empty_like(raw)
         ws = _bytes(lib.dl_prob_bwd_workspace_bytes(*ctx.dims), gy.device)
-        nat.check(lib.dl_prob_layer_bwd(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(plan.inv_ptr), nat.ptr(plan.inv_pos),
+        nat.check(lib.dl_prob_layer_bwd(nat.ptr(x), nat.ptr(saved), nat.ptr(plan.idx32), nat.ptr(plan.inv_ptr),
+                                        nat.ptr(plan.inv_pos),
                                         nat.ptr(raw), ctx.T, nat.ptr(gy), nat.ptr(gx), nat.ptr(graw), nat.ptr(ws),
                                         ws.numel(), *ctx.dims, nat.stream()))
         return gx, graw, None, None

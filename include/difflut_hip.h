@@ -104,15 +104,17 @@ int dl_dwn_layer_eval(const float *x, const int32_t *idx32, const float *luts, f
  *   x_j = x[b, idx[n,j]] used as given (no clamping: inputs are probabilities).
  * Backward is the exact derivative of that expression (what autograd gives the
  * reference's CPU path): gx [B,I] (nullable), graw [N,L,O]; both overwritten.
- * Both directions re-tile their [batch, feature] operands into the workspace
- * (lanes = batch rows inside the kernels); nothing is kept between the calls.
+ * Both directions re-tile their [batch, feature] operands (lanes = batch rows inside
+ * the kernels).
  * ------------------------------------------------------------------------ */
-size_t dl_prob_fwd_workspace_bytes(int B, int I, int N, int k, int O);
+size_t dl_prob_saved_bytes(int B, int I, int N, int k, int O);
 size_t dl_prob_bwd_workspace_bytes(int B, int I, int N, int k, int O);
+/* `saved` (dl_prob_saved_bytes) receives the sigmoid table and the re-tiled input. */
 int dl_prob_layer_fwd(const float *x, const int32_t *idx32, const float *raw_w, float temperature,
-                      float *y, void *ws, size_t ws_bytes,
+                      float *y, void *saved, size_t saved_bytes,
                       int B, int I, int N, int k, int O, void *stream);
-int dl_prob_layer_bwd(const float *x, const int32_t *idx32,
+/* `saved` may be null: then both are rebuilt from x, raw_w and temperature. */
+int dl_prob_layer_bwd(const float *x, const void *saved, const int32_t *idx32,
                       const int32_t *inv_ptr, const int32_t *inv_pos,
                       const float *raw_w, float temperature, const float *gy,
                       float *gx, float *graw, void *ws, size_t ws_bytes,
