@@ -97,29 +97,47 @@ __global__ __launch_bounds__(64 * PROB_FW) void prob_fwd_t(const float *__restri
     const int wbeg = wave * PROB_WC;
     const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc((void *)(xT + (size_t)t * I * 64), 0, I * 256, PROB_RSRC);
     const int lane4 = lane * 4;
-    for (int q = 0; q < PROB_WC; ++q) {
-        const int cc = wbeg + q;
-        if (cc >= cend) break;  // wave-uniform
-        const int c = c0 + cc;
-        const int n = c / O;
-        float xs[K];
+    // slot s = (column within my 16) * K + j  ->  lane s % 64 of register s / 64: byte offset of the input's row
+    constexpr int NIDX = (PROB_WC * K + 63) / 64;
+    int myoff[NIDX];
 #pragma unroll
-        for (int j = 0; j < K; ++j)
-            xs[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_x, lane4, idx32[(size_t)n * K + j] * 256, 0));
-        float tab[L];
-        prob_load_table<K>(sig, c, tab);
-        float v[L / 2 > 0 ? L / 2 : 1];
-        {
-            const float om = 1.0f - xs[0];
+    for (int v = 0; v < NIDX; ++v) {
+        const int s = v * 64 + lane;
+        const int c = min(c0 + wbeg + min(s / K, PROB_WC - 1), NO - 1);
+        myoff[v] = idx32[(size_t)(c / O) * K + s % K] * 256;
+    }
+    constexpr int CG = 4;  // columns whose input rows are requested together
 #pragma unroll
-            for (int a = 0; a < L / 2; ++a) v[a] = fmaf(tab[2 * a + 1], xs[0], tab[2 * a] * om);
+    for (int g = 0; g < PROB_WC; g += CG) {
+        if (wbeg + g >= cend) break;  // wave-uniform
+        float xs[CG][K];
+#pragma unroll
+        for (int q = 0; q < CG; ++q)
+#pragma unroll
+            for (int j = 0; j < K; ++j) {
+                const int s = (g + q) * K + j;  // compile-time after unrolling
+                const int off = __builtin_amdgcn_readlane(myoff[s / 64], s % 64);
+                xs[q][j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_x, lane4, off, 0));
+            }
+#pragma unroll
+        for (int q = 0; q < CG; ++q) {
+            const int cc = wbeg + g + q;
+            if (cc >= cend) break;  // wave-uniform
+            float tab[L];
+            prob_load_table<K>(sig, c0 + cc, tab);
+            float v[L / 2 > 0 ? L / 2 : 1];
+            {
+                const float om = 1.0f - xs[q][0];
+#pragma unroll
+                for (int a = 0; a < L / 2; ++a) v[a] = fmaf(tab[2 * a + 1], xs[q][0], tab[2 * a] * om);
+            }
+#pragma unroll
+            for (int j = 1; j < K; ++j) {
+#pragma unroll
+                for (int a = 0; a < (L >> (j + 1)); ++a) v[a] = v[2 * a] + xs[q][j] * (v[2 * a + 1] - v[2 * a]);
+            }
+            tile[cc][lane] = v[0];
         }
-#pragma unroll
-        for (int j = 1; j < K; ++j) {
-#pragma unroll
-            for (int a = 0; a < (L >> (j + 1)); ++a) v[a] = v[2 * a] + xs[j] * (v[2 * a + 1] - v[2 * a]);
-        }
-        tile[cc][lane] = v[0];
     }
     __syncthreads();
     for (int e = threadIdx.x; e < 64 * PROB_TC; e += 64 * PROB_FW) {
@@ -152,12 +170,20 @@ __global__ __launch_bounds__(256) void prob_bwd_t(const float *__restrict__ xT, 
 #pragma unroll
     for (int a = 0; a < L; ++a) acc[a] = 0.0f;
     const int t0 = chunk * tiles_per_chunk, t1 = min(BT, t0 + tiles_per_chunk);
-    for (int t = t0; t < t1; ++t) {
+    float nxs[K], ng = 0.0f;  // operands of the next batch tile, requested one tile ahead
+    auto request = [&](int t) {
         const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc((void *)(xT + (size_t)t * I * 64), 0, I * 256, PROB_RSRC);
+#pragma unroll
+        for (int j = 0; j < K; ++j) nxs[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_x, lane4, off[j], 0));
+        ng = gyT[((size_t)t * NO + c) * 64 + lane];
+    };
+    if (t0 < t1) request(t0);
+    for (int t = t0; t < t1; ++t) {
         float xs[K];
 #pragma unroll
-        for (int j = 0; j < K; ++j) xs[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_x, lane4, off[j], 0));
-        const float g = gyT[((size_t)t * NO + c) * 64 + lane];
+        for (int j = 0; j < K; ++j) xs[j] = nxs[j];
+        const float g = ng;
+        if (t + 1 < t1) request(t + 1);
         // forward fold, keeping the differences d_j[a] = lvl_j[2a+1] - lvl_j[2a] of every level
         float diff[L > 1 ? L - 1 : 1];  // level j occupies [L - (L >> j), L - (L >> (j+1)))
         float v[L / 2 > 0 ? L / 2 : 1];
@@ -203,16 +229,28 @@ __global__ __launch_bounds__(256) void prob_bwd_t(const float *__restrict__ xT, 
             for (int j = 0; j < K; ++j) gmT[(((size_t)t * NO + c) * K + j) * 64 + lane] = g * dx[j];
         }
     }
-    // sum the 64 per-row partials of every table entry, lane a keeps entry a
-    float mine = 0.0f;
+    // Sum the 64 per-row partials of every table entry with L - 1 + (6 - K) exchanges instead of 6 L:
+    // round r pairs the entries (2i, 2i+1); the half of the wavefront with lane bit (5 - r) set keeps
+    // the odd one and hands over the even one, so after K rounds a lane holds one entry,
+    // a = sum_r ((lane >> (5 - r)) & 1) << r, summed over the lanes that differ in the top K bits.
 #pragma unroll
-    for (int a = 0; a < L; ++a) {
-        float r = acc[a];
+    for (int r = 0; r < K; ++r) {
+        const int width = 32 >> r;
+        const bool upper = (lane & width) != 0;
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) r += __shfl_xor(r, o);
-        if (lane == a) mine = r;
+        for (int i = 0; i < (L >> (r + 1)); ++i) {
+            const float keep = upper ? acc[2 * i + 1] : acc[2 * i];
+            const float send = upper ? acc[2 * i] : acc[2 * i + 1];
+            acc[i] = keep + __shfl_xor(send, width);
+        }
     }
-    if (lane < L) gpart[((size_t)chunk * NO + c) * L + lane] = mine;
+    float mine = acc[0];
+#pragma unroll
+    for (int width = 32 >> K; width > 0; width >>= 1) mine += __shfl_xor(mine, width);
+    int a = 0;
+#pragma unroll
+    for (int r = 0; r < K; ++r) a |= ((lane >> (5 - r)) & 1) << r;
+    if ((lane & ((64 >> K) - 1)) == 0) gpart[((size_t)chunk * NO + c) * L + a] = mine;
 }
 
 // graw[n,a,d] = sigmoid'(w/T)/T * sum over chunks of gpart[chunk][c][a]
@@ -435,7 +473,7 @@ static inline int prob_bt(int B) { return (B + 63) / 64; }
 // batch tiles per wavefront of prob_bwd_t: enough (column, chunk) wavefronts to fill the chip
 static inline int prob_tiles_per_chunk(int B, int N, int O) {
     const int BT = prob_bt(B);
-    int chunks = dl_ceil_div(8192, (long long)N * O);
+    int chunks = dl_ceil_div(4096, (long long)N * O);
     if (chunks > BT) chunks = BT;
     if (chunks < 1) chunks = 1;
     return dl_ceil_div(BT, chunks);
