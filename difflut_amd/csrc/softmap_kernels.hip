@@ -188,7 +188,7 @@ __device__ __forceinline__ void softmap_tile(const SoftmapArgs &g, float *sm_lds
             bmx[p] = stats[2 * col]; brs[p] = stats[2 * col + 1];
         }
     }
-    auto fetch = [&](int p, int k0) {
+    auto fetch = [&](int p, int k0) __attribute__((always_inline)) {
         if (EDGE) {
             if (A_RED_CONTIG) {
                 const int row = r0 + a_o + RP * p, k = k0 + a_q * 4;
@@ -222,13 +222,14 @@ __device__ __forceinline__ void softmap_tile(const SoftmapArgs &g, float *sm_lds
             }
         }
     };
-    auto commit = [&](int p, int buf) {
+    auto commit = [&](int p, int buf) __attribute__((always_inline)) {
         float *Ab = As + buf * KC * LDA, *Bb = Bs + buf * KC * LDB;
         if (A_RED_CONTIG) {
             float *d = Ab + (a_q * 4) * LDA + a_o + RP * p;
             d[0] = pa[p].x; d[LDA] = pa[p].y; d[2 * LDA] = pa[p].z; d[3 * LDA] = pa[p].w;
         } else {
-            *reinterpret_cast<float4 *>(Ab + (a_o + 8 * p) * LDA + a_q * 4) = pa[p];
+            const float4 va = make_float4(pa[p].x, pa[p].y, pa[p].z, pa[p].w);  // by value: keeps pa in registers
+            *reinterpret_cast<float4 *>(Ab + (a_o + 8 * p) * LDA + a_q * 4) = va;
         }
         float4 v = pb[p];
         if (!EDGE && MODE != 2) {  // W values -> softmax entries (the predicated path did it on load)
@@ -266,7 +267,7 @@ __device__ __forceinline__ void softmap_tile(const SoftmapArgs &g, float *sm_lds
     const int kh = lane >> 5, l32 = lane & 31;
     // one stage: MFMAs over buffer s&1; between MFMA groups, piece p of stage s+1 goes from
     // registers to the other buffer and piece p of stage s+2 is requested from memory
-    auto stage = [&](int s, auto do_commit, auto do_fetch) {
+    auto stage = [&](int s, auto do_commit, auto do_fetch) __attribute__((always_inline)) {
         const int cur = s & 1;
         const float *Ab = As + cur * KC * LDA + kh * LDA + wm + l32;
         const float *Bb = Bs + cur * KC * LDB + kh * LDB + wn + l32;
@@ -305,24 +306,48 @@ __device__ __forceinline__ void softmap_tile(const SoftmapArgs &g, float *sm_lds
     }
     // accumulator layout of a 32x32 tile: register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4, column l%32
     float *dst = g.out + (size_t)zc * R * C;
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
+    float *rowst = reinterpret_cast<float *>(sm_lds);  // MODE 2: per tile row {max, 1/sum, r}, staged once
+    if (MODE == 2) {
+        if (tid < SM_T) {
+            const int row = min(r0 + tid, R - 1);
+            rowst[tid * 4] = stats[2 * row];
+            rowst[tid * 4 + 1] = stats[2 * row + 1];
+            rowst[tid * 4 + 2] = g.r[row];
+        }
+        __syncthreads();
+    }
+    if (MODE == 2) {
+        // one 32x32 sub-tile per trip of a loop that is kept rolled: unrolled, the scheduler puts all
+        // 64 W loads in flight at once and the registers that costs push the staging buffers of
+        // the main loop into scratch memory
+#pragma clang loop unroll(disable)
+        for (int ij = 0; ij < 4; ++ij) {
+            const int i = ij >> 1, j = ij & 1;
+            const floatx16 a = ij == 0 ? acc[0][0] : ij == 1 ? acc[0][1] : ij == 2 ? acc[1][0] : acc[1][1];
             const int col = c0 + wn + j * 32 + (lane & 31);
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int row = r0 + wm + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                const int lr = wm + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                const int row = r0 + lr;
                 if (!EDGE || (row < R && col < C)) {
-                    float val = acc[i][j][v];
-                    if (MODE == 2) {
-                        const float sv = softmap_s(W[(size_t)row * I + col], stats[2 * row], stats[2 * row + 1], scale);
-                        val = sv * (val - g.r[row]) * g.inv_tau;
-                    }
-                    dst[(size_t)row * C + col] = val;
+                    const float sv = softmap_s(W[(size_t)row * I + col], rowst[lr * 4], rowst[lr * 4 + 1], scale);
+                    dst[(size_t)row * C + col] = sv * (a[v] - rowst[lr * 4 + 2]) * g.inv_tau;
                 }
             }
         }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int col = c0 + wn + j * 32 + (lane & 31);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = r0 + wm + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                    if (!EDGE || (row < R && col < C)) dst[(size_t)row * C + col] = acc[i][j][v];
+                }
+            }
+    }
 }
 
 // 1-D grid decoded so that blocks which share the large operand tile (W, or the gm column slab in
@@ -421,7 +446,7 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
             bmx[p] = stats[2 * col]; brs[p] = stats[2 * col + 1];
         }
     }
-    auto fetch = [&](int p, int k0) {
+    auto fetch = [&](int p, int k0) __attribute__((always_inline)) {
         if (A_RED_CONTIG) {
             const int row = r0 + a_o + 32 * p, k = k0 + a_q * 4;
             if (EDGE) pa[p] = make_float4(in_a(row, k), in_a(row, k + 1), in_a(row, k + 2), in_a(row, k + 3));
@@ -444,7 +469,7 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
             }
         }
     };
-    auto soft = [&](int p) -> float4 {
+    auto soft = [&](int p) __attribute__((always_inline)) -> float4 {
         float4 v = pb[p];
         if (!EDGE && MODE != 2) {
             v.x = softmap_s(v.x, bmx[p], brs[p], scale); v.y = softmap_s(v.y, bmx[p], brs[p], scale);
@@ -452,7 +477,7 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
         }
         return v;
     };
-    auto commit = [&](int p, int buf) {
+    auto commit = [&](int p, int buf) __attribute__((always_inline)) {
         char *Ab = As + buf * STAGE, *Bb = Bs + buf * STAGE;
         if (A_RED_CONTIG) {
             *reinterpret_cast<uint2 *>(Ab + (a_o + 32 * p) * SB_LD + a_q * 8) =
@@ -499,7 +524,7 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
     }
     __syncthreads();
     const int kh = lane >> 5, l32 = lane & 31;
-    auto stage = [&](int s, auto do_commit, auto do_fetch) {
+    auto stage = [&](int s, auto do_commit, auto do_fetch) __attribute__((always_inline)) {
         const int cur = s & 1;
         const char *Ab = As + cur * STAGE + (wm + l32) * SB_LD + kh * 16;
         const char *Bb = Bs + cur * STAGE + (wn + l32) * SB_LD + kh * 16;
@@ -530,24 +555,48 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
         if (s < nst) stage(s, F{}, F{});
     }
     float *dst = g.out + (size_t)zc * R * C;
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
+    float *rowst = reinterpret_cast<float *>(lds);  // MODE 2: per tile row {max, 1/sum, r}, staged once
+    if (MODE == 2) {
+        if (tid < SM_T) {
+            const int row = min(r0 + tid, R - 1);
+            rowst[tid * 4] = stats[2 * row];
+            rowst[tid * 4 + 1] = stats[2 * row + 1];
+            rowst[tid * 4 + 2] = g.r[row];
+        }
+        __syncthreads();
+    }
+    if (MODE == 2) {
+        // one 32x32 sub-tile per trip of a loop that is kept rolled: unrolled, the scheduler puts all
+        // 64 W loads in flight at once and the registers that costs push the staging buffers of
+        // the main loop into scratch memory
+#pragma clang loop unroll(disable)
+        for (int ij = 0; ij < 4; ++ij) {
+            const int i = ij >> 1, j = ij & 1;
+            const floatx16 a = ij == 0 ? acc[0][0] : ij == 1 ? acc[0][1] : ij == 2 ? acc[1][0] : acc[1][1];
             const int col = c0 + wn + j * 32 + (lane & 31);
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int row = r0 + wm + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                const int lr = wm + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                const int row = r0 + lr;
                 if (!EDGE || (row < R && col < C)) {
-                    float val = acc[i][j][v];
-                    if (MODE == 2) {
-                        const float sv = softmap_s(W[(size_t)row * I + col], stats[2 * row], stats[2 * row + 1], scale);
-                        val = sv * (val - g.r[row]) * g.inv_tau;
-                    }
-                    dst[(size_t)row * C + col] = val;
+                    const float sv = softmap_s(W[(size_t)row * I + col], rowst[lr * 4], rowst[lr * 4 + 1], scale);
+                    dst[(size_t)row * C + col] = sv * (a[v] - rowst[lr * 4 + 2]) * g.inv_tau;
                 }
             }
         }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int col = c0 + wn + j * 32 + (lane & 31);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = r0 + wm + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                    if (!EDGE || (row < R && col < C)) dst[(size_t)row * C + col] = acc[i][j][v];
+                }
+            }
+    }
 }
 
 template <int MODE>
@@ -579,28 +628,23 @@ static int softmap_check(int B, int I, int M, int precision) {
     return DL_OK;
 }
 
-// The gx product reduces over M.  It is cut into chunks so that the grid fills the chip: the chunk
-// count is the one whose block count comes closest to whole rounds of the 768 resident blocks
-// (256 CUs x 3 blocks), smallest count first on ties.
-static inline int softmap_gx_chunks(int B, int I, int M) {
+// The gx product reduces over M.  It is cut into chunks, one block per (output tile, chunk), about
+// 4096 blocks in all: measured on the 512 x 3136 x 48000 case the kernel keeps getting faster down
+// to chunks of about 1000 (short blocks keep the gm and W slabs of the blocks resident on an XCD
+// within its L2), while the fixed-order reduction of the partial products costs 2 us per chunk.
+static inline int softmap_gx_chunks(int B, int I, int M, int precision) {
+    (void)precision;
     const long long tiles = (long long)dl_ceil_div(I, SM_T) * dl_ceil_div(B, SM_T);
+    int chunks = dl_ceil_div(4096, tiles);
     const int max_chunks = dl_ceil_div(M, 256);
-    const int lo = dl_ceil_div(512, tiles), hi = dl_ceil_div(2304, tiles);
-    int best = 1;
-    double best_fill = 0.0;
-    for (int c = lo < 1 ? 1 : lo; c <= hi && c <= max_chunks; ++c) {
-        const long long blocks = tiles * c;
-        const double fill = (double)blocks / (double)(((blocks + 767) / 768) * 768);
-        if (fill > best_fill + 1e-9) { best_fill = fill; best = c; }
-    }
-    return best;
+    if (chunks > max_chunks) chunks = max_chunks;
+    return chunks < 1 ? 1 : chunks;
 }
 
 extern "C" size_t dl_soft_map_workspace_bytes(int B, int I, int M, int precision) {
-    (void)precision;
     if (B <= 0 || I <= 0 || M <= 0) return 256;
     return dl_align256((size_t)M * sizeof(float)) +
-           dl_align256((size_t)softmap_gx_chunks(B, I, M) * B * I * sizeof(float));
+           dl_align256((size_t)softmap_gx_chunks(B, I, M, precision) * B * I * sizeof(float));
 }
 
 extern "C" int dl_soft_map_fwd(const float *x, const float *W, float tau, float *m, float *stats, void *ws,
@@ -632,7 +676,7 @@ extern "C" int dl_soft_map_bwd(const float *x, const float *W, float tau, const 
     const float inv_tau = 1.0f / tau, scale = SM_LOG2E / tau;
     float *r = (float *)ws;
     float *part = (float *)((char *)ws + dl_align256((size_t)M * sizeof(float)));
-    const int chunks = softmap_gx_chunks(B, I, M);
+    const int chunks = softmap_gx_chunks(B, I, M, precision);
     int red_chunk = dl_ceil_div(M, chunks);
     red_chunk = dl_ceil_div(red_chunk, 32) * 32;  // whole stages, so float4 loads stay aligned
     const int col_tiles = dl_ceil_div(I, SM_T), used_chunks = dl_ceil_div(M, red_chunk);
