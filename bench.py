@@ -27,6 +27,12 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+# HBM bytes per launch of a workload's dominant kernel, from rocprofv3 counter runs of this file
+# (FETCH_SIZE scaled by 2.0 after calibration against a plain copy, plus WRITE_SIZE; the runs and
+# the calibration are written up under profiles/).  Measured, not computed: None where no run exists.
+MEASURED_TRAFFIC = {
+    ("dwn_k6_b4096_i16384_n8192", "dwn_bwd_gx"): 905969664,  # (303.8 * 2 + 256.0) MiB
+}
 
 WORKLOADS = {
     # name: (B, I, N, k, O)
@@ -239,7 +245,8 @@ def main():
         "config": {"workload": args.workload, "batch": B, "inputs": I, "nodes": N, "k": k, "output_dim": O,
                    "pass": "forward + EFD backward (input and table gradients)", "seed": 0, "mapping_seed": 42},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": dom_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": dom_gbs / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": split[dominant],
+                     "frac": dom_gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get((args.workload, dominant)),
+                     "algorithmic_bytes_per_launch": split[dominant],
                      "avg_launch_ms": avg[dominant]},
         "roofline_step": {"bound": "hbm", "achieved": step_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                           "frac": step_gbs / HBM_PEAK_GBS, "algorithmic_bytes_per_step": fwd_b + bwd_b},
