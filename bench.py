@@ -41,6 +41,8 @@ WORKLOADS = {
     # secondary workloads of the same path, reported with their own metric names (see run_secondary)
     "prob_k4_b1024_i4096_n4096": (1024, 4096, 4096, 4, 1),
     "softmap_b512_i3136_m48000": (512, 3136, 8000, 6, 1),
+    # whole training step through the layer API (BASELINE configs[4]): (B, features, first layer width, k, O)
+    "dwn_stack_b8192_train_step": (8192, 784, 16000, 6, 1),
 }
 
 
@@ -83,6 +85,50 @@ def kernel_times(step, reps):
             per.setdefault(name, []).append(ms)
     nat.profile_enable(False)
     return {name: float(np.mean(v)) for name, v in per.items()}
+
+
+def run_stack(args):
+    """Thermometer(4) -> RandomLayer+DWN k=6 with 16000 -> 8000 -> 4000 -> 2000 nodes -> GroupSum(10) ->
+    cross-entropy, backward, Adam on the tables: the reference's layer API end to end, one step per batch."""
+    from difflut_amd import REGISTRY
+    from difflut_amd import _native as nat
+    from difflut_amd.nodes.node_config import NodeConfig
+    from difflut_amd.utils import GroupSum
+
+    dev = torch.device("cuda:0")
+    B, F, _, k, O = WORKLOADS[args.workload]
+    widths = [16000, 8000, 4000, 2000]
+    torch.manual_seed(0)
+    x = torch.rand(B, F, device=dev)
+    labels = torch.randint(0, 10, (B,), device=dev)
+    enc = REGISTRY.build_encoder("thermometer", num_bits=4).fit(x)
+    layers, width = [], F * 4
+    for n in widths:
+        layers.append(REGISTRY.get_layer("random")(width, n, REGISTRY.get_node("dwn"),
+                                                   NodeConfig(input_dim=k, output_dim=O), seed=42).to(dev))
+        width = n * O
+    head = GroupSum(k=10, tau=1.0, use_randperm=False)
+    params = [p for layer in layers for p in layer.bank_parameters()]
+    opt = torch.optim.Adam(params, lr=1e-3)
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        h = enc.encode(x)
+        for layer in layers:
+            h = layer(h)
+        loss = torch.nn.functional.cross_entropy(head(h), labels)
+        loss.backward()
+        opt.step()
+
+    ms = time_steps(step, args.steps, args.warmup)
+    evals = B * sum(widths)
+    out = {"metric": "LUT-node evals/sec, training step (thermometer -> 4 DWN k=6 layers -> GroupSum -> CE, Adam)",
+           "value": evals / (ms * 1e-3), "unit": "node-evals/s", "ms_per_step": ms, "dtype": "f32",
+           "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "data": "synthetic",
+           "config": {"workload": args.workload, "batch": B, "features": F, "layers": widths, "k": k},
+           "kernel_ms": kernel_times(step, min(args.steps, 5))}
+    print(json.dumps(out))
 
 
 def run_secondary(args):
@@ -175,6 +221,8 @@ def main():
     lib = nat.lib()  # raises if the HIP library has not been built
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a ROCm device")
+    if args.workload.startswith("dwn_stack"):
+        return run_stack(args)
     if not args.workload.startswith("dwn"):
         return run_secondary(args)
     dev = torch.device("cuda:0")

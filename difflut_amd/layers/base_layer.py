@@ -202,6 +202,15 @@ class BaseLUTLayer(ABC, LUTLayerMixin, nn.Module):
             bank.tie(keep_grad=None if grads[name] is None else fn(grads[name]))
         return self
 
+    def bank_parameters(self):
+        """The layer's trainable tensors with every node parameter as ONE leaf [N, ...] (the storage the
+        per-node parameters are views of) followed by the layer's own parameters.  Handing these to an
+        optimizer instead of `parameters()` (N small tensors) makes its step one kernel per tensor;
+        both see the same memory.  Call after the layer is on its device: `.to()` re-creates the leaves."""
+        banks = [bank.tensor() for bank in self._banks.values()]
+        own = [p for name, p in self.named_parameters() if not name.startswith("nodes.")]
+        return banks + own
+
     def _run_nodes(self, x, plan):
         """All nodes on x [batch, width] through `plan` (index table over width) -> [batch, N*O]."""
         first = self.nodes[0]

@@ -201,6 +201,17 @@ def test_adam_steps_change_tables_in_place():
         losses.append(loss.item())
     assert losses[-1] < losses[0] and not np.array_equal(before, stacked(layer, "luts"))
     assert layer._banks["luts"].tied()
+    # one leaf per node parameter: same memory as the per-node views, one optimizer tensor
+    (flat,) = layer.bank_parameters()
+    assert flat.shape == (40, 1, 64) and flat.is_leaf and flat.requires_grad
+    opt = torch.optim.Adam([flat], lr=0.01)
+    before = stacked(layer, "luts").copy()
+    opt.zero_grad()
+    ((layer(x) - target) ** 2).mean().backward()
+    assert torch.equal(flat.grad[3], layer.nodes[3].luts.grad)
+    opt.step()
+    assert not np.array_equal(before, stacked(layer, "luts"))
+    assert np.array_equal(flat.detach().cpu().numpy(), stacked(layer, "luts"))
 
 
 # ------------------------------------------------------------------------------ benchmark shape
