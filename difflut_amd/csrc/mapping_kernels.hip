@@ -161,13 +161,16 @@ static struct {
 
 void dl_prof_begin(const char *kernel_name, hipStream_t s) {
     if (!g_prof.on || g_prof.count >= DL_PROF_MAX) return;
-    while (g_prof.created < 2 * (g_prof.count + 1)) hipEventCreate(&g_prof.ev[g_prof.created++]);
+    while (g_prof.created < 2 * (g_prof.count + 1)) {
+        if (hipEventCreate(&g_prof.ev[g_prof.created]) != hipSuccess) { g_prof.on = 0; return; }
+        ++g_prof.created;
+    }
     g_prof.name[g_prof.count] = kernel_name;
-    hipEventRecord(g_prof.ev[2 * g_prof.count], s);
+    (void)hipEventRecord(g_prof.ev[2 * g_prof.count], s);
 }
 void dl_prof_end(hipStream_t s) {
     if (!g_prof.on || g_prof.count >= DL_PROF_MAX) return;
-    hipEventRecord(g_prof.ev[2 * g_prof.count + 1], s);
+    (void)hipEventRecord(g_prof.ev[2 * g_prof.count + 1], s);
     ++g_prof.count;
 }
 
@@ -182,9 +185,10 @@ extern "C" int dl_profile_read(char *names, size_t names_bytes, float *ms, int m
     size_t used = 0;
     if (names && names_bytes) names[0] = 0;
     for (int i = 0; i < n; ++i) {
-        hipEventSynchronize(g_prof.ev[2 * i + 1]);
         float t = 0.0f;
-        hipEventElapsedTime(&t, g_prof.ev[2 * i], g_prof.ev[2 * i + 1]);
+        if (hipEventSynchronize(g_prof.ev[2 * i + 1]) != hipSuccess ||
+            hipEventElapsedTime(&t, g_prof.ev[2 * i], g_prof.ev[2 * i + 1]) != hipSuccess)
+            t = -1.0f;  // a failed measurement is reported as negative, never as zero
         if (ms) ms[i] = t;
         if (names) {
             const char *nm = g_prof.name[i];
