@@ -174,7 +174,7 @@ def run_secondary(args):
         x = torch.rand(B, I, device=dev)
         W = torch.randn(M, I, device=dev) * 0.01
         gm = torch.randn(B, M, device=dev)
-        m = torch.empty(B, M, device=dev); stats = torch.empty(2 * M, device=dev)
+        m = torch.empty(B, M, device=dev); stats = torch.empty(max(lib.dl_soft_map_saved_bytes(B, I, M, precision), 256), dtype=torch.uint8, device=dev)
         gx = torch.empty_like(x); gW = torch.empty_like(W)
         ws = torch.empty(max(lib.dl_soft_map_workspace_bytes(B, I, M, precision), 256), dtype=torch.uint8, device=dev)
 

@@ -462,21 +462,23 @@ static int dwn_check(int B, int I, int N, int k, int O) {
     if ((long long)N * O * ((long long)1 << k) > 0x7fffffffLL) return DL_ERR_UNSUPPORTED;
     return DL_OK;
 }
-// the fast kernels pack a node number into 23 bits of an entry record
-static inline bool dwn_fast(int N, int k) { return k <= DL_MAX_FAST_K && N < (1 << 23); }
+// the fast kernels pack a node number into 23 bits of an entry record and address table rows and
+// saved addresses with 32-bit byte offsets (column * 2^k * 4 and node * 64)
+static inline bool dwn_fast(int N, int k, int O) {
+    return k <= DL_MAX_FAST_K && N < (1 << 23) && (long long)N * O * ((long long)4 << k) < 0x7fffffffLL;
+}
 
 extern "C" size_t dl_dwn_saved_bytes(int B, int I, int N, int k, int O) {
-    (void)I; (void)O;
-    if (!dwn_fast(N, k)) return 256;  // nothing is kept; a token allocation keeps callers simple
+    (void)I;
+    if (!dwn_fast(N, k, O)) return 256;  // nothing is kept; a token allocation keeps callers simple
     return dl_align256((size_t)N * dwn_bt(B) * 64);
 }
 extern "C" size_t dl_dwn_fwd_workspace_bytes(int B, int I, int N, int k, int O) {
-    (void)O;
-    return dwn_fast(N, k) ? dwn_planes_bytes(B, I) : 256;
+    return dwn_fast(N, k, O) ? dwn_planes_bytes(B, I) : 256;
 }
 extern "C" size_t dl_dwn_bwd_workspace_bytes(int B, int I, int N, int k, int O) {
     (void)I;
-    return dwn_fast(N, k) ? dwn_table_bytes(N, k, O) + dwn_gyT_bytes(B, N, O) : 256;
+    return dwn_fast(N, k, O) ? dwn_table_bytes(N, k, O) + dwn_gyT_bytes(B, N, O) : 256;
 }
 
 template <int K>
@@ -498,7 +500,7 @@ extern "C" int dl_dwn_layer_fwd(const float *x, const int32_t *idx32, const floa
     int rc = dwn_check(B, I, N, k, O);
     if (rc) return rc;
     hipStream_t s = (hipStream_t)stream;
-    if (!dwn_fast(N, k)) return dwn_generic_forward(x, idx32, luts, y, B, I, N, k, O, s);
+    if (!dwn_fast(N, k, O)) return dwn_generic_forward(x, idx32, luts, y, B, I, N, k, O, s);
     if (!saved || !ws) return DL_ERR_NULL;
     if (ws_bytes < dl_dwn_fwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
     u64 *planes = (u64 *)ws;
@@ -544,7 +546,7 @@ extern "C" int dl_dwn_layer_bwd(const float *x, const void *saved, const int32_t
     hipStream_t s = (hipStream_t)stream;
     const long long NO = (long long)N * O;
     const int L = 1 << k;
-    if (!dwn_fast(N, k)) {
+    if (!dwn_fast(N, k, O)) {
         if (!x) return DL_ERR_NULL;
         return dwn_generic_backward(x, idx32, inv_ptr, inv_pos, luts, gy, alpha, beta, gx, gluts, B, I, N, k, O, s);
     }

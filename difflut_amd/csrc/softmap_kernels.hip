@@ -127,6 +127,8 @@ struct SoftmapArgs {
     float *out;
     int B, I, M;
     int inner_count, outer_count, col_tiles, red_chunk;
+    const unsigned short *Eb;  // precision 1: bf16 softmax numerators [M][I]
+    const float *rs;           // precision 1: 1 / row sum [M]
 };
 
 // MODE 0: forward   rows=b cols=o red=i   A = x[b,i]  (red contiguous)   B = S[o,i] (red contiguous)
@@ -381,9 +383,12 @@ static void softmap_launch(const SoftmapArgs &g, hipStream_t s) {
 }
 
 // ---------------------------------------------------------------------------------
-// bf16 operands, fp32 accumulation (v_mfma_f32_32x32x16_bf16).  Same tiling and operand modes as
-// the fp32 kernel; operands are rounded to bf16 (nearest even) while they are staged, the row
-// statistics, r and the gW epilogue stay fp32.  A lane feeds the MFMA eight consecutive k of one
+// bf16 operands, fp32 accumulation (v_mfma_f32_32x32x16_bf16), precision = 1.  Same tiling and
+// operand modes as the fp32 kernel.  Here the softmax numerators E[o,i] = exp((W - max)/tau) are
+// written once, rounded to bf16, by the row-statistics pass (301 MB for the 48000 x 3136 case, kept
+// with the statistics for the backward); 1/sum stays a per-row fp32 factor that is applied to the
+// forward output, to the gm operand of the gx product and in the gW epilogue.  x and gm are rounded
+// to bf16 (nearest even) while they are staged.  A lane feeds the MFMA eight consecutive k of one
 // row, so LDS holds a stage row-major, As[row][32 k] with 16 bytes of padding per row.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -395,18 +400,57 @@ __device__ __forceinline__ unsigned softmap_pk_bf16(float lo, float hi) {
     const floatx2 v = {lo, hi};
     return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2));
 }
+__device__ __forceinline__ float softmap_bf16_f32(unsigned short h) { return __uint_as_float((unsigned)h << 16); }
+
+// one wavefront per row of W: max, then E = bf16(exp2((w - max) * scale)) and 1 / sum of the rounded E
+__global__ __launch_bounds__(256) void softmap_rowstats_bf16(const float *__restrict__ W, float scale, float *__restrict__ mxs,
+                                                              float *__restrict__ rss, unsigned short *__restrict__ Eb,
+                                                              int M, int I) {
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= M) return;
+    const float *w = W + (size_t)row * I;
+    unsigned short *e = Eb + (size_t)row * I;
+    float mx = -INFINITY, sum = 0.0f;
+    if (I % 4 == 0) {
+        const float4 *w4 = reinterpret_cast<const float4 *>(w);
+        const int n4 = I >> 2;
+        for (int i = lane; i < n4; i += 64) {
+            const float4 a = w4[i];
+            mx = fmaxf(mx, fmaxf(fmaxf(a.x, a.y), fmaxf(a.z, a.w)));
+        }
+        for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+        for (int i = lane; i < n4; i += 64) {
+            const float4 a = w4[i];
+            const unsigned lo = softmap_pk_bf16(softmap_e(a.x, mx, scale), softmap_e(a.y, mx, scale));
+            const unsigned hi = softmap_pk_bf16(softmap_e(a.z, mx, scale), softmap_e(a.w, mx, scale));
+            sum += (__uint_as_float(lo << 16) + __uint_as_float(lo & 0xffff0000u)) +
+                   (__uint_as_float(hi << 16) + __uint_as_float(hi & 0xffff0000u));
+            *reinterpret_cast<uint2 *>(e + 4 * i) = make_uint2(lo, hi);
+        }
+    } else {
+        for (int i = lane; i < I; i += 64) mx = fmaxf(mx, w[i]);
+        for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+        for (int i = lane; i < I; i += 64) {
+            const unsigned short h = (unsigned short)(softmap_pk_bf16(softmap_e(w[i], mx, scale), 0.0f) & 0xffffu);
+            sum += softmap_bf16_f32(h);
+            e[i] = h;
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+    if (lane == 0) { mxs[row] = mx; rss[row] = 1.0f / sum; }
+}
 
 template <int MODE, bool EDGE>
 __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *lds, int rt, int ct, int zc) {
-    constexpr int KC = SB_K, P = 4;
+    constexpr int KC = SB_K;
     constexpr bool A_RED_CONTIG = MODE != 2;
-    constexpr bool B_RED_CONTIG = MODE == 0;
     constexpr int STAGE = SM_T * SB_LD;  // bytes of one operand stage
     char *const As = lds;                // [2][128][SB_LD]
     char *const Bs = lds + 2 * STAGE;
-    const float *__restrict__ x = g.x, *__restrict__ W = g.W, *__restrict__ stats = g.stats, *__restrict__ gm = g.gm;
+    const float *__restrict__ x = g.x, *__restrict__ gm = g.gm, *__restrict__ rs = g.rs;
+    const unsigned short *__restrict__ Eb = g.Eb;
     const int B = g.B, I = g.I, M = g.M;
-    const float scale = g.scale;
     const int R = MODE == 2 ? M : B, C = MODE == 0 ? M : I;
     const int KD = MODE == 0 ? I : (MODE == 1 ? M : B);
     const int r0 = rt * SM_T, c0 = ct * SM_T;
@@ -415,73 +459,46 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
-    float4 pa[P], pb[P];
-    float bmx[P], brs[P];
 
-    // red-contiguous operand: float4 along k, 8 per row, rows q_o + 32 p.
-    // row/col-contiguous operand: float4 along the row/col axis for one k; piece p holds
-    // k = 2 q_o + (p & 1) + 16 (p >> 1), so pieces 2j and 2j+1 are neighbours in k and go to LDS
-    // as packed pairs.
+    // ---- A operand, fp32 in memory (x; gm scaled by 1/sum of its column in the gx product; gm).
+    // red-contiguous: float4 along k, 8 per row, rows a_o + 32 p.  row-contiguous: float4 along the
+    // rows for one k; piece p holds k = 2 a_o + (p & 1) + 16 (p >> 1), so pieces 2j and 2j+1 are
+    // neighbours in k and go to LDS as packed pairs.
+    float4 pa[4];
+    float4 ars[2];  // gx product: 1/sum of the four k of pieces {0,1} and {2,3}
     const int a_q = A_RED_CONTIG ? (tid & 7) : (tid & 31), a_o = A_RED_CONTIG ? (tid >> 3) : (tid >> 5);
-    const int b_q = B_RED_CONTIG ? (tid & 7) : (tid & 31), b_o = B_RED_CONTIG ? (tid >> 3) : (tid >> 5);
     const int lda = MODE == 0 ? I : M;
     auto k_of = [](int o, int p) { return 2 * o + (p & 1) + 16 * (p >> 1); };
-
     auto in_a = [&](int row, int k) -> float {
         if (row >= R || k >= k_end) return 0.0f;
         if (MODE == 0) return x[(size_t)row * I + k];
-        if (MODE == 1) return gm[(size_t)row * M + k];
+        if (MODE == 1) return gm[(size_t)row * M + k] * rs[k];
         return gm[(size_t)k * M + row];
     };
-    auto in_b = [&](int k, int col) -> float {
-        if (col >= C || k >= k_end) return 0.0f;
-        if (MODE == 0) return softmap_s(W[(size_t)col * I + k], stats[2 * col], stats[2 * col + 1], scale);
-        if (MODE == 1) return softmap_s(W[(size_t)k * I + col], stats[2 * k], stats[2 * k + 1], scale);
-        return x[(size_t)k * I + col];
-    };
-    if (!EDGE && MODE == 0) {
-#pragma unroll
-        for (int p = 0; p < P; ++p) {
-            const int col = c0 + b_o + 32 * p;
-            bmx[p] = stats[2 * col]; brs[p] = stats[2 * col + 1];
-        }
-    }
-    auto fetch = [&](int p, int k0) __attribute__((always_inline)) {
+    auto fetch_a = [&](int p, int k0) __attribute__((always_inline)) {
         if (A_RED_CONTIG) {
             const int row = r0 + a_o + 32 * p, k = k0 + a_q * 4;
             if (EDGE) pa[p] = make_float4(in_a(row, k), in_a(row, k + 1), in_a(row, k + 2), in_a(row, k + 3));
-            else pa[p] = *reinterpret_cast<const float4 *>((MODE == 0 ? x : gm) + (size_t)row * lda + k);
+            else {
+                pa[p] = *reinterpret_cast<const float4 *>((MODE == 0 ? x : gm) + (size_t)row * lda + k);
+                if (MODE == 1 && (p & 1) == 0) ars[p >> 1] = *reinterpret_cast<const float4 *>(rs + k);
+            }
         } else {
             const int k = k0 + k_of(a_o, p), row = r0 + a_q * 4;
             if (EDGE) pa[p] = make_float4(in_a(row, k), in_a(row + 1, k), in_a(row + 2, k), in_a(row + 3, k));
             else pa[p] = *reinterpret_cast<const float4 *>(gm + (size_t)k * M + row);
         }
-        if (B_RED_CONTIG) {
-            const int col = c0 + b_o + 32 * p, k = k0 + b_q * 4;
-            if (EDGE) pb[p] = make_float4(in_b(k, col), in_b(k + 1, col), in_b(k + 2, col), in_b(k + 3, col));
-            else pb[p] = *reinterpret_cast<const float4 *>(W + (size_t)col * I + k);
-        } else {
-            const int k = k0 + k_of(b_o, p), col = c0 + b_q * 4;
-            if (EDGE) pb[p] = make_float4(in_b(k, col), in_b(k, col + 1), in_b(k, col + 2), in_b(k, col + 3));
-            else {
-                pb[p] = *reinterpret_cast<const float4 *>((MODE == 1 ? W : x) + (size_t)k * I + col);
-                if (MODE == 1) { bmx[p] = stats[2 * k]; brs[p] = stats[2 * k + 1]; }
-            }
-        }
     };
-    auto soft = [&](int p) __attribute__((always_inline)) -> float4 {
-        float4 v = pb[p];
-        if (!EDGE && MODE != 2) {
-            v.x = softmap_s(v.x, bmx[p], brs[p], scale); v.y = softmap_s(v.y, bmx[p], brs[p], scale);
-            v.z = softmap_s(v.z, bmx[p], brs[p], scale); v.w = softmap_s(v.w, bmx[p], brs[p], scale);
-        }
-        return v;
-    };
-    auto commit = [&](int p, int buf) __attribute__((always_inline)) {
-        char *Ab = As + buf * STAGE, *Bb = Bs + buf * STAGE;
+    auto commit_a = [&](int p, int buf) __attribute__((always_inline)) {
+        char *Ab = As + buf * STAGE;
         if (A_RED_CONTIG) {
+            float4 v = make_float4(pa[p].x, pa[p].y, pa[p].z, pa[p].w);
+            if (!EDGE && MODE == 1) {
+                const float4 f = ars[p >> 1];
+                v.x *= f.x; v.y *= f.y; v.z *= f.z; v.w *= f.w;
+            }
             *reinterpret_cast<uint2 *>(Ab + (a_o + 32 * p) * SB_LD + a_q * 8) =
-                make_uint2(softmap_pk_bf16(pa[p].x, pa[p].y), softmap_pk_bf16(pa[p].z, pa[p].w));
+                make_uint2(softmap_pk_bf16(v.x, v.y), softmap_pk_bf16(v.z, v.w));
         } else if (p & 1) {
             char *d = Ab + (a_q * 4) * SB_LD + k_of(a_o, p - 1) * 2;
             *reinterpret_cast<unsigned *>(d) = softmap_pk_bf16(pa[p - 1].x, pa[p].x);
@@ -489,18 +506,92 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
             *reinterpret_cast<unsigned *>(d + 2 * SB_LD) = softmap_pk_bf16(pa[p - 1].z, pa[p].z);
             *reinterpret_cast<unsigned *>(d + 3 * SB_LD) = softmap_pk_bf16(pa[p - 1].w, pa[p].w);
         }
-        if (B_RED_CONTIG) {
-            const float4 v = soft(p);
-            *reinterpret_cast<uint2 *>(Bb + (b_o + 32 * p) * SB_LD + b_q * 8) =
-                make_uint2(softmap_pk_bf16(v.x, v.y), softmap_pk_bf16(v.z, v.w));
-        } else if (p & 1) {
-            const float4 u = soft(p - 1), v = soft(p);
-            char *d = Bb + (b_q * 4) * SB_LD + k_of(b_o, p - 1) * 2;
-            *reinterpret_cast<unsigned *>(d) = softmap_pk_bf16(u.x, v.x);
-            *reinterpret_cast<unsigned *>(d + SB_LD) = softmap_pk_bf16(u.y, v.y);
-            *reinterpret_cast<unsigned *>(d + 2 * SB_LD) = softmap_pk_bf16(u.z, v.z);
-            *reinterpret_cast<unsigned *>(d + 3 * SB_LD) = softmap_pk_bf16(u.w, v.w);
+    };
+
+    // ---- B operand
+    //  MODE 0: exp2((W[o, k] - max[o]) * scale) from the fp32 W, red-contiguous, four float4 pieces like
+    //          the A operand (the bf16 copy E would be read in half cache lines per stage here)
+    //  MODE 1: E[k, i] bf16, column-contiguous: rows 2 kp and 2 kp + 1, 8 columns each -> packed pairs
+    //  MODE 2: x[k, i] fp32, column-contiguous: as the A operand
+    uint4 pe[2];
+    float4 pb[MODE == 1 ? 1 : 4];
+    float bmx[4];  // MODE 0: row maxima of the W rows this thread stages
+    const int e_q = tid & 15, e_o = tid >> 4;
+    const int b_q = MODE == 0 ? (tid & 7) : (tid & 31), b_o = MODE == 0 ? (tid >> 3) : (tid >> 5);
+    auto eb = [&](int o, int i) -> unsigned {  // predicated scalar access, bits of E[o,i]
+        return (o < M && i < I) ? (unsigned)Eb[(size_t)o * I + i] : 0u;
+    };
+    if (MODE == 0) {
+#pragma unroll
+        for (int p = 0; p < 4; ++p) bmx[p] = g.stats[min(c0 + b_o + 32 * p, C - 1)];
+    }
+    auto fetch_b = [&](int p, int k0) __attribute__((always_inline)) {
+        if (MODE == 0) {
+            const int col = c0 + b_o + 32 * p, k = k0 + b_q * 4;
+            auto wv = [&](int kk) -> float { return (col < C && kk < k_end) ? g.W[(size_t)col * I + kk] : -INFINITY; };
+            if (EDGE) pb[p] = make_float4(wv(k), wv(k + 1), wv(k + 2), wv(k + 3));
+            else pb[p] = *reinterpret_cast<const float4 *>(g.W + (size_t)col * I + k);
+        } else if (MODE == 1) {
+            const int k = k0 + 2 * e_o + p, col = c0 + e_q * 8;  // p = 0, 1: the two rows of the pair
+            if (EDGE) {
+                unsigned wv[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const unsigned lo = k < k_end ? eb(k, col + 2 * j) : 0u;
+                    const unsigned hi = k < k_end ? eb(k, col + 2 * j + 1) : 0u;
+                    wv[j] = lo | (hi << 16);
+                }
+                pe[p] = make_uint4(wv[0], wv[1], wv[2], wv[3]);
+            } else {
+                pe[p] = *reinterpret_cast<const uint4 *>(Eb + (size_t)k * I + col);
+            }
+        } else {
+            const int k = k0 + k_of(b_o, p), col = c0 + b_q * 4;
+            auto xv = [&](int kk, int cc) -> float { return (kk < k_end && cc < C) ? x[(size_t)kk * I + cc] : 0.0f; };
+            if (EDGE) pb[p] = make_float4(xv(k, col), xv(k, col + 1), xv(k, col + 2), xv(k, col + 3));
+            else pb[p] = *reinterpret_cast<const float4 *>(x + (size_t)k * I + col);
         }
+    };
+    auto commit_b = [&](int p, int buf) __attribute__((always_inline)) {
+        char *Bb = Bs + buf * STAGE;
+        if (MODE == 0) {
+            // exp2(-inf) = 0 covers the predicated path's padding
+            const float e0 = softmap_e(pb[p].x, bmx[p], g.scale), e1 = softmap_e(pb[p].y, bmx[p], g.scale);
+            const float e2 = softmap_e(pb[p].z, bmx[p], g.scale), e3 = softmap_e(pb[p].w, bmx[p], g.scale);
+            *reinterpret_cast<uint2 *>(Bb + (b_o + 32 * p) * SB_LD + b_q * 8) =
+                make_uint2(softmap_pk_bf16(e0, e1), softmap_pk_bf16(e2, e3));
+        } else if (MODE == 1) {
+            if (p == 1) {
+                const unsigned ra[4] = {pe[0].x, pe[0].y, pe[0].z, pe[0].w};
+                const unsigned rb[4] = {pe[1].x, pe[1].y, pe[1].z, pe[1].w};
+                char *d = Bb + (e_q * 8) * SB_LD + (2 * e_o) * 2;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const unsigned a = ra[j >> 1], b = rb[j >> 1];
+                    // low halves (even column) or high halves (odd column) of the two rows -> (k, k+1)
+                    const unsigned v = (j & 1) ? __builtin_amdgcn_perm(b, a, 0x07060302u) : __builtin_amdgcn_perm(b, a, 0x05040100u);
+                    *reinterpret_cast<unsigned *>(d + j * SB_LD) = v;
+                }
+            }
+        } else if (p & 1) {
+            char *d = Bb + (b_q * 4) * SB_LD + k_of(b_o, p - 1) * 2;
+            *reinterpret_cast<unsigned *>(d) = softmap_pk_bf16(pb[p - 1].x, pb[p].x);
+            *reinterpret_cast<unsigned *>(d + SB_LD) = softmap_pk_bf16(pb[p - 1].y, pb[p].y);
+            *reinterpret_cast<unsigned *>(d + 2 * SB_LD) = softmap_pk_bf16(pb[p - 1].z, pb[p].z);
+            *reinterpret_cast<unsigned *>(d + 3 * SB_LD) = softmap_pk_bf16(pb[p - 1].w, pb[p].w);
+        }
+    };
+    // pieces handled after the first (h = 0) and the second (h = 1) half of a stage's MFMAs
+    // (the two rows of a MODE 1 pair travel together in the second half: they are packed in one go)
+    auto fetch_half = [&](int h, int k0) __attribute__((always_inline)) {
+        fetch_a(2 * h, k0); fetch_a(2 * h + 1, k0);
+        if (MODE != 1) { fetch_b(2 * h, k0); fetch_b(2 * h + 1, k0); }
+        else if (h == 1) { fetch_b(0, k0); fetch_b(1, k0); }
+    };
+    auto commit_half = [&](int h, int buf) __attribute__((always_inline)) {
+        commit_a(2 * h, buf); commit_a(2 * h + 1, buf);
+        if (MODE != 1) { commit_b(2 * h, buf); commit_b(2 * h + 1, buf); }
+        else if (h == 1) commit_b(1, buf);
     };
 
     floatx16 acc[2][2];
@@ -513,14 +604,9 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
 
     const int nst = (k_end - k_begin + KC - 1) / KC;
     if (nst > 0) {
-#pragma unroll
-        for (int p = 0; p < P; ++p) fetch(p, k_begin);
-#pragma unroll
-        for (int p = 0; p < P; ++p) commit(p, 0);
-        if (nst > 1) {
-#pragma unroll
-            for (int p = 0; p < P; ++p) fetch(p, k_begin + KC);
-        }
+        fetch_half(0, k_begin); fetch_half(1, k_begin);
+        commit_half(0, 0); commit_half(1, 0);
+        if (nst > 1) { fetch_half(0, k_begin + KC); fetch_half(1, k_begin + KC); }
     }
     __syncthreads();
     const int kh = lane >> 5, l32 = lane & 31;
@@ -538,11 +624,8 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
             acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b1, acc[0][1], 0, 0, 0);
             acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b0, acc[1][0], 0, 0, 0);
             acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b1, acc[1][1], 0, 0, 0);
-            if constexpr (decltype(do_commit)::value) { commit(2 * kk, cur ^ 1); commit(2 * kk + 1, cur ^ 1); }
-            if constexpr (decltype(do_fetch)::value) {
-                fetch(2 * kk, k_begin + (s + 2) * KC);
-                fetch(2 * kk + 1, k_begin + (s + 2) * KC);
-            }
+            if constexpr (decltype(do_commit)::value) commit_half(kk, cur ^ 1);
+            if constexpr (decltype(do_fetch)::value) fetch_half(kk, k_begin + (s + 2) * KC);
         }
         __syncthreads();
     };
@@ -555,20 +638,15 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
         if (s < nst) stage(s, F{}, F{});
     }
     float *dst = g.out + (size_t)zc * R * C;
-    float *rowst = reinterpret_cast<float *>(lds);  // MODE 2: per tile row {max, 1/sum, r}, staged once
     if (MODE == 2) {
+        float *rowst = reinterpret_cast<float *>(lds);  // per tile row {1/sum, r}
         if (tid < SM_T) {
             const int row = min(r0 + tid, R - 1);
-            rowst[tid * 4] = stats[2 * row];
-            rowst[tid * 4 + 1] = stats[2 * row + 1];
-            rowst[tid * 4 + 2] = g.r[row];
+            rowst[tid * 2] = rs[row];
+            rowst[tid * 2 + 1] = g.r[row];
         }
         __syncthreads();
-    }
-    if (MODE == 2) {
-        // one 32x32 sub-tile per trip of a loop that is kept rolled: unrolled, the scheduler puts all
-        // 64 W loads in flight at once and the registers that costs push the staging buffers of
-        // the main loop into scratch memory
+        // rolled on purpose (see the fp32 kernel): gW = S (G - r) / tau with S = E / sum
 #pragma clang loop unroll(disable)
         for (int ij = 0; ij < 4; ++ij) {
             const int i = ij >> 1, j = ij & 1;
@@ -579,8 +657,8 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
                 const int lr = wm + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
                 const int row = r0 + lr;
                 if (!EDGE || (row < R && col < C)) {
-                    const float sv = softmap_s(W[(size_t)row * I + col], rowst[lr * 4], rowst[lr * 4 + 1], scale);
-                    dst[(size_t)row * C + col] = sv * (a[v] - rowst[lr * 4 + 2]) * g.inv_tau;
+                    const float sv = softmap_bf16_f32(Eb[(size_t)row * I + col]) * rowst[lr * 2];
+                    dst[(size_t)row * C + col] = sv * (a[v] - rowst[lr * 2 + 1]) * g.inv_tau;
                 }
             }
         }
@@ -590,10 +668,11 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const int col = c0 + wn + j * 32 + (lane & 31);
+                const float f = MODE == 0 ? rs[min(col, C - 1)] : 1.0f;  // forward: columns are rows of W
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const int row = r0 + wm + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                    if (!EDGE || (row < R && col < C)) dst[(size_t)row * C + col] = acc[i][j][v];
+                    if (!EDGE || (row < R && col < C)) dst[(size_t)row * C + col] = acc[i][j][v] * f;
                 }
             }
     }
@@ -611,7 +690,7 @@ __global__ __launch_bounds__(256, 3) void softmap_mfma_bf16(SoftmapArgs g) {
     const int KD = MODE == 0 ? g.I : (MODE == 1 ? g.M : g.B);
     const int k_begin = zc * g.red_chunk, k_end = min(KD, k_begin + g.red_chunk);
     const bool inside = (rt + 1) * SM_T <= R && (ct + 1) * SM_T <= C && (k_end - k_begin) % SB_K == 0 &&
-                        g.red_chunk % 4 == 0 && g.I % 4 == 0 && g.M % 4 == 0;
+                        g.red_chunk % 4 == 0 && g.I % 8 == 0 && g.M % 4 == 0;
     if (inside) softmap_tile_bf16<MODE, false>(g, lds, rt, ct, zc);
     else softmap_tile_bf16<MODE, true>(g, lds, rt, ct, zc);
 }
@@ -641,6 +720,15 @@ static inline int softmap_gx_chunks(int B, int I, int M, int precision) {
     return chunks < 1 ? 1 : chunks;
 }
 
+// what the forward leaves for the backward in `stats`: fp32 operands: {max, 1/sum} per row of W;
+// bf16 operands: max[M], 1/sum[M] and the bf16 softmax numerators [M][I]
+static inline size_t softmap_stats_bytes(int M) { return dl_align256((size_t)2 * M * sizeof(float)); }
+extern "C" size_t dl_soft_map_saved_bytes(int B, int I, int M, int precision) {
+    (void)B;
+    if (I <= 0 || M <= 0) return 256;
+    return softmap_stats_bytes(M) + (precision == 1 ? dl_align256((size_t)M * I * sizeof(unsigned short)) : 0);
+}
+
 extern "C" size_t dl_soft_map_workspace_bytes(int B, int I, int M, int precision) {
     if (B <= 0 || I <= 0 || M <= 0) return 256;
     return dl_align256((size_t)M * sizeof(float)) +
@@ -656,11 +744,19 @@ extern "C" int dl_soft_map_fwd(const float *x, const float *W, float tau, float 
     if (!(tau > 0.0f)) return DL_ERR_SHAPE;
     hipStream_t s = (hipStream_t)stream;
     const float inv_tau = 1.0f / tau, scale = SM_LOG2E / tau;
-    DL_TIMED("softmap_rowstats", s, (softmap_rowstats<<<dl_ceil_div(M, 4), 256, 0, s>>>(W, scale, stats, M, I)));
-    const SoftmapArgs g{x, W, stats, nullptr, nullptr, scale, inv_tau, m, B, I, M,
-                        dl_ceil_div(B, SM_T), dl_ceil_div(M, SM_T), 1, dl_ceil_div(I, 4) * 4};
-    if (precision == 1) DL_TIMED("softmap_bf16_fwd", s, (softmap_launch_bf16<0>(g, s)));
-    else DL_TIMED("softmap_mfma_fwd", s, (softmap_launch<0, SM_K0>(g, s)));
+    SoftmapArgs g{x, W, stats, nullptr, nullptr, scale, inv_tau, m, B, I, M,
+                  dl_ceil_div(B, SM_T), dl_ceil_div(M, SM_T), 1, dl_ceil_div(I, 4) * 4, nullptr, nullptr};
+    if (precision == 1) {
+        unsigned short *Eb = (unsigned short *)((char *)stats + softmap_stats_bytes(M));
+        DL_TIMED("softmap_rowstats_bf16", s,
+                 (softmap_rowstats_bf16<<<dl_ceil_div(M, 4), 256, 0, s>>>(W, scale, stats, stats + M, Eb, M, I)));
+        g.Eb = Eb;
+        g.rs = stats + M;
+        DL_TIMED("softmap_bf16_fwd", s, (softmap_launch_bf16<0>(g, s)));
+    } else {
+        DL_TIMED("softmap_rowstats", s, (softmap_rowstats<<<dl_ceil_div(M, 4), 256, 0, s>>>(W, scale, stats, M, I)));
+        DL_TIMED("softmap_mfma_fwd", s, (softmap_launch<0, SM_K0>(g, s)));
+    }
     return dl_launch_status();
 }
 
@@ -680,9 +776,11 @@ extern "C" int dl_soft_map_bwd(const float *x, const float *W, float tau, const 
     int red_chunk = dl_ceil_div(M, chunks);
     red_chunk = dl_ceil_div(red_chunk, 32) * 32;  // whole stages, so float4 loads stay aligned
     const int col_tiles = dl_ceil_div(I, SM_T), used_chunks = dl_ceil_div(M, red_chunk);
+    const unsigned short *Eb = precision == 1 ? (const unsigned short *)((const char *)stats + softmap_stats_bytes(M)) : nullptr;
+    const float *rs = precision == 1 ? stats + M : nullptr;
     DL_TIMED("softmap_rowdot", s, (softmap_rowdot<<<dl_ceil_div(M, 32), 256, 0, s>>>(gm, m, r, B, M)));
     const SoftmapArgs ggx{x, W, stats, gm, nullptr, scale, inv_tau, used_chunks > 1 ? part : gx, B, I, M,
-                          dl_ceil_div(B, SM_T), col_tiles * used_chunks, col_tiles, red_chunk};
+                          dl_ceil_div(B, SM_T), col_tiles * used_chunks, col_tiles, red_chunk, Eb, rs};
     if (precision == 1) DL_TIMED("softmap_bf16_gx", s, (softmap_launch_bf16<1>(ggx, s)));
     else DL_TIMED("softmap_mfma_gx", s, (softmap_launch<1, SM_K1>(ggx, s)));
     if (used_chunks > 1)
@@ -690,7 +788,7 @@ extern "C" int dl_soft_map_bwd(const float *x, const float *W, float tau, const 
                  (softmap_reduce_chunks<<<dl_ceil_div((long long)B * I, 256), 256, 0, s>>>(part, gx, (long long)B * I,
                                                                                          used_chunks)));
     const SoftmapArgs ggw{x, W, stats, gm, r, scale, inv_tau, gW, B, I, M,
-                          col_tiles, dl_ceil_div(M, SM_T), 1, dl_ceil_div(B, 4) * 4};
+                          col_tiles, dl_ceil_div(M, SM_T), 1, dl_ceil_div(B, 4) * 4, Eb, rs};
     if (precision == 1) DL_TIMED("softmap_bf16_gw", s, (softmap_launch_bf16<2>(ggw, s)));
     else DL_TIMED("softmap_mfma_gw", s, (softmap_launch<2, SM_K2>(ggw, s)));
     return dl_launch_status();

@@ -208,7 +208,7 @@ class SoftMapFunction(torch.autograd.Function):
             raise RuntimeError(f"shape mismatch: x {tuple(x.shape)} vs W {tuple(W.shape)}")
         lib = nat.lib()
         m = torch.empty((B, M), dtype=torch.float32, device=x.device)
-        stats = torch.empty((2 * M,), dtype=torch.float32, device=x.device)
+        stats = _bytes(lib.dl_soft_map_saved_bytes(B, I, M, precision), x.device)
         ws = _bytes(lib.dl_soft_map_workspace_bytes(B, I, M, precision), x.device)
         nat.check(lib.dl_soft_map_fwd(nat.ptr(x), nat.ptr(W), float(tau), nat.ptr(m), nat.ptr(stats), nat.ptr(ws),
                                       ws.numel(), B, I, M, precision, nat.stream()))

@@ -133,10 +133,12 @@ int dl_prob_layer_eval(const float *x, const int32_t *idx32, const float *raw_w,
  *   x [B,I], W [M,I], m [B,M];   S = softmax(W / tau) along I, never materialised.
  * precision: 0 = fp32 operands on the fp32 matrix cores (reference numerics),
  *            1 = bf16 operands, fp32 accumulation (tolerance documented with the tests).
- * stats [2*M] floats is written by the forward (row max and 1/sum of exp) and
- * read by the backward.
+ * stats (dl_soft_map_saved_bytes bytes) is written by the forward and read by the backward.
  *   gx = gm * S,   gW = S * (G - r) / tau with G = gm^T x and r[o] = sum_b gm[b,o] m[b,o].
  * ------------------------------------------------------------------------ */
+/* size of `stats`: what the forward keeps for the backward (row maximum and 1/sum; with
+ * precision 1 also the bf16 softmax numerators, M*I*2 bytes) */
+size_t dl_soft_map_saved_bytes(int B, int I, int M, int precision);
 size_t dl_soft_map_workspace_bytes(int B, int I, int M, int precision);
 int dl_soft_map_fwd(const float *x, const float *W, float tau, float *m, float *stats,
                     void *ws, size_t ws_bytes, int B, int I, int M, int precision, void *stream);
