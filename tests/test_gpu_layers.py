@@ -258,6 +258,67 @@ def test_full_size_properties_dwn_k6_b4096_n8192():
     torch.testing.assert_close(gl1[:, 0, :].double(), want, rtol=1e-5, atol=1e-4)
 
 
+def test_full_size_probabilistic_k4_b1024_n4096():
+    """BASELINE configs[1] shape against a float64 torch restatement of the same fold (the checker runs on
+    the GPU; the first nodes also go through the numpy oracle)."""
+    from difflut_amd import ops
+    torch.manual_seed(1)
+    B, I, N, k, T = 1024, 4096, 4096, 4, 1.0
+    x = torch.sigmoid(torch.randn(B, I, device="cuda"))
+    idx = orc.random_mapping(I, N, k, seed=42)
+    plan = ops.MappingPlan(idx.cuda(), I)
+    raw = torch.rand(N, 1 << k, 1, device="cuda")
+    gy = torch.randn(B, N, device="cuda")
+    xg = x.clone().requires_grad_(); wg = raw.clone().requires_grad_()
+    y = ops.ProbLayerFunction.apply(xg, wg, plan, T)
+    y.backward(gy)
+    # float64 reference: multilinear interpolation of the sigmoid table, folded input by input
+    xd = x.double().requires_grad_(); wd = raw.double().requires_grad_()
+    m = xd[:, idx.long().cuda()]                                   # [B,N,k]
+    v = torch.sigmoid(wd[:, :, 0] / T)[None].expand(B, N, 1 << k)
+    for j in range(k):
+        v = v[..., 0::2] + m[..., j:j + 1] * (v[..., 1::2] - v[..., 0::2])
+    yd = v[..., 0]
+    yd.backward(gy.double())
+    torch.testing.assert_close(y.detach().double(), yd.detach(), rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(xg.grad.double(), xd.grad, rtol=1e-5, atol=2e-6)
+    # a table gradient sums 1024 terms of size <= |gy| p_a sigmoid'(w) <= 0.25 |gy|
+    torch.testing.assert_close(wg.grad.double(), wd.grad, rtol=1e-5, atol=2e-5)
+    # first nodes through the numpy oracle as well
+    n0 = 64
+    want = orc.prob_layer_forward(x.cpu().numpy(), idx.numpy()[:n0], raw.cpu().numpy()[:n0], T, dtype=torch.float64)
+    np.testing.assert_allclose(y.detach().cpu().numpy()[:, :n0], want[:, :, 0], rtol=1e-5, atol=1e-6)
+    # deterministic: fixed summation orders everywhere
+    xg2 = x.clone().requires_grad_(); wg2 = raw.clone().requires_grad_()
+    ops.ProbLayerFunction.apply(xg2, wg2, plan, T).backward(gy)
+    assert torch.equal(xg2.grad, xg.grad) and torch.equal(wg2.grad, wg.grad)
+
+
+@pytest.mark.parametrize("precision", [0, 1])
+def test_full_size_soft_mapping_b512_i3136_m48000(precision):
+    """BASELINE configs[3] shape against float64 torch autograd of softmax + matmul (learnable_layer.py:254-255).
+    fp32 operands: rtol 1e-4 on sums of 3136 .. 48000 terms; bf16 operands: 1e-2 of the tensor's largest value."""
+    from difflut_amd import ops
+    torch.manual_seed(2)
+    B, I, M, tau = 512, 3136, 48000, 1.0
+    x = torch.rand(B, I, device="cuda")
+    W = torch.randn(M, I, device="cuda") * 0.01
+    gm = torch.randn(B, M, device="cuda")
+    xg = x.clone().requires_grad_(); Wg = W.clone().requires_grad_()
+    m = ops.SoftMapFunction.apply(xg, Wg, tau, precision)
+    m.backward(gm)
+    xd = x.double().requires_grad_(); Wd = W.double().requires_grad_()
+    md = xd @ torch.softmax(Wd / tau, dim=-1).t()
+    md.backward(gm.double())
+    if precision == 0:
+        torch.testing.assert_close(m.detach().double(), md.detach(), rtol=1e-5, atol=1e-6)
+        torch.testing.assert_close(xg.grad.double(), xd.grad, rtol=1e-4, atol=2e-5 * float(xd.grad.abs().max()))
+        torch.testing.assert_close(Wg.grad.double(), Wd.grad, rtol=1e-4, atol=2e-5 * float(Wd.grad.abs().max()))
+    else:
+        for got, want in ((m.detach(), md.detach()), (xg.grad, xd.grad), (Wg.grad, Wd.grad)):
+            assert float((got.double() - want).abs().max()) <= 1e-2 * float(want.abs().max())
+
+
 def test_legacy_extension_names_and_signatures(golden):
     """tests/test_layers/test_fused_kernels.py:159-179 imports efd_cuda / efd_fused_cuda by bare name;
     the shims answer with the reference's signatures."""
