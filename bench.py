@@ -110,12 +110,17 @@ def run_stack(args):
     head = GroupSum(k=10, tau=1.0, use_randperm=False)
     params = [p for layer in layers for p in layer.bank_parameters()]
     opt = torch.optim.Adam(params, lr=1e-3)
+    from difflut_amd.layers import DWNStack
+    stack = DWNStack(layers).train()  # same layers; bit-planes / tile-major gradients between them
 
     def step():
         opt.zero_grad(set_to_none=True)
         h = enc.encode(x)
-        for layer in layers:
-            h = layer(h)
+        if args.layer_by_layer:
+            for layer in layers:
+                h = layer(h)
+        else:
+            h = stack(h)
         loss = torch.nn.functional.cross_entropy(head(h), labels)
         loss.backward()
         opt.step()
@@ -126,7 +131,8 @@ def run_stack(args):
            "value": evals / (ms * 1e-3), "unit": "node-evals/s", "ms_per_step": ms, "dtype": "f32",
            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
            "vs_baseline": None, "data": "synthetic",
-           "config": {"workload": args.workload, "batch": B, "features": F, "layers": widths, "k": k},
+           "config": {"workload": args.workload, "batch": B, "features": F, "layers": widths, "k": k,
+                      "execution": "layer by layer" if args.layer_by_layer else "chained (DWNStack)"},
            "kernel_ms": kernel_times(step, min(args.steps, 5))}
     print(json.dumps(out))
 
@@ -208,6 +214,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=4096, help="batch rows of the workload the CPU baseline runs")
     ap.add_argument("--precision", type=int, default=0, help="soft-connectivity workload: 0 fp32, 1 bf16 operands")
+    ap.add_argument("--layer-by-layer", action="store_true", help="stack workload: call the layers one by one")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no collective); run with --gpus 1",

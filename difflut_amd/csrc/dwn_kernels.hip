@@ -103,9 +103,10 @@ __global__ __launch_bounds__(256) void dwn_pack_planes(const float *__restrict__
 template <int K, bool O1>
 __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restrict__ planes, const int *__restrict__ idx32,
                                                                const float *__restrict__ luts, float *__restrict__ y,
-                                                               uint8_t *__restrict__ addrT, int B, int I, int N, int O,
-                                                               int BT) {
+                                                               uint8_t *__restrict__ addrT, u64 *__restrict__ planes_out,
+                                                               int B, int I, int N, int O, int BT) {
     __shared__ float tile[DWN_TC][65];  // [column][row]
+    __shared__ u64 plane_tile[DWN_TC];  // thresholded outputs of the tile's columns, one bit per row
     constexpr int L = 1 << K;
     constexpr int NIDX = (DWN_WC * K + 63) / 64;  // index registers per lane
     const int NO = N * O;
@@ -159,6 +160,10 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
                 const float v = dl_lane_read(entry[q], (int)addr);
                 if (cc < cend) {
                     tile[cc][lane] = v;
+                    if (planes_out) {  // the next layer's view of this column: bit r = (y[64t+r][c] >= 0.5)
+                        const u64 m = __ballot(v >= 0.5f);
+                        if (lane == 0) plane_tile[cc] = m;
+                    }
                     const int c = c0 + cc;
                     const int n = O1 ? c : c / O;
                     if (O1 || c - n * O == 0) __builtin_amdgcn_raw_buffer_store_b8((uint8_t)addr, rs_addr, lane, n * 64, 0);
@@ -167,6 +172,12 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
         }
     }
     __syncthreads();
+    if (planes_out && (int)threadIdx.x < cend) {
+        const int rows = min(64, B - t * 64);  // rows past B read as 0, like the planes packed from x
+        const u64 valid = rows == 64 ? ~0ull : ((1ull << rows) - 1ull);
+        planes_out[(size_t)t * NO + c0 + threadIdx.x] = plane_tile[threadIdx.x] & valid;
+    }
+    if (!y) return;
     for (int e = threadIdx.x; e < 64 * DWN_TC; e += 64 * DWN_FW) {
         const int r = e / DWN_TC, cc = e % DWN_TC;
         const int b = t * 64 + r;
@@ -232,7 +243,9 @@ __device__ __forceinline__ int dwn_quad_xor(int v) {
     constexpr int ctrl = X == 1 ? 0xB1 : (X == 2 ? 0x4E : 0x1B);  // quad_perm [1,0,3,2] / [2,3,0,1] / [3,2,1,0]
     return __builtin_amdgcn_update_dpp(0, v, ctrl, 0xf, 0xf, true);
 }
-template <bool WRITE_T>
+// IN_T: gy arrives tile-major already ([B/64][N*O][64], e.g. the input gradient a following layer
+// wrote in that form); only the histogram is left to do.
+template <bool WRITE_T, bool IN_T = false>
 __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__restrict__ gy, const uint8_t *__restrict__ addrT,
                                                                float *__restrict__ gyT, float *__restrict__ gluts,
                                                                int B, int NO, int O, int L, int BP, int BT,
@@ -253,12 +266,15 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
     const int wc0 = wave * (DWN_HC / 4);  // my wavefront's first column
     float4 pre[4];
     unsigned apre[DWN_HC / 4];  // addresses of my 16 columns for the tile being fetched (lane = row)
+    const int tc = threadIdx.x >> 2, tr = (threadIdx.x & 3) * 16;  // IN_T: my column, my first row
     auto fetch = [&](int t) {
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
             const int b = t * 64 + rr + 16 * p;
             pre[p] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (b < B) {
+            if (IN_T) {
+                if (tc < cend) pre[p] = *reinterpret_cast<const float4 *>(gy + ((size_t)t * NO + c0 + tc) * 64 + tr + 4 * p);
+            } else if (b < B) {
                 const float *src = gy + (size_t)b * NO + c0 + q * 4;
                 if (vec4) {
                     pre[p] = *reinterpret_cast<const float4 *>(src);
@@ -282,8 +298,13 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
         __syncthreads();  // previous tile fully consumed (and hist cleared on the first pass)
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
-            float *dst = &tile[rr + 16 * p][q * 4];
-            dst[0] = pre[p].x; dst[1] = pre[p].y; dst[2] = pre[p].z; dst[3] = pre[p].w;
+            if (IN_T) {
+                tile[tr + 4 * p][tc] = pre[p].x; tile[tr + 4 * p + 1][tc] = pre[p].y;
+                tile[tr + 4 * p + 2][tc] = pre[p].z; tile[tr + 4 * p + 3][tc] = pre[p].w;
+            } else {
+                float *dst = &tile[rr + 16 * p][q * 4];
+                dst[0] = pre[p].x; dst[1] = pre[p].y; dst[2] = pre[p].z; dst[3] = pre[p].w;
+            }
         }
 #pragma unroll
         for (int u = 0; u < DWN_HC / 4; ++u) atile[wc0 + u][lane] = (uint8_t)apre[u];
@@ -332,7 +353,7 @@ template <int K, bool O1, bool SFORM>
 __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT, const uint8_t *__restrict__ addrT,
                                                    const float *__restrict__ D, const int *__restrict__ inv_ptr,
                                                    const int *__restrict__ inv_pos, float *__restrict__ gx,
-                                                   int B, int I, int N, int O, int BT) {
+                                                   int B, int I, int N, int O, int BT, int out_tiled) {
     __shared__ float tile[DWN_IS][65];  // [input][row]
     constexpr int Lh = 1 << (K - 1);
     int slab, t;
@@ -436,6 +457,15 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT,
         }
     }
     if (cur >= 0) tile[wbeg + cur][lane] = acc;
+    if (out_tiled) {
+        // gx as [B/64][I][64] for a preceding layer that takes its gy in that form: my 16 inputs, 256 B each
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int r = 0; r < DWN_WI; ++r)
+            if (wbeg + r < iend) gx[((size_t)t * I + i0 + wbeg + r) * 64 + lane] = tile[wbeg + r][lane];
+        return;
+    }
     __syncthreads();
     for (int e = threadIdx.x; e < 64 * DWN_IS; e += 256) {
         const int r = e / DWN_IS, ii = e % DWN_IS;
@@ -483,15 +513,17 @@ extern "C" size_t dl_dwn_bwd_workspace_bytes(int B, int I, int N, int k, int O) 
 
 template <int K>
 static void dwn_launch_lookup(const u64 *planes, const int *idx32, const float *luts, float *y, uint8_t *addrT,
-                              int B, int I, int N, int O, hipStream_t s) {
+                              u64 *planes_out, int B, int I, int N, int O, hipStream_t s) {
     const int BT = dwn_bt(B);
     const int grid = dl_xcd_grid(dl_ceil_div((long long)N * O, DWN_TC), BT);
     if (O == 1)
         DL_TIMED("dwn_lookup_fwd", s,
-                 (dwn_lookup_fwd<K, true><<<grid, 64 * DWN_FW, 0, s>>>(planes, idx32, luts, y, addrT, B, I, N, O, BT)));
+                 (dwn_lookup_fwd<K, true><<<grid, 64 * DWN_FW, 0, s>>>(planes, idx32, luts, y, addrT, planes_out, B, I, N, O,
+                                                                      BT)));
     else
         DL_TIMED("dwn_lookup_fwd", s,
-                 (dwn_lookup_fwd<K, false><<<grid, 64 * DWN_FW, 0, s>>>(planes, idx32, luts, y, addrT, B, I, N, O, BT)));
+                 (dwn_lookup_fwd<K, false><<<grid, 64 * DWN_FW, 0, s>>>(planes, idx32, luts, y, addrT, planes_out, B, I, N, O,
+                                                                       BT)));
 }
 
 extern "C" int dl_dwn_layer_fwd(const float *x, const int32_t *idx32, const float *luts, float *y, void *saved,
@@ -511,23 +543,23 @@ extern "C" int dl_dwn_layer_fwd(const float *x, const int32_t *idx32, const floa
         DL_TIMED("dwn_pack_planes", s, (dwn_pack_planes<1><<<dim3(dl_ceil_div(I, 256), BT), 256, 0, s>>>(x, planes, B, I)));
     uint8_t *addrT = (uint8_t *)saved;
     switch (k) {
-        case 1: dwn_launch_lookup<1>(planes, idx32, luts, y, addrT, B, I, N, O, s); break;
-        case 2: dwn_launch_lookup<2>(planes, idx32, luts, y, addrT, B, I, N, O, s); break;
-        case 3: dwn_launch_lookup<3>(planes, idx32, luts, y, addrT, B, I, N, O, s); break;
-        case 4: dwn_launch_lookup<4>(planes, idx32, luts, y, addrT, B, I, N, O, s); break;
-        case 5: dwn_launch_lookup<5>(planes, idx32, luts, y, addrT, B, I, N, O, s); break;
-        default: dwn_launch_lookup<6>(planes, idx32, luts, y, addrT, B, I, N, O, s); break;
+        case 1: dwn_launch_lookup<1>(planes, idx32, luts, y, addrT, nullptr, B, I, N, O, s); break;
+        case 2: dwn_launch_lookup<2>(planes, idx32, luts, y, addrT, nullptr, B, I, N, O, s); break;
+        case 3: dwn_launch_lookup<3>(planes, idx32, luts, y, addrT, nullptr, B, I, N, O, s); break;
+        case 4: dwn_launch_lookup<4>(planes, idx32, luts, y, addrT, nullptr, B, I, N, O, s); break;
+        case 5: dwn_launch_lookup<5>(planes, idx32, luts, y, addrT, nullptr, B, I, N, O, s); break;
+        default: dwn_launch_lookup<6>(planes, idx32, luts, y, addrT, nullptr, B, I, N, O, s); break;
     }
     return dl_launch_status();
 }
 
 template <int K>
 static void dwn_launch_gx(const float *gyT, const uint8_t *addrT, const float *D, const int *inv_ptr, const int *inv_pos,
-                          float *gx, int B, int I, int N, int O, bool sform, hipStream_t s) {
+                          float *gx, int B, int I, int N, int O, bool sform, int out_tiled, hipStream_t s) {
     const int BT = dwn_bt(B);
     const int grid = dl_xcd_grid(dl_ceil_div(I, DWN_IS), BT);
 #define DWN_GX(O1_, S_) \
-    DL_TIMED("dwn_bwd_gx", s, (dwn_bwd_gx<K, O1_, S_><<<grid, 256, 0, s>>>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, BT)))
+    DL_TIMED("dwn_bwd_gx", s, (dwn_bwd_gx<K, O1_, S_><<<grid, 256, 0, s>>>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, BT, out_tiled)))
     if (O == 1 && sform) DWN_GX(true, true);
     else if (O == 1) DWN_GX(true, false);
     else if (sform) DWN_GX(false, true);
@@ -535,23 +567,13 @@ static void dwn_launch_gx(const float *gyT, const uint8_t *addrT, const float *D
 #undef DWN_GX
 }
 
-extern "C" int dl_dwn_layer_bwd(const float *x, const void *saved, const int32_t *idx32, const int32_t *inv_ptr,
-                                const int32_t *inv_pos, const float *luts, const float *gy, float alpha, float beta,
-                                float *gx, float *gluts, void *ws, size_t ws_bytes, int B, int I, int N, int k, int O,
-                                void *stream) {
-    if (!idx32 || !luts || !gy || !gluts) return DL_ERR_NULL;
-    if (gx && (!inv_ptr || !inv_pos)) return DL_ERR_NULL;
-    int rc = dwn_check(B, I, N, k, O);
-    if (rc) return rc;
-    hipStream_t s = (hipStream_t)stream;
+// backward of the k <= 6 path; gy row-major [B, N*O] or (gy_tiled) tile-major [B/64][N*O][64];
+// gx row-major [B, I] or (gx_tiled) tile-major [B/64][I][64]
+static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos, const float *luts,
+                             const float *gy, int gy_tiled, float alpha, float beta, float *gx, int gx_tiled,
+                             float *gluts, void *ws, int B, int I, int N, int k, int O, hipStream_t s) {
     const long long NO = (long long)N * O;
     const int L = 1 << k;
-    if (!dwn_fast(N, k, O)) {
-        if (!x) return DL_ERR_NULL;
-        return dwn_generic_backward(x, idx32, inv_ptr, inv_pos, luts, gy, alpha, beta, gx, gluts, B, I, N, k, O, s);
-    }
-    if (!saved || !ws) return DL_ERR_NULL;
-    if (ws_bytes < dl_dwn_bwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
     const uint8_t *addrT = (const uint8_t *)saved;
     float *D = (float *)ws;
     float *gyT = (float *)((char *)ws + dwn_table_bytes(N, k, O));
@@ -563,24 +585,104 @@ extern "C" int dl_dwn_layer_bwd(const float *x, const void *saved, const int32_t
     if (chunks > BT) chunks = BT;
     const int tpc = dl_ceil_div(BT, chunks);
     chunks = dl_ceil_div(BT, tpc);
-    if (gx) {
-        const bool sform = beta >= -0.5f && beta <= 0.5f;
+    const dim3 hgrid(col_tiles, chunks);
+    const bool sform = beta >= -0.5f && beta <= 0.5f;
+    if (gx)
         DL_TIMED("dwn_efd_table", s,
                  (dwn_efd_table<<<dl_ceil_div(NO, 4), 256, 0, s>>>(luts, D, gluts, (int)NO, k, alpha, beta, sform ? 1 : 0)));
-        DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<true><<<dim3(col_tiles, chunks), 256, 0, s>>>(
-                                                  gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc)));
-        switch (k) {
-            case 1: dwn_launch_gx<1>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, s); break;
-            case 2: dwn_launch_gx<2>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, s); break;
-            case 3: dwn_launch_gx<3>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, s); break;
-            case 4: dwn_launch_gx<4>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, s); break;
-            case 5: dwn_launch_gx<5>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, s); break;
-            default: dwn_launch_gx<6>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, s); break;
-        }
-    } else {
+    else
         dl_fill_zero(gluts, NO * L, s);
-        DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<false><<<dim3(col_tiles, chunks), 256, 0, s>>>(
+    if (gy_tiled)
+        DL_TIMED("dwn_bwd_hist_tiled", s, (dwn_bwd_transpose_hist<false, true><<<hgrid, 256, 0, s>>>(
+                                              gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc)));
+    else if (gx)
+        DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<true><<<hgrid, 256, 0, s>>>(
                                                   gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc)));
+    else
+        DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<false><<<hgrid, 256, 0, s>>>(
+                                                  gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc)));
+    if (gx) {
+        const float *src = gy_tiled ? gy : gyT;
+        switch (k) {
+            case 1: dwn_launch_gx<1>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, s); break;
+            case 2: dwn_launch_gx<2>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, s); break;
+            case 3: dwn_launch_gx<3>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, s); break;
+            case 4: dwn_launch_gx<4>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, s); break;
+            case 5: dwn_launch_gx<5>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, s); break;
+            default: dwn_launch_gx<6>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, s); break;
+        }
     }
     return dl_launch_status();
+}
+
+extern "C" int dl_dwn_layer_bwd(const float *x, const void *saved, const int32_t *idx32, const int32_t *inv_ptr,
+                                const int32_t *inv_pos, const float *luts, const float *gy, float alpha, float beta,
+                                float *gx, float *gluts, void *ws, size_t ws_bytes, int B, int I, int N, int k, int O,
+                                void *stream) {
+    if (!idx32 || !luts || !gy || !gluts) return DL_ERR_NULL;
+    if (gx && (!inv_ptr || !inv_pos)) return DL_ERR_NULL;
+    int rc = dwn_check(B, I, N, k, O);
+    if (rc) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    if (!dwn_fast(N, k, O)) {
+        if (!x) return DL_ERR_NULL;
+        return dwn_generic_backward(x, idx32, inv_ptr, inv_pos, luts, gy, alpha, beta, gx, gluts, B, I, N, k, O, s);
+    }
+    if (!saved || !ws) return DL_ERR_NULL;
+    if (ws_bytes < dl_dwn_bwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
+    return dwn_backward_fast(saved, inv_ptr, inv_pos, luts, gy, 0, alpha, beta, gx, 0, gluts, ws, B, I, N, k, O, s);
+}
+
+// ---------------------------------------------------------------------------------
+// Chained layers: activations between two DWN layers never take their [B, N] fp32 form.
+extern "C" size_t dl_dwn_planes_bytes(int B, int C) { return (B > 0 && C > 0) ? dwn_planes_bytes(B, C) : 256; }
+extern "C" size_t dl_dwn_tiled_bytes(int B, int C) {
+    return (B > 0 && C > 0) ? dl_align256((size_t)dwn_bt(B) * C * 64 * sizeof(float)) : 256;
+}
+
+extern "C" int dl_dwn_pack_planes(const float *x, void *planes, int B, int I, void *stream) {
+    if (!x || !planes) return DL_ERR_NULL;
+    if (B <= 0 || I <= 0) return DL_ERR_SHAPE;
+    hipStream_t s = (hipStream_t)stream;
+    const int BT = dwn_bt(B);
+    if (I % 4 == 0 && ((uintptr_t)x & 15) == 0)
+        DL_TIMED("dwn_pack_planes", s, (dwn_pack_planes<4><<<dim3(dl_ceil_div(I, 1024), BT), 256, 0, s>>>(x, (u64 *)planes, B, I)));
+    else
+        DL_TIMED("dwn_pack_planes", s, (dwn_pack_planes<1><<<dim3(dl_ceil_div(I, 256), BT), 256, 0, s>>>(x, (u64 *)planes, B, I)));
+    return dl_launch_status();
+}
+
+extern "C" int dl_dwn_layer_fwd_planes(const void *planes_in, const int32_t *idx32, const float *luts, float *y,
+                                       void *planes_out, void *saved, int B, int I, int N, int k, int O, void *stream) {
+    if (!planes_in || !idx32 || !luts || !saved || (!y && !planes_out)) return DL_ERR_NULL;
+    int rc = dwn_check(B, I, N, k, O);
+    if (rc) return rc;
+    if (!dwn_fast(N, k, O)) return DL_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+    const u64 *planes = (const u64 *)planes_in;
+    uint8_t *addrT = (uint8_t *)saved;
+    u64 *po = (u64 *)planes_out;
+    switch (k) {
+        case 1: dwn_launch_lookup<1>(planes, idx32, luts, y, addrT, po, B, I, N, O, s); break;
+        case 2: dwn_launch_lookup<2>(planes, idx32, luts, y, addrT, po, B, I, N, O, s); break;
+        case 3: dwn_launch_lookup<3>(planes, idx32, luts, y, addrT, po, B, I, N, O, s); break;
+        case 4: dwn_launch_lookup<4>(planes, idx32, luts, y, addrT, po, B, I, N, O, s); break;
+        case 5: dwn_launch_lookup<5>(planes, idx32, luts, y, addrT, po, B, I, N, O, s); break;
+        default: dwn_launch_lookup<6>(planes, idx32, luts, y, addrT, po, B, I, N, O, s); break;
+    }
+    return dl_launch_status();
+}
+
+extern "C" int dl_dwn_layer_bwd_tiled(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos,
+                                      const float *luts, const float *gy, int gy_tiled, float alpha, float beta,
+                                      float *gx, int gx_tiled, float *gluts, void *ws, size_t ws_bytes, int B, int I, int N,
+                                      int k, int O, void *stream) {
+    if (!saved || !luts || !gy || !gluts || !ws) return DL_ERR_NULL;
+    if (gx && (!inv_ptr || !inv_pos)) return DL_ERR_NULL;
+    int rc = dwn_check(B, I, N, k, O);
+    if (rc) return rc;
+    if (!dwn_fast(N, k, O)) return DL_ERR_UNSUPPORTED;
+    if (ws_bytes < dl_dwn_bwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
+    return dwn_backward_fast(saved, inv_ptr, inv_pos, luts, gy, gy_tiled, alpha, beta, gx, gx_tiled, gluts, ws, B, I, N, k, O,
+                             (hipStream_t)stream);
 }

@@ -132,6 +132,69 @@ class DWNLayerFunction(torch.autograd.Function):
         return gx, gl, None, None, None
 
 
+class DWNStackFunction(torch.autograd.Function):
+    """A chain of RandomLayer + DWN layers in one autograd node.  A following DWN layer only thresholds
+    what it is given, so between layers the activations stay bit-planes and the gradients stay
+    tile-major: no [B, N] fp32 tensor is written or read except the last layer's output (and the
+    first layer's input gradient, if asked for).  Same arithmetic as calling the layers one by one."""
+
+    @staticmethod
+    def forward(ctx, x, plans, scalars, *luts):
+        nat.require_device(x, *luts)
+        x = _f32(x)
+        luts = tuple(_f32(t) for t in luts)
+        B, width = x.shape
+        lib = nat.lib()
+        planes = _bytes(lib.dl_dwn_planes_bytes(B, width), x.device)
+        nat.check(lib.dl_dwn_pack_planes(nat.ptr(x), nat.ptr(planes), B, width, nat.stream()))
+        saved, dims_all, y = [], [], None
+        for l, (plan, lut) in enumerate(zip(plans, luts)):
+            N, O, L = lut.shape
+            k = plan.k
+            if k > FAST_K or (N, 1 << k, width) != (plan.N, L, plan.I):
+                raise RuntimeError(f"layer {l}: cannot chain (k={k}, tables {tuple(lut.shape)}, mapping [{plan.N},{k}] over "
+                                   f"{plan.I} inputs, incoming width {width})")
+            dims = (B, width, N, k, O)
+            last = l == len(plans) - 1
+            keep = _bytes(lib.dl_dwn_saved_bytes(*dims), x.device)
+            y = torch.empty((B, N * O), dtype=torch.float32, device=x.device) if last else None
+            nxt = None if last else _bytes(lib.dl_dwn_planes_bytes(B, N * O), x.device)
+            nat.check(lib.dl_dwn_layer_fwd_planes(nat.ptr(planes), nat.ptr(plan.idx32), nat.ptr(lut), nat.ptr(y),
+                                                  nat.ptr(nxt), nat.ptr(keep), *dims, nat.stream()))
+            saved.append(keep)
+            dims_all.append(dims)
+            planes, width = nxt, N * O
+        ctx.save_for_backward(*luts, *saved)
+        ctx.plans, ctx.scalars, ctx.dims_all = plans, scalars, dims_all
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        n = len(ctx.plans)
+        luts, saved = ctx.saved_tensors[:n], ctx.saved_tensors[n:]
+        lib = nat.lib()
+        g, tiled = _f32(gy), 0
+        grads = [None] * n
+        for l in range(n - 1, -1, -1):
+            B, I, N, k, O = dims = ctx.dims_all[l]
+            plan = ctx.plans[l]
+            alpha, beta = ctx.scalars[l]
+            if l > 0:
+                gx = torch.empty(lib.dl_dwn_tiled_bytes(B, I) // 4, dtype=torch.float32, device=g.device)
+                gx_tiled = 1
+            else:
+                gx = torch.empty((B, I), dtype=torch.float32, device=g.device) if ctx.needs_input_grad[0] else None
+                gx_tiled = 0
+            grads[l] = torch.empty_like(luts[l])
+            ws = _bytes(lib.dl_dwn_bwd_workspace_bytes(*dims), g.device)
+            nat.check(lib.dl_dwn_layer_bwd_tiled(nat.ptr(saved[l]), nat.ptr(plan.inv_ptr), nat.ptr(plan.inv_pos),
+                                                 nat.ptr(luts[l]), nat.ptr(g), tiled, float(alpha), float(beta),
+                                                 nat.ptr(gx), gx_tiled, nat.ptr(grads[l]), nat.ptr(ws), ws.numel(), *dims,
+                                                 nat.stream()))
+            g, tiled = gx, gx_tiled
+        return (g, None, None, *grads)
+
+
 def dwn_layer_eval(x, luts, plan):
     nat.require_device(x, luts)
     x, luts = _f32(x), _f32(luts)

@@ -89,6 +89,25 @@ int dl_dwn_layer_bwd(const float *x, const void *saved, const int32_t *idx32,
                      const float *luts, const float *gy, float alpha, float beta,
                      float *gx, float *gluts, void *ws, size_t ws_bytes,
                      int B, int I, int N, int k, int O, void *stream);
+/* Chained DWN layers.  No counterpart in the reference, which materialises the [B, N] fp32
+ * activations between layers (random_layer.py:306-340 per layer): a following DWN layer only
+ * thresholds them, so layer l can hand layer l+1 its output as bit-planes
+ * ([ceil(B/64)][C] uint64, bit r of word (t, c) = (value[64t+r][c] >= 0.5)), and layer l+1 can hand
+ * back its input gradient tile-major ([ceil(B/64)][C][64] fp32), which is the form the backward
+ * of layer l reads.  k <= DL_MAX_FAST_K only (DL_ERR_UNSUPPORTED otherwise).
+ *   dl_dwn_pack_planes      : x [B,I] fp32 -> planes
+ *   dl_dwn_layer_fwd_planes : planes_in -> y [B,N*O] (nullable) and/or planes_out (nullable); saved as above
+ *   dl_dwn_layer_bwd_tiled  : gy row-major [B,N*O] or (gy_tiled) tile-major; gx (nullable) row-major
+ *                             [B,I] or (gx_tiled) tile-major; workspace dl_dwn_bwd_workspace_bytes */
+size_t dl_dwn_planes_bytes(int B, int C);
+size_t dl_dwn_tiled_bytes(int B, int C);
+int dl_dwn_pack_planes(const float *x, void *planes, int B, int I, void *stream);
+int dl_dwn_layer_fwd_planes(const void *planes_in, const int32_t *idx32, const float *luts, float *y,
+                            void *planes_out, void *saved, int B, int I, int N, int k, int O, void *stream);
+int dl_dwn_layer_bwd_tiled(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos,
+                           const float *luts, const float *gy, int gy_tiled, float alpha, float beta,
+                           float *gx, int gx_tiled, float *gluts, void *ws, size_t ws_bytes,
+                           int B, int I, int N, int k, int O, void *stream);
 /* Eval forward (DWNNode.forward_eval, dwn_node.py:457-483): addr = floor(sum_j x_j 2^j)
  * with no thresholding of x (clamped to the table), y = (luts[n,d,addr] >= 0.5) as 0/1. */
 int dl_dwn_layer_eval(const float *x, const int32_t *idx32, const float *luts, float *y,

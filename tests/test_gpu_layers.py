@@ -319,6 +319,53 @@ def test_full_size_soft_mapping_b512_i3136_m48000(precision):
             assert float((got.double() - want).abs().max()) <= 1e-2 * float(want.abs().max())
 
 
+@pytest.mark.parametrize("shape", [((70, 50), [40, 33, 20], 6), ((130, 64), [128, 64], 4), ((64, 30), [25], 3),
+                                   ((200, 96), [300, 150, 75, 10], 6)])
+@pytest.mark.parametrize("input_grad", [True, False])
+def test_dwn_stack_equals_layer_by_layer(shape, input_grad):
+    """Chained execution (bit-planes forward, tile-major gradients backward) against the same layers
+    called one after the other: outputs bit-exact, gradients to rtol 1e-5 (same kernels, same
+    summation orders; only the layouts between the layers differ)."""
+    REGISTRY, NodeConfig, uniform_init, _ = _api()
+    from difflut_amd.layers import DWNStack
+    (B, I), widths, k = shape
+    torch.manual_seed(sum(widths) + B)
+    layers, width = [], I
+    for li, n in enumerate(widths):
+        layers.append(REGISTRY.get_layer("random")(width, n, REGISTRY.get_node("dwn"),
+                                                   NodeConfig(input_dim=k, output_dim=1, init_fn=uniform_init,
+                                                              init_kwargs={"a": -1.0, "b": 2.0}), seed=li + 3).cuda())
+        width = n
+    x = torch.rand(B, I, device="cuda")
+    gy = torch.randn(B, widths[-1], device="cuda")
+    xa = x.clone().requires_grad_(input_grad)
+    h = xa
+    for layer in layers:
+        h = layer(h)
+    h.backward(gy)
+    want_y = h.detach().clone()
+    want_gl = [layer._banks["luts"].flat.grad.clone() for layer in layers]
+    want_gx = xa.grad.clone() if input_grad else None
+    for layer in layers:
+        layer._banks["luts"].flat.grad = None
+    stack = DWNStack(layers).train()
+    xb = x.clone().requires_grad_(input_grad)
+    y = stack(xb)
+    assert torch.equal(y.detach(), want_y)
+    y.backward(gy)
+    for layer, want in zip(layers, want_gl):
+        torch.testing.assert_close(layer._banks["luts"].flat.grad, want, rtol=1e-5, atol=1e-6)
+    if input_grad:
+        torch.testing.assert_close(xb.grad, want_gx, rtol=1e-5, atol=2e-6)
+    # eval mode and non-chainable members fall back to the members' own forward
+    stack.eval()
+    he = x
+    for layer in layers:
+        layer.eval()
+        he = layer(he)
+    assert torch.equal(stack(x), he)
+
+
 def test_legacy_extension_names_and_signatures(golden):
     """tests/test_layers/test_fused_kernels.py:159-179 imports efd_cuda / efd_fused_cuda by bare name;
     the shims answer with the reference's signatures."""
