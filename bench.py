@@ -127,12 +127,19 @@ def run_stack(args):
 
     ms = time_steps(step, args.steps, args.warmup)
     evals = B * sum(widths)
+    # compulsory fp32 traffic of the layer-by-layer formulation: per layer x and y forward, gy, x and gx
+    # backward (no gx for the first layer), plus nine passes over the tables (forward, backward, gradient, Adam)
+    ins = [F * 4] + widths[:-1]
+    nbytes = sum(4 * B * (2 * i + 2 * n + (i if li else 0)) for li, (i, n) in enumerate(zip(ins, widths)))
+    nbytes += 9 * sum(widths) * (1 << k) * 4
     out = {"metric": "LUT-node evals/sec, training step (thermometer -> 4 DWN k=6 layers -> GroupSum -> CE, Adam)",
            "value": evals / (ms * 1e-3), "unit": "node-evals/s", "ms_per_step": ms, "dtype": "f32",
            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
            "vs_baseline": None, "data": "synthetic",
            "config": {"workload": args.workload, "batch": B, "features": F, "layers": widths, "k": k,
                       "execution": "layer by layer" if args.layer_by_layer else "chained (DWNStack)"},
+           "roofline_step": {"bound": "hbm", "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes_per_step": nbytes},
            "kernel_ms": kernel_times(step, min(args.steps, 5))}
     print(json.dumps(out))
 
