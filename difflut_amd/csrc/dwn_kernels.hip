@@ -100,13 +100,14 @@ __global__ __launch_bounds__(256) void dwn_pack_planes(const float *__restrict__
 #define DWN_FW 8                      // wavefronts per block
 #define DWN_WC (DWN_TC / DWN_FW)      // columns per wavefront
 #define DWN_CG 4                      // columns per group
-template <int K, bool O1>
+// CHAIN: the variant for chained layers, which can also (or only) emit the columns as bit-planes.
+template <int K, bool O1, bool CHAIN = false>
 __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restrict__ planes, const int *__restrict__ idx32,
                                                                const float *__restrict__ luts, float *__restrict__ y,
                                                                uint8_t *__restrict__ addrT, u64 *__restrict__ planes_out,
                                                                int B, int I, int N, int O, int BT) {
     __shared__ float tile[DWN_TC][65];  // [column][row]
-    __shared__ u64 plane_tile[DWN_TC];  // thresholded outputs of the tile's columns, one bit per row
+    __shared__ u64 plane_tile[CHAIN ? DWN_TC : 1];  // thresholded outputs of the tile's columns, one bit per row
     constexpr int L = 1 << K;
     constexpr int NIDX = (DWN_WC * K + 63) / 64;  // index registers per lane
     const int NO = N * O;
@@ -160,7 +161,7 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
                 const float v = dl_lane_read(entry[q], (int)addr);
                 if (cc < cend) {
                     tile[cc][lane] = v;
-                    if (planes_out) {  // the next layer's view of this column: bit r = (y[64t+r][c] >= 0.5)
+                    if (CHAIN && planes_out) {  // the next layer's view of this column: bit r = (y[64t+r][c] >= 0.5)
                         const u64 m = __ballot(v >= 0.5f);
                         if (lane == 0) plane_tile[cc] = m;
                     }
@@ -172,12 +173,12 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
         }
     }
     __syncthreads();
-    if (planes_out && (int)threadIdx.x < cend) {
+    if (CHAIN && planes_out && (int)threadIdx.x < cend) {
         const int rows = min(64, B - t * 64);  // rows past B read as 0, like the planes packed from x
         const u64 valid = rows == 64 ? ~0ull : ((1ull << rows) - 1ull);
         planes_out[(size_t)t * NO + c0 + threadIdx.x] = plane_tile[threadIdx.x] & valid;
     }
-    if (!y) return;
+    if (CHAIN && !y) return;
     for (int e = threadIdx.x; e < 64 * DWN_TC; e += 64 * DWN_FW) {
         const int r = e / DWN_TC, cc = e % DWN_TC;
         const int b = t * 64 + r;
@@ -516,14 +517,16 @@ static void dwn_launch_lookup(const u64 *planes, const int *idx32, const float *
                               u64 *planes_out, int B, int I, int N, int O, hipStream_t s) {
     const int BT = dwn_bt(B);
     const int grid = dl_xcd_grid(dl_ceil_div((long long)N * O, DWN_TC), BT);
-    if (O == 1)
-        DL_TIMED("dwn_lookup_fwd", s,
-                 (dwn_lookup_fwd<K, true><<<grid, 64 * DWN_FW, 0, s>>>(planes, idx32, luts, y, addrT, planes_out, B, I, N, O,
-                                                                      BT)));
-    else
-        DL_TIMED("dwn_lookup_fwd", s,
-                 (dwn_lookup_fwd<K, false><<<grid, 64 * DWN_FW, 0, s>>>(planes, idx32, luts, y, addrT, planes_out, B, I, N, O,
-                                                                       BT)));
+#define DWN_LOOKUP(O1_, CHAIN_)                                                                                        \
+    DL_TIMED("dwn_lookup_fwd", s,                                                                                      \
+             (dwn_lookup_fwd<K, O1_, CHAIN_><<<grid, 64 * DWN_FW, 0, s>>>(planes, idx32, luts, y, addrT, planes_out, B, I, \
+                                                                         N, O, BT)))
+    const bool chain = planes_out != nullptr || y == nullptr;
+    if (O == 1 && !chain) DWN_LOOKUP(true, false);
+    else if (O == 1) DWN_LOOKUP(true, true);
+    else if (!chain) DWN_LOOKUP(false, false);
+    else DWN_LOOKUP(false, true);
+#undef DWN_LOOKUP
 }
 
 extern "C" int dl_dwn_layer_fwd(const float *x, const int32_t *idx32, const float *luts, float *y, void *saved,
