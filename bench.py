@@ -41,7 +41,7 @@ WORKLOADS = {
     # secondary workloads of the same path, reported with their own metric names (see run_secondary)
     "prob_k4_b1024_i4096_n4096": (1024, 4096, 4096, 4, 1),
     "softmap_b512_i3136_m48000": (512, 3136, 8000, 6, 1),
-    # whole training step through the layer API (BASELINE configs[4]): (B, features, first layer width, k, O)
+    # whole training step of the deep stack through the layer API: (B, features, first layer width, k, O)
     "dwn_stack_b8192_train_step": (8192, 784, 16000, 6, 1),
 }
 
@@ -145,7 +145,7 @@ def run_stack(args):
 
 
 def run_secondary(args):
-    """Probabilistic layer (BASELINE configs[1]) and soft connectivity (configs[3]) through the C ABI."""
+    """Probabilistic layer (k=4, 1024 x 4096 -> 4096 nodes) and soft connectivity (512 x 3136 -> 48000 rows) through the C ABI."""
     from difflut_amd import _native as nat
     from difflut_amd import ops
     from oracle import difflut_oracle as orc

@@ -259,7 +259,7 @@ def test_full_size_properties_dwn_k6_b4096_n8192():
 
 
 def test_full_size_probabilistic_k4_b1024_n4096():
-    """BASELINE configs[1] shape against a float64 torch restatement of the same fold (the checker runs on
+    """The probabilistic benchmark shape against a float64 torch restatement of the same fold (the checker runs on
     the GPU; the first nodes also go through the numpy oracle)."""
     from difflut_amd import ops
     torch.manual_seed(1)
@@ -296,7 +296,7 @@ def test_full_size_probabilistic_k4_b1024_n4096():
 
 @pytest.mark.parametrize("precision", [0, 1])
 def test_full_size_soft_mapping_b512_i3136_m48000(precision):
-    """BASELINE configs[3] shape against float64 torch autograd of softmax + matmul (learnable_layer.py:254-255).
+    """The soft-connectivity benchmark shape against float64 torch autograd of softmax + matmul (learnable_layer.py:254-255).
     fp32 operands: rtol 1e-4 on sums of 3136 .. 48000 terms; bf16 operands: 1e-2 of the tensor's largest value."""
     from difflut_amd import ops
     torch.manual_seed(2)
