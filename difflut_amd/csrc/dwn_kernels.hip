@@ -406,7 +406,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT,
                     if (SFORM)
                         G.coef[q] = D[(size_t)rn * (2 * Lh) + (lane & (2 * Lh - 1))];
                     else
-                        G.coef[q] = __builtin_nontemporal_load(&D[((size_t)rn * K + G.rj[q]) * Lh + (lane & (Lh - 1))]);
+                        G.coef[q] = D[((size_t)rn * K + G.rj[q]) * Lh + (lane & (Lh - 1))];
                 } else {
                     G.g[q] = __int_as_float(rn);  // node number; outputs are walked in evaluate()
                 }
