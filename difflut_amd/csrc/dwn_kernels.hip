@@ -267,14 +267,15 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
     const int wc0 = wave * (DWN_HC / 4);  // my wavefront's first column
     float4 pre[4];
     unsigned apre[DWN_HC / 4];  // addresses of my 16 columns for the tile being fetched (lane = row)
-    const int tc = threadIdx.x >> 2, tr = (threadIdx.x & 3) * 16;  // IN_T: my column, my first row
+    const int tc = threadIdx.x >> 4, tr = (threadIdx.x & 15) * 4;  // IN_T: my column in a pass of 16, my 4 rows
     auto fetch = [&](int t) {
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
             const int b = t * 64 + rr + 16 * p;
             pre[p] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (IN_T) {
-                if (tc < cend) pre[p] = *reinterpret_cast<const float4 *>(gy + ((size_t)t * NO + c0 + tc) * 64 + tr + 4 * p);
+            if (IN_T) {  // 16 threads x 16 B = the 256 contiguous bytes of one column
+                if (tc + 16 * p < cend)
+                    pre[p] = *reinterpret_cast<const float4 *>(gy + ((size_t)t * NO + c0 + tc + 16 * p) * 64 + tr);
             } else if (b < B) {
                 const float *src = gy + (size_t)b * NO + c0 + q * 4;
                 if (vec4) {
@@ -300,8 +301,8 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
             if (IN_T) {
-                tile[tr + 4 * p][tc] = pre[p].x; tile[tr + 4 * p + 1][tc] = pre[p].y;
-                tile[tr + 4 * p + 2][tc] = pre[p].z; tile[tr + 4 * p + 3][tc] = pre[p].w;
+                tile[tr][tc + 16 * p] = pre[p].x; tile[tr + 1][tc + 16 * p] = pre[p].y;
+                tile[tr + 2][tc + 16 * p] = pre[p].z; tile[tr + 3][tc + 16 * p] = pre[p].w;
             } else {
                 float *dst = &tile[rr + 16 * p][q * 4];
                 dst[0] = pre[p].x; dst[1] = pre[p].y; dst[2] = pre[p].z; dst[3] = pre[p].w;
