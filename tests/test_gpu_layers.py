@@ -366,6 +366,49 @@ def test_dwn_stack_equals_layer_by_layer(shape, input_grad):
     assert torch.equal(stack(x), he)
 
 
+def test_dwn_layer_step_replays_from_a_hip_graph():
+    """The library never allocates or synchronises, and clears buffers with kernels, so a forward +
+    backward can be captured once and replayed; every replay is checked against an eager run on
+    the same inputs (eager work and synchronisations in between)."""
+    from difflut_amd import ops
+    torch.manual_seed(5)
+    B, I, N, k = 192, 96, 80, 6
+    idx = orc.random_mapping(I, N, k, seed=7)
+    plan = ops.MappingPlan(idx.cuda(), I)
+    alpha, beta = 0.5 * 0.75 ** 5, 1 / 3
+    x = torch.rand(B, I, device="cuda").requires_grad_()
+    luts = (torch.rand(N, 1, 64, device="cuda") * 2 - 1).requires_grad_()
+    gy = torch.randn(B, N, device="cuda")
+
+    def eager(xv, lv, gv):
+        xa, la = xv.clone().requires_grad_(), lv.clone().requires_grad_()
+        y = ops.DWNLayerFunction.apply(xa, la, plan, alpha, beta)
+        y.backward(gv)
+        return y.detach(), xa.grad, la.grad
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up outside the capture
+        for _ in range(2):
+            y = ops.DWNLayerFunction.apply(x, luts, plan, alpha, beta)
+            gxs, gls = torch.autograd.grad(y, (x, luts), gy)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = ops.DWNLayerFunction.apply(x, luts, plan, alpha, beta)
+        gxs, gls = torch.autograd.grad(y, (x, luts), gy)
+    for rep in range(3):
+        with torch.no_grad():
+            x.copy_(torch.rand(B, I, device="cuda"))
+            luts.copy_(torch.rand(N, 1, 64, device="cuda") * 2 - 1)
+            gy.copy_(torch.randn(B, N, device="cuda"))
+        graph.replay()
+        torch.cuda.synchronize()
+        wy, wgx, wgl = eager(x.detach(), luts.detach(), gy)
+        assert torch.equal(y, wy) and torch.equal(gxs, wgx)
+        torch.testing.assert_close(gls, wgl, rtol=1e-5, atol=1e-6)  # float atomics: order may differ
+
+
 def test_legacy_extension_names_and_signatures(golden):
     """tests/test_layers/test_fused_kernels.py:159-179 imports efd_cuda / efd_fused_cuda by bare name;
     the shims answer with the reference's signatures."""
