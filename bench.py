@@ -41,6 +41,9 @@ WORKLOADS = {
     # secondary workloads of the same path, reported with their own metric names (see run_secondary)
     "prob_k4_b1024_i4096_n4096": (1024, 4096, 4096, 4, 1),
     "softmap_b512_i3136_m48000": (512, 3136, 8000, 6, 1),
+    # the headline layer shape with the two other table-lookup node types
+    "stable_k6_b4096_i16384_n8192": (4096, 16384, 8192, 6, 1),
+    "hybrid_k6_b4096_i16384_n8192": (4096, 16384, 8192, 6, 1),
     # whole training step of the deep stack through the layer API: (B, features, first layer width, k, O)
     "dwn_stack_b8192_train_step": (8192, 784, 16000, 6, 1),
 }
@@ -145,7 +148,8 @@ def run_stack(args):
 
 
 def run_secondary(args):
-    """Probabilistic layer (k=4, 1024 x 4096 -> 4096 nodes) and soft connectivity (512 x 3136 -> 48000 rows) through the C ABI."""
+    """Probabilistic layer (k=4, 1024 x 4096 -> 4096 nodes), DWN-stable and hybrid layers at the headline shape, and
+    soft connectivity (512 x 3136 -> 48000 rows), all through the C ABI."""
     from difflut_amd import _native as nat
     from difflut_amd import ops
     from oracle import difflut_oracle as orc
@@ -181,6 +185,45 @@ def run_secondary(args):
                                  "unit": "GB/s", "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                                  "algorithmic_bytes_per_step": nbytes},
                "valu": {"achieved_tflops": flops / (ms * 1e-3) / 1e12, "peak_tflops": 157.3}}
+    elif args.workload.startswith(("stable", "hybrid")):
+        stable = args.workload.startswith("stable")
+        dims = (B, I, N, k, O)
+        count = N * O * (1 << k)
+        x = torch.rand(B, I, device=dev)  # real-valued: the hybrid backward differentiates at x itself
+        plan = ops.MappingPlan(orc.random_mapping(I, N, k, seed=42).to(dev), I)
+        raw = torch.randn(N, O, 1 << k, device=dev)
+        scale = torch.full((N,), 1.25, device=dev)
+        gy = torch.randn(B, N * O, device=dev)
+        luts = torch.empty_like(raw); gl = torch.empty_like(raw); graw = torch.empty_like(raw)
+        y = torch.empty(B, N * O, device=dev); gx = torch.empty(B, I, device=dev)
+        saved = torch.empty(lib.dl_dwn_saved_bytes(*dims), dtype=torch.uint8, device=dev)
+        ws = torch.empty(max(lib.dl_dwn_fwd_workspace_bytes(*dims), lib.dl_dwn_bwd_workspace_bytes(*dims),
+                             lib.dl_hybrid_bwd_workspace_bytes(*dims)), dtype=torch.uint8, device=dev)
+
+        def step():
+            nat.check(lib.dl_table_sigmoid_fwd(raw.data_ptr(), luts.data_ptr(), count, stream))
+            nat.check(lib.dl_dwn_layer_fwd(x.data_ptr(), plan.idx32.data_ptr(), luts.data_ptr(), y.data_ptr(),
+                                           saved.data_ptr(), ws.data_ptr(), ws.numel(), *dims, stream))
+            if stable:
+                nat.check(lib.dl_dwn_stable_layer_bwd(None, saved.data_ptr(), plan.idx32.data_ptr(), plan.inv_ptr.data_ptr(),
+                                                      plan.inv_pos.data_ptr(), luts.data_ptr(), gy.data_ptr(),
+                                                      scale.data_ptr(), gx.data_ptr(), gl.data_ptr(), ws.data_ptr(),
+                                                      ws.numel(), *dims, stream))
+            else:
+                nat.check(lib.dl_hybrid_layer_bwd(x.data_ptr(), plan.idx32.data_ptr(), plan.inv_ptr.data_ptr(),
+                                                  plan.inv_pos.data_ptr(), luts.data_ptr(), gy.data_ptr(), gx.data_ptr(),
+                                                  gl.data_ptr(), ws.data_ptr(), ws.numel(), *dims, stream))
+            nat.check(lib.dl_table_sigmoid_bwd(gl.data_ptr(), luts.data_ptr(), graw.data_ptr(), count, stream))
+
+        ms = time_steps(step, args.steps, args.warmup)
+        fwd_b, bwd_b, _ = algorithmic_bytes(B, I, N, k, O)  # same tensors cross HBM as for the DWN node
+        nbytes = fwd_b + bwd_b
+        name = "DWN-stable" if stable else "hybrid"
+        out = {"metric": f"LUT-node evals/sec fwd+bwd ({name} k=6, B=4096, 8192 nodes)", "value": B * N / (ms * 1e-3),
+               "unit": "node-evals/s", "ms_per_step": ms, "dtype": "f32",
+               "roofline_step": {"bound": "hbm", "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
+                                 "unit": "GB/s", "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                 "algorithmic_bytes_per_step": nbytes}}
     else:
         M = N * k
         precision = args.precision

@@ -1,9 +1,10 @@
 // Launchers of the generic (any k) DWN kernels, defined in dwn_generic.hip.
+// scale == null: EFD weights alpha * beta^h; otherwise scale[n] / (h + 1), which also multiplies the table gradient.
 #pragma once
 #include <hip/hip_runtime.h>
 
 int dwn_generic_forward(const float *x, const int *idx32, const float *luts, float *y, int B, int I, int N, int k, int O,
                         hipStream_t s);
 int dwn_generic_backward(const float *x, const int *idx32, const int *inv_ptr, const int *inv_pos, const float *luts,
-                         const float *gy, float alpha, float beta, float *gx, float *gluts, int B, int I, int N, int k,
-                         int O, hipStream_t s);
+                         const float *gy, float alpha, float beta, const float *scale, float *gx, float *gluts, int B, int I,
+                         int N, int k, int O, hipStream_t s);

@@ -27,15 +27,15 @@ __global__ __launch_bounds__(256) void dwn_generic_fwd(const float *__restrict__
 __global__ __launch_bounds__(256) void dwn_generic_bwd_gx(const float *__restrict__ x, const int *__restrict__ idx32,
                                                            const int *__restrict__ inv_ptr, const int *__restrict__ inv_pos,
                                                            const float *__restrict__ luts, const float *__restrict__ gy,
-                                                           float alpha, float beta, float *__restrict__ gx,
-                                                           int B, int I, int N, int K, int O) {
+                                                           float alpha, float beta, const float *__restrict__ scale,
+                                                           float *__restrict__ gx, int B, int I, int N, int K, int O) {
     const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
     if (gid >= (long long)B * I) return;
     const int b = (int)(gid / I), i = (int)(gid % I);
     const int L = 1 << K;
     double bp[DL_MAX_K + 1];
     bp[0] = 1.0;
-    for (int h = 1; h <= K; ++h) bp[h] = bp[h - 1] * (double)beta;
+    for (int h = 1; h <= K; ++h) bp[h] = scale ? 1.0 / (double)(h + 1) : bp[h - 1] * (double)beta;
     float acc = 0.0f;
     for (int e = inv_ptr[i]; e < inv_ptr[i + 1]; ++e) {
         const int p = inv_pos[e];
@@ -49,15 +49,15 @@ __global__ __launch_bounds__(256) void dwn_generic_bwd_gx(const float *__restric
                 const double w = bp[__popc((a ^ (unsigned)kap) & keep)];
                 s += (((unsigned)kap >> j) & 1u) ? (double)lut[kap] * w : -(double)lut[kap] * w;
             }
-            acc += gy[((size_t)b * N + n) * O + d] * (float)((double)alpha * s);
+            acc += gy[((size_t)b * N + n) * O + d] * (float)((scale ? (double)scale[n] : (double)alpha) * s);
         }
     }
     gx[gid] = acc;
 }
 
 __global__ __launch_bounds__(256) void dwn_generic_bwd_luts(const float *__restrict__ x, const int *__restrict__ idx32,
-                                                             const float *__restrict__ gy, float *__restrict__ gluts,
-                                                             int B, int I, int N, int K, int O) {
+                                                             const float *__restrict__ gy, const float *__restrict__ scale,
+                                                             float *__restrict__ gluts, int B, int I, int N, int K, int O) {
     const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
     const long long NO = (long long)N * O;
     if (gid >= (long long)B * NO) return;
@@ -65,7 +65,7 @@ __global__ __launch_bounds__(256) void dwn_generic_bwd_luts(const float *__restr
     const long long c = gid % NO;
     const int n = (int)(c / O);
     const unsigned a = dwn_addr_generic(x + (size_t)b * I, idx32 + (size_t)n * K, K);
-    atomicAdd(&gluts[(c << K) + a], gy[gid]);
+    atomicAdd(&gluts[(c << K) + a], scale ? gy[gid] * scale[n] : gy[gid]);
 }
 
 // Eval: address = floor(sum_j x_j 2^j), no thresholding of x; table value binarised at 0.5.
@@ -99,14 +99,14 @@ int dwn_generic_forward(const float *x, const int *idx32, const float *luts, flo
 }
 
 int dwn_generic_backward(const float *x, const int *idx32, const int *inv_ptr, const int *inv_pos, const float *luts,
-                         const float *gy, float alpha, float beta, float *gx, float *gluts, int B, int I, int N, int k,
-                         int O, hipStream_t s) {
+                         const float *gy, float alpha, float beta, const float *scale, float *gx, float *gluts, int B, int I,
+                         int N, int k, int O, hipStream_t s) {
     const long long NO = (long long)N * O;
     dwn_generic_zero<<<dl_ceil_div(NO << k, 256), 256, 0, s>>>(gluts, NO << k);
-    dwn_generic_bwd_luts<<<dl_ceil_div((long long)B * NO, 256), 256, 0, s>>>(x, idx32, gy, gluts, B, I, N, k, O);
+    dwn_generic_bwd_luts<<<dl_ceil_div((long long)B * NO, 256), 256, 0, s>>>(x, idx32, gy, scale, gluts, B, I, N, k, O);
     if (gx)
         dwn_generic_bwd_gx<<<dl_ceil_div((long long)B * I, 256), 256, 0, s>>>(x, idx32, inv_ptr, inv_pos, luts, gy, alpha,
-                                                                            beta, gx, B, I, N, k, O);
+                                                                            beta, scale, gx, B, I, N, k, O);
     return dl_launch_status();
 }
 

@@ -228,6 +228,62 @@ __global__ __launch_bounds__(256) void dwn_efd_table(const float *__restrict__ l
     }
 }
 
+// stable_table: the D form for the gradient-stabilised node, whose weight of a table entry at
+// Hamming distance h (over the other k-1 inputs) is scale[n] / (h + 1) instead of alpha * beta^h.
+// That weight is not a product over inputs, so the sums are taken directly, in double: one wavefront
+// per table keeps it in LDS and shares out the k * 2^(k-1) outputs (j, a'), one 2^(k-1)-term sum
+//   D[c][j][a'] = scale * sum_kappa' (lut[kappa' with bit j set] - lut[kappa' with bit j clear]) / (popc(a' ^ kappa') + 1)
+// each.  Also clears the table's gradient row.
+__global__ __launch_bounds__(256) void dwn_stable_table(const float *__restrict__ luts, const float *__restrict__ scale,
+                                                         float *__restrict__ D, float *__restrict__ gluts, int NO, int K,
+                                                         int O) {
+    __shared__ double rec[8];
+    __shared__ float tab[4][64];
+    if (threadIdx.x < 8) rec[threadIdx.x] = 1.0 / (double)(threadIdx.x + 1);
+    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int c = blockIdx.x * 4 + w;
+    const int L = 1 << K, Lh = L >> 1;
+    if (c < NO && lane < L) {
+        tab[w][lane] = luts[(size_t)c * L + lane];
+        gluts[(size_t)c * L + lane] = 0.0f;
+    }
+    __syncthreads();
+    if (c >= NO) return;
+    const double sc = (double)scale[c / O];
+    for (int o = lane; o < K * Lh; o += 64) {
+        const int j = o / Lh, ap = o - j * Lh;
+        const int low = (1 << j) - 1;
+        double acc = 0.0;
+        for (int kp = 0; kp < Lh; ++kp) {
+            const int lo = (kp & low) | ((kp & ~low) << 1);  // kappa' with a clear bit j put in
+            acc += ((double)tab[w][lo | (1 << j)] - (double)tab[w][lo]) * rec[__popc(ap ^ kp)];
+        }
+        D[((size_t)c * K + j) * Lh + ap] = (float)(sc * acc);
+    }
+}
+
+// gluts[c][a] *= scale[c / O]: the stabilised node scales its table gradient as well
+__global__ __launch_bounds__(256) void dwn_scale_tables(float *__restrict__ gluts, const float *__restrict__ scale,
+                                                         long long total, int L, int O) {
+    const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (e < total) gluts[e] *= scale[(e / L) / O];
+}
+
+// luts = sigmoid(raw) and its adjoint graw = gluts * luts * (1 - luts), elementwise
+__global__ __launch_bounds__(256) void dwn_table_sigmoid(const float *__restrict__ raw, float *__restrict__ luts,
+                                                          long long total) {
+    const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (e < total) luts[e] = 1.0f / (1.0f + expf(-raw[e]));
+}
+__global__ __launch_bounds__(256) void dwn_table_sigmoid_bwd(const float *__restrict__ gluts, const float *__restrict__ luts,
+                                                              float *__restrict__ graw, long long total) {
+    const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (e < total) {
+        const float v = luts[e];
+        graw[e] = gluts[e] * v * (1.0f - v);
+    }
+}
+
 // ---------------------------------------------------------------------------------
 // transpose_hist: grid (ceil(N*O / 64), chunks); a block streams `tiles_per_chunk` 64-row tiles
 // of its 64 columns.  The next tile (gy values and their addresses) is prefetched into registers
@@ -573,9 +629,11 @@ static void dwn_launch_gx(const float *gyT, const uint8_t *addrT, const float *D
 
 // backward of the k <= 6 path; gy row-major [B, N*O] or (gy_tiled) tile-major [B/64][N*O][64];
 // gx row-major [B, I] or (gx_tiled) tile-major [B/64][I][64]
+// scale == null: EFD weights alpha * beta^h; otherwise the stabilised weights scale[n] / (h + 1),
+// which also multiply the table gradient
 static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos, const float *luts,
-                             const float *gy, int gy_tiled, float alpha, float beta, float *gx, int gx_tiled,
-                             float *gluts, void *ws, int B, int I, int N, int k, int O, hipStream_t s) {
+                             const float *gy, int gy_tiled, float alpha, float beta, const float *scale, float *gx,
+                             int gx_tiled, float *gluts, void *ws, int B, int I, int N, int k, int O, hipStream_t s) {
     const long long NO = (long long)N * O;
     const int L = 1 << k;
     const uint8_t *addrT = (const uint8_t *)saved;
@@ -590,8 +648,11 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
     const int tpc = dl_ceil_div(BT, chunks);
     chunks = dl_ceil_div(BT, tpc);
     const dim3 hgrid(col_tiles, chunks);
-    const bool sform = beta >= -0.5f && beta <= 0.5f;
-    if (gx)
+    const bool sform = !scale && beta >= -0.5f && beta <= 0.5f;
+    if (gx && scale)
+        DL_TIMED("dwn_stable_table", s,
+                 (dwn_stable_table<<<dl_ceil_div(NO, 4), 256, 0, s>>>(luts, scale, D, gluts, (int)NO, k, O)));
+    else if (gx)
         DL_TIMED("dwn_efd_table", s,
                  (dwn_efd_table<<<dl_ceil_div(NO, 4), 256, 0, s>>>(luts, D, gluts, (int)NO, k, alpha, beta, sform ? 1 : 0)));
     else
@@ -616,6 +677,9 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
             default: dwn_launch_gx<6>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, s); break;
         }
     }
+    if (scale)
+        DL_TIMED("dwn_scale_tables", s,
+                 (dwn_scale_tables<<<dl_ceil_div(NO * L, 256), 256, 0, s>>>(gluts, scale, NO * L, L, O)));
     return dl_launch_status();
 }
 
@@ -630,11 +694,48 @@ extern "C" int dl_dwn_layer_bwd(const float *x, const void *saved, const int32_t
     hipStream_t s = (hipStream_t)stream;
     if (!dwn_fast(N, k, O)) {
         if (!x) return DL_ERR_NULL;
-        return dwn_generic_backward(x, idx32, inv_ptr, inv_pos, luts, gy, alpha, beta, gx, gluts, B, I, N, k, O, s);
+        return dwn_generic_backward(x, idx32, inv_ptr, inv_pos, luts, gy, alpha, beta, nullptr, gx, gluts, B, I, N, k, O, s);
     }
     if (!saved || !ws) return DL_ERR_NULL;
     if (ws_bytes < dl_dwn_bwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
-    return dwn_backward_fast(saved, inv_ptr, inv_pos, luts, gy, 0, alpha, beta, gx, 0, gluts, ws, B, I, N, k, O, s);
+    return dwn_backward_fast(saved, inv_ptr, inv_pos, luts, gy, 0, alpha, beta, nullptr, gx, 0, gluts, ws, B, I, N, k, O, s);
+}
+
+extern "C" int dl_dwn_stable_layer_bwd(const float *x, const void *saved, const int32_t *idx32, const int32_t *inv_ptr,
+                                       const int32_t *inv_pos, const float *luts, const float *gy,
+                                       const float *gradient_scale, float *gx, float *gluts, void *ws, size_t ws_bytes,
+                                       int B, int I, int N, int k, int O, void *stream) {
+    if (!idx32 || !luts || !gy || !gluts || !gradient_scale) return DL_ERR_NULL;
+    if (gx && (!inv_ptr || !inv_pos)) return DL_ERR_NULL;
+    int rc = dwn_check(B, I, N, k, O);
+    if (rc) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    if (!dwn_fast(N, k, O)) {
+        if (!x) return DL_ERR_NULL;
+        return dwn_generic_backward(x, idx32, inv_ptr, inv_pos, luts, gy, 0.0f, 0.0f, gradient_scale, gx, gluts, B, I, N, k,
+                                    O, s);
+    }
+    if (!saved || !ws) return DL_ERR_NULL;
+    if (ws_bytes < dl_dwn_bwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
+    return dwn_backward_fast(saved, inv_ptr, inv_pos, luts, gy, 0, 0.0f, 0.0f, gradient_scale, gx, 0, gluts, ws, B, I, N, k,
+                             O, s);
+}
+
+extern "C" int dl_table_sigmoid_fwd(const float *raw, float *luts, long long count, void *stream) {
+    if (!raw || !luts) return DL_ERR_NULL;
+    if (count <= 0 || count > 0x7fffffffLL * 256) return DL_ERR_SHAPE;
+    hipStream_t s = (hipStream_t)stream;
+    DL_TIMED("dwn_table_sigmoid", s, (dwn_table_sigmoid<<<dl_ceil_div(count, 256), 256, 0, s>>>(raw, luts, count)));
+    return dl_launch_status();
+}
+
+extern "C" int dl_table_sigmoid_bwd(const float *gluts, const float *luts, float *graw, long long count, void *stream) {
+    if (!gluts || !luts || !graw) return DL_ERR_NULL;
+    if (count <= 0 || count > 0x7fffffffLL * 256) return DL_ERR_SHAPE;
+    hipStream_t s = (hipStream_t)stream;
+    DL_TIMED("dwn_table_sigmoid_bwd", s,
+             (dwn_table_sigmoid_bwd<<<dl_ceil_div(count, 256), 256, 0, s>>>(gluts, luts, graw, count)));
+    return dl_launch_status();
 }
 
 // ---------------------------------------------------------------------------------
@@ -687,6 +788,6 @@ extern "C" int dl_dwn_layer_bwd_tiled(const void *saved, const int32_t *inv_ptr,
     if (rc) return rc;
     if (!dwn_fast(N, k, O)) return DL_ERR_UNSUPPORTED;
     if (ws_bytes < dl_dwn_bwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
-    return dwn_backward_fast(saved, inv_ptr, inv_pos, luts, gy, gy_tiled, alpha, beta, gx, gx_tiled, gluts, ws, B, I, N, k, O,
+    return dwn_backward_fast(saved, inv_ptr, inv_pos, luts, gy, gy_tiled, alpha, beta, nullptr, gx, gx_tiled, gluts, ws, B, I, N, k, O,
                              (hipStream_t)stream);
 }

@@ -10,6 +10,7 @@ __device__ __forceinline__ float dl_sigmoid(float v) { return 1.0f / (1.0f + exp
 
 typedef float prob_f4 __attribute__((ext_vector_type(4)));
 #define PROB_RSRC 0x00020000
+#define PROB_HYBRID_EPS 1e-8f
 
 // ---------------------------------------------------------------------------------
 // k <= 6 path.  As for the DWN nodes, a wavefront's 64 lanes are 64 batch rows and everything
@@ -147,8 +148,10 @@ __global__ __launch_bounds__(64 * PROB_FW) void prob_fwd_t(const float *__restri
     }
 }
 
-// one wavefront per (column, chunk of batch tiles); 4 wavefronts per block
-template <int K>
+// one wavefront per (column, chunk of batch tiles); 4 wavefronts per block.
+// HYB (hybrid node): the table is used as given and the input gradient carries the factor
+// q / (q + 1e-8), q = x_j (1 - x_j), of that node's backward.
+template <int K, bool HYB>
 __global__ __launch_bounds__(256) void prob_bwd_t(const float *__restrict__ xT, const float *__restrict__ gyT,
                                                    const int *__restrict__ idx32, const float *__restrict__ sig,
                                                    float *__restrict__ gmT, float *__restrict__ gpart, int I, int N,
@@ -213,8 +216,12 @@ __global__ __launch_bounds__(256) void prob_bwd_t(const float *__restrict__ xT, 
             float sum = 0.0f;
 #pragma unroll
             for (int a = 0; a < cnt; ++a) sum = fmaf(bar[a], diff[base + a], sum);
-            dx[j] = sum;
             const float om = 1.0f - xs[j];
+            if (HYB) {
+                const float q = xs[j] * om;
+                sum = sum * q / (q + PROB_HYBRID_EPS);
+            }
+            dx[j] = sum;
 #pragma unroll
             for (int a = cnt - 1; a >= 0; --a) {
                 const float w = bar[a];
@@ -253,7 +260,8 @@ __global__ __launch_bounds__(256) void prob_bwd_t(const float *__restrict__ xT, 
     if ((lane & ((64 >> K) - 1)) == 0) gpart[((size_t)chunk * NO + c) * L + a] = mine;
 }
 
-// graw[n,a,d] = sigmoid'(w/T)/T * sum over chunks of gpart[chunk][c][a]
+// graw[n,a,d] = sigmoid'(w/T)/T * sum over chunks of gpart[chunk][c][a];
+// sig == null (hybrid node): the plain sum, kept in the table's own layout [c][a]
 __global__ __launch_bounds__(256) void prob_reduce_weights(const float *__restrict__ gpart, const float *__restrict__ sig,
                                                             float inv_t, float *__restrict__ graw, int N, int L, int O,
                                                             int chunks) {
@@ -262,6 +270,10 @@ __global__ __launch_bounds__(256) void prob_reduce_weights(const float *__restri
     if (e >= total) return;
     float acc = 0.0f;
     for (int ch = 0; ch < chunks; ++ch) acc += gpart[(size_t)ch * total + e];
+    if (!sig) {
+        graw[e] = acc;
+        return;
+    }
     const int a = (int)(e % L);
     const long long c = e / L;
     const int n = (int)(c / O), d = (int)(c % O);
@@ -405,10 +417,12 @@ __global__ __launch_bounds__(256) void prob_generic_fwd(const float *__restrict_
     y[gid] = acc;
 }
 
+// hybrid: `raw` is the table itself in the layout [n][d][a] and the input gradient carries q / (q + 1e-8)
 __global__ __launch_bounds__(256) void prob_generic_bwd(const float *__restrict__ x, const int *__restrict__ idx32,
                                                          const float *__restrict__ raw, float inv_t,
                                                          const float *__restrict__ gy, float *__restrict__ gx,
-                                                         float *__restrict__ graw, int B, int I, int N, int K, int O) {
+                                                         float *__restrict__ graw, int B, int I, int N, int K, int O,
+                                                         int hybrid) {
     const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
     if (gid >= (long long)B * N) return;
     const int b = (int)(gid / N), n = (int)(gid % N);
@@ -418,11 +432,11 @@ __global__ __launch_bounds__(256) void prob_generic_bwd(const float *__restrict_
     for (int d = 0; d < O; ++d) {
         const float g = gy[((size_t)b * N + n) * O + d];
         for (int a = 0; a < L; ++a) {
-            const size_t w = ((size_t)n * L + a) * O + d;
-            const float s = dl_sigmoid(raw[w] * inv_t);
+            const size_t w = hybrid ? ((size_t)n * O + d) * L + a : ((size_t)n * L + a) * O + d;
+            const float s = hybrid ? raw[w] : dl_sigmoid(raw[w] * inv_t);
             float p = 1.0f;
             for (int j = 0; j < K; ++j) p *= ((a >> j) & 1) ? xs[j] : 1.0f - xs[j];
-            atomicAdd(&graw[w], g * p * s * (1.0f - s) * inv_t);
+            atomicAdd(&graw[w], hybrid ? g * p : g * p * s * (1.0f - s) * inv_t);
             if (gx) {
                 for (int j = 0; j < K; ++j) {
                     float q = 1.0f;
@@ -434,7 +448,10 @@ __global__ __launch_bounds__(256) void prob_generic_bwd(const float *__restrict_
         }
     }
     if (gx)
-        for (int j = 0; j < K; ++j) atomicAdd(&gx[(size_t)b * I + idx32[(size_t)n * K + j]], gxs[j]);
+        for (int j = 0; j < K; ++j) {
+            const float q = xs[j] * (1.0f - xs[j]);
+            atomicAdd(&gx[(size_t)b * I + idx32[(size_t)n * K + j]], hybrid ? gxs[j] * q / (q + PROB_HYBRID_EPS) : gxs[j]);
+        }
 }
 
 __global__ __launch_bounds__(256) void prob_eval_kernel(const float *__restrict__ x, const int *__restrict__ idx32,
@@ -540,7 +557,7 @@ extern "C" int dl_prob_layer_bwd(const float *x, const void *saved, const int32_
         DL_TIMED("prob_fill_zero", s, (prob_fill_zero<<<dl_ceil_div(WT, 256), 256, 0, s>>>(graw, WT)));
         if (gx) prob_fill_zero<<<dl_ceil_div((long long)B * I, 256), 256, 0, s>>>(gx, (long long)B * I);
         DL_TIMED("prob_generic_bwd", s, (prob_generic_bwd<<<dl_ceil_div((long long)B * N, 256), 256, 0, s>>>(x, idx32, raw_w, inv_t, gy, gx, graw, B, I, N,
-                                                                          k, O)));
+                                                                          k, O, 0)));
         return dl_launch_status();
     }
     if (!ws) return DL_ERR_NULL;
@@ -564,12 +581,65 @@ extern "C" int dl_prob_layer_bwd(const float *x, const void *saved, const int32_
     DL_TIMED("prob_to_tiles_gy", s, (prob_to_tiles<<<dim3(dl_ceil_div(NO, 64), BT), 256, 0, s>>>(gy, gyT, B, NO)));
 #define CALL(KK)                                                                                                    \
     DL_TIMED("prob_bwd_t", s,                                                                                       \
-             (prob_bwd_t<KK><<<dim3(dl_ceil_div(NO, 4), chunks), 256, 0, s>>>(xT, gyT, idx32, sig, gmT, gpart, I, N, O, BT, \
-                                                                           tpc, gx != nullptr)))
+             (prob_bwd_t<KK, false><<<dim3(dl_ceil_div(NO, 4), chunks), 256, 0, s>>>(xT, gyT, idx32, sig, gmT, gpart, I, N, O, \
+                                                                                  BT, tpc, gx != nullptr)))
     PROB_DISPATCH(k, CALL)
 #undef CALL
     DL_TIMED("prob_reduce_weights", s,
              (prob_reduce_weights<<<dl_ceil_div(WT, 256), 256, 0, s>>>(gpart, sig, inv_t, graw, N, L, O, chunks)));
+    if (gx && O == 1)
+        DL_TIMED("prob_gather_t", s,
+                 (prob_gather_t<true><<<dl_xcd_grid(dl_ceil_div(I, PROB_IS), BT), 256, 0, s>>>(gmT, inv_ptr, inv_pos, gx, B, I,
+                                                                                             N, k, O, BT)));
+    else if (gx)
+        DL_TIMED("prob_gather_t", s,
+                 (prob_gather_t<false><<<dl_xcd_grid(dl_ceil_div(I, PROB_IS), BT), 256, 0, s>>>(gmT, inv_ptr, inv_pos, gx, B, I,
+                                                                                              N, k, O, BT)));
+    return dl_launch_status();
+}
+
+// Hybrid nodes: the forward is the DWN lookup; the backward is the probabilistic one on the table as given.
+extern "C" size_t dl_hybrid_bwd_workspace_bytes(int B, int I, int N, int k, int O) {
+    if (B <= 0 || I <= 0 || N <= 0 || k <= 0 || O <= 0 || !prob_fast(I, N, k, O)) return 256;
+    return dl_prob_bwd_workspace_bytes(B, I, N, k, O) - prob_sig_bytes(N, k, O);
+}
+
+extern "C" int dl_hybrid_layer_bwd(const float *x, const int32_t *idx32, const int32_t *inv_ptr, const int32_t *inv_pos,
+                                   const float *luts, const float *gy, float *gx, float *gluts, void *ws, size_t ws_bytes,
+                                   int B, int I, int N, int k, int O, void *stream) {
+    if (!x || !idx32 || !luts || !gy || !gluts) return DL_ERR_NULL;
+    if (gx && (!inv_ptr || !inv_pos)) return DL_ERR_NULL;
+    int rc = prob_check(B, I, N, k, O);
+    if (rc) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    const long long WT = (long long)N * ((long long)1 << k) * O;
+    if (!prob_fast(I, N, k, O)) {
+        DL_TIMED("prob_fill_zero", s, (prob_fill_zero<<<dl_ceil_div(WT, 256), 256, 0, s>>>(gluts, WT)));
+        if (gx) prob_fill_zero<<<dl_ceil_div((long long)B * I, 256), 256, 0, s>>>(gx, (long long)B * I);
+        DL_TIMED("prob_generic_bwd", s, (prob_generic_bwd<<<dl_ceil_div((long long)B * N, 256), 256, 0, s>>>(
+                                            x, idx32, luts, 1.0f, gy, gx, gluts, B, I, N, k, O, 1)));
+        return dl_launch_status();
+    }
+    if (!ws) return DL_ERR_NULL;
+    if (ws_bytes < dl_hybrid_bwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
+    const int BT = prob_bt(B), L = 1 << k, NO = N * O;
+    const int tpc = prob_tiles_per_chunk(B, N, O);
+    const int chunks = dl_ceil_div(BT, tpc);
+    char *w = (char *)ws;
+    float *xT = (float *)w; w += prob_xT_bytes(B, I);
+    float *gyT = (float *)w; w += dl_align256((size_t)BT * NO * 64 * sizeof(float));
+    float *gmT = (float *)w; w += dl_align256((size_t)BT * NO * k * 64 * sizeof(float));
+    float *gpart = (float *)w;
+    DL_TIMED("prob_to_tiles_x", s, (prob_to_tiles<<<dim3(dl_ceil_div(I, 64), BT), 256, 0, s>>>(x, xT, B, I)));
+    DL_TIMED("prob_to_tiles_gy", s, (prob_to_tiles<<<dim3(dl_ceil_div(NO, 64), BT), 256, 0, s>>>(gy, gyT, B, NO)));
+#define CALL(KK)                                                                                                          \
+    DL_TIMED("hybrid_bwd_t", s,                                                                                           \
+             (prob_bwd_t<KK, true><<<dim3(dl_ceil_div(NO, 4), chunks), 256, 0, s>>>(xT, gyT, idx32, luts, gmT, gpart, I, N, O, \
+                                                                                 BT, tpc, gx != nullptr)))
+    PROB_DISPATCH(k, CALL)
+#undef CALL
+    DL_TIMED("prob_reduce_weights", s,
+             (prob_reduce_weights<<<dl_ceil_div(WT, 256), 256, 0, s>>>(gpart, nullptr, 1.0f, gluts, N, L, O, chunks)));
     if (gx && O == 1)
         DL_TIMED("prob_gather_t", s,
                  (prob_gather_t<true><<<dl_xcd_grid(dl_ceil_div(I, PROB_IS), BT), 256, 0, s>>>(gmT, inv_ptr, inv_pos, gx, B, I,

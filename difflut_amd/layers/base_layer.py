@@ -5,7 +5,7 @@ Public surface of difflut/layers/base_layer.py:35-576: constructor arguments and
 `get_mapping`, `regularization`, the bit-flip augmentation and the gradient-stabilisation hook.
 
 What is different underneath: when every node is of a type the device library covers
-(DWNNode, ProbabilisticNode) the layer runs all nodes in ONE call on one contiguous
+(DWNNode, DWNStableNode, HybridNode, ProbabilisticNode) the layer runs all nodes in ONE call on one contiguous
 [N, ...] parameter tensor instead of looping over N modules.  The per-node Parameters that
 users, optimisers and state_dict see (`nodes.{i}.luts`, ...) are views into that tensor:
   * `ParameterBank.flat` is the [N, ...] leaf the fused autograd Function differentiates;
@@ -179,18 +179,24 @@ class BaseLUTLayer(ABC, LUTLayerMixin, nn.Module):
             self._banks["luts"] = ParameterBank(self.nodes, "luts")
         elif self._fused == "probabilistic":
             self._banks["raw_weights"] = ParameterBank(self.nodes, "raw_weights")
+        elif self._fused == "dwn_stable":
+            self._banks["raw_luts"] = ParameterBank(self.nodes, "raw_luts")
+            self._banks["gradient_scale"] = ParameterBank(self.nodes, "gradient_scale")
+        elif self._fused == "hybrid":
+            self._banks["raw_luts"] = ParameterBank(self.nodes, "raw_luts")
         self._validate_layer_config()
 
     # ------------------------------------------------------------------ fused execution
     def _detect_fused_kind(self):
         from ..nodes.dwn_node import DWNNode
+        from ..nodes.dwn_stable_node import DWNStableNode
+        from ..nodes.hybrid_node import HybridNode
         from ..nodes.probabilistic_node import ProbabilisticNode
 
         kinds = {type(node) for node in self.nodes}
-        if kinds == {DWNNode}:
-            return "dwn"
-        if kinds == {ProbabilisticNode}:
-            return "probabilistic"
+        for cls in (DWNNode, ProbabilisticNode, DWNStableNode, HybridNode):
+            if kinds == {cls}:
+                return cls.fused_kind
         return None  # other node types: per-node loop over the gathered inputs
 
     def _apply(self, fn, *args, **kwargs):
@@ -229,6 +235,17 @@ class BaseLUTLayer(ABC, LUTLayerMixin, nn.Module):
             if self.training:
                 return ops.ProbLayerFunction.apply(x, raw, plan, first.temperature_value())
             return ops.prob_layer_eval(x, raw.detach(), plan, first.temperature_value())
+        if self._fused in ("dwn_stable", "hybrid"):
+            from .. import ops
+
+            raw = self._banks["raw_luts"].tensor()
+            if not self.training:
+                with torch.no_grad():
+                    return ops.dwn_layer_eval(x, ops.TableSigmoidFunction.apply(raw), plan)
+            luts = ops.TableSigmoidFunction.apply(raw)
+            if self._fused == "hybrid":
+                return ops.HybridLayerFunction.apply(x, luts, plan)
+            return ops.DWNStableLayerFunction.apply(x, luts, self._banks["gradient_scale"].tensor().detach(), plan)
         return None
 
     def _loop_nodes(self, mapped):

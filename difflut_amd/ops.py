@@ -206,6 +206,109 @@ def dwn_layer_eval(x, luts, plan):
     return y
 
 
+# ----------------------------------------------------------------------------- DWN-stable and hybrid nodes
+class TableSigmoidFunction(torch.autograd.Function):
+    """luts = sigmoid(raw_luts), elementwise, for a whole bank of tables at once
+    (`_get_luts`, dwn_stable_node.py:289-295, hybrid_node.py:309-315)."""
+
+    @staticmethod
+    def forward(ctx, raw):
+        nat.require_device(raw)
+        raw = _f32(raw)
+        luts = torch.empty_like(raw)
+        nat.check(nat.lib().dl_table_sigmoid_fwd(nat.ptr(raw), nat.ptr(luts), raw.numel(), nat.stream()))
+        ctx.save_for_backward(luts)
+        return luts
+
+    @staticmethod
+    def backward(ctx, gl):
+        (luts,) = ctx.saved_tensors
+        gl = _f32(gl)
+        graw = torch.empty_like(luts)
+        nat.check(nat.lib().dl_table_sigmoid_bwd(nat.ptr(gl), nat.ptr(luts), nat.ptr(graw), luts.numel(), nat.stream()))
+        return graw
+
+
+def _dwn_lookup(x, luts, plan):
+    """Training forward shared by the DWN-type nodes: (y, saved, dims)."""
+    B, I = x.shape
+    N, O, L = luts.shape
+    k = plan.k
+    if (N, 1 << k, I) != (plan.N, L, plan.I):
+        raise RuntimeError(f"shape mismatch: x {tuple(x.shape)}, luts {tuple(luts.shape)}, mapping [{plan.N},{k}] "
+                           f"over {plan.I} inputs")
+    lib = nat.lib()
+    dims = (B, I, N, k, O)
+    y = torch.empty((B, N * O), dtype=torch.float32, device=x.device)
+    saved = _bytes(lib.dl_dwn_saved_bytes(*dims), x.device)
+    ws = _bytes(lib.dl_dwn_fwd_workspace_bytes(*dims), x.device)
+    nat.check(lib.dl_dwn_layer_fwd(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(luts), nat.ptr(y), nat.ptr(saved),
+                                   nat.ptr(ws), ws.numel(), *dims, nat.stream()))
+    return y, saved, dims
+
+
+class DWNStableLayerFunction(torch.autograd.Function):
+    """Thresholded lookup with the gradient-stabilised backward: the EFD sum weighted 1/(h+1) and
+    multiplied, like the table gradient, by the node's gradient scale (dwn_stable_node.py:36-206).
+    `scale` is a device tensor [N] (one value per node); it gets no gradient, as in the reference."""
+
+    @staticmethod
+    def forward(ctx, x, luts, scale, plan):
+        nat.require_device(x, luts, scale)
+        x, luts = _f32(x), _f32(luts)
+        scale = _f32(scale.detach()).reshape(-1)
+        if scale.numel() != luts.shape[0]:
+            raise RuntimeError(f"gradient_scale has {scale.numel()} entries for {luts.shape[0]} nodes")
+        y, saved, dims = _dwn_lookup(x, luts, plan)
+        ctx.save_for_backward(luts, saved, scale, x if plan.k > FAST_K else None)
+        ctx.plan, ctx.dims = plan, dims
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        luts, saved, scale, x = ctx.saved_tensors
+        B, I, N, k, O = ctx.dims
+        plan = ctx.plan
+        gy = _f32(gy)
+        lib = nat.lib()
+        gx = torch.empty((B, I), dtype=torch.float32, device=gy.device) if ctx.needs_input_grad[0] else None
+        gl = torch.empty_like(luts)
+        ws = _bytes(lib.dl_dwn_bwd_workspace_bytes(*ctx.dims), gy.device)
+        nat.check(lib.dl_dwn_stable_layer_bwd(nat.ptr(x), nat.ptr(saved), nat.ptr(plan.idx32), nat.ptr(plan.inv_ptr),
+                                              nat.ptr(plan.inv_pos), nat.ptr(luts), nat.ptr(gy), nat.ptr(scale),
+                                              nat.ptr(gx), nat.ptr(gl), nat.ptr(ws), ws.numel(), *ctx.dims,
+                                              nat.stream()))
+        return gx, gl, None, None
+
+
+class HybridLayerFunction(torch.autograd.Function):
+    """Thresholded lookup forward, probabilistic backward on the real-valued inputs (hybrid_node.py:33-204)."""
+
+    @staticmethod
+    def forward(ctx, x, luts, plan):
+        nat.require_device(x, luts)
+        x, luts = _f32(x), _f32(luts)
+        y, _, dims = _dwn_lookup(x, luts, plan)
+        ctx.save_for_backward(x, luts)
+        ctx.plan, ctx.dims = plan, dims
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        x, luts = ctx.saved_tensors
+        B, I, N, k, O = ctx.dims
+        plan = ctx.plan
+        gy = _f32(gy)
+        lib = nat.lib()
+        gx = torch.empty((B, I), dtype=torch.float32, device=gy.device) if ctx.needs_input_grad[0] else None
+        gl = torch.empty_like(luts)
+        ws = _bytes(lib.dl_hybrid_bwd_workspace_bytes(*ctx.dims), gy.device)
+        nat.check(lib.dl_hybrid_layer_bwd(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(plan.inv_ptr), nat.ptr(plan.inv_pos),
+                                          nat.ptr(luts), nat.ptr(gy), nat.ptr(gx), nat.ptr(gl), nat.ptr(ws), ws.numel(),
+                                          *ctx.dims, nat.stream()))
+        return gx, gl, None
+
+
 # ----------------------------------------------------------------------------- Probabilistic
 class ProbLayerFunction(torch.autograd.Function):
     """y[b, n*O+d] = sum_a sigmoid(raw[n,a,d]/T) prod_j (x_j a_j + (1-x_j)(1-a_j))."""

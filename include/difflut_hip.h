@@ -114,6 +114,50 @@ int dl_dwn_layer_eval(const float *x, const int32_t *idx32, const float *luts, f
                       int B, int I, int N, int k, int O, void *stream);
 
 /* ------------------------------------------------------------------------
+ * RandomLayer + gradient-stabilised DWN nodes (node type "dwn_stable").
+ * Replaces the node loop over dwn_stable_cuda.forward/.backward
+ * (difflut/nodes/cuda/dwn_stable_cuda_kernel.cu:13-74, 84-242) and
+ * GradientStabilizedFunctionCPU (difflut/nodes/dwn_stable_node.py:113-206).
+ * The training forward is the DWN lookup on luts = sigmoid(raw_luts): dl_table_sigmoid_fwd, then
+ * dl_dwn_layer_fwd.  The backward is the EFD sum with the weight 1/(h+1) in place of
+ * alpha*beta^h, h = popc((addr ^ kappa) & ~(1<<j)), times the node's gradient scale:
+ *   gx[b,i]      = sum_{(n,j): idx=i} scale[n] * sum_d gy[b,n,d] *
+ *                  sum_kappa s(kappa_j) luts[n,d,kappa] / (h + 1)
+ *   gluts[n,d,e] = scale[n] * sum_b [addr(b,n) = e] gy[b,n,d]
+ * gradient_scale [N] is a DEVICE array (the nodes' `gradient_scale` parameters stacked), so no
+ * value has to be read back by the host.  saved / ws / x as for dl_dwn_layer_bwd.
+ * dl_table_sigmoid_bwd is the adjoint of the table sigmoid: graw = gluts * luts * (1 - luts)
+ * (what autograd applies for `_get_luts`, dwn_stable_node.py:289-295, hybrid_node.py:309-315).
+ * ------------------------------------------------------------------------ */
+int dl_table_sigmoid_fwd(const float *raw, float *luts, long long count, void *stream);
+int dl_table_sigmoid_bwd(const float *gluts, const float *luts, float *graw, long long count, void *stream);
+int dl_dwn_stable_layer_bwd(const float *x, const void *saved, const int32_t *idx32,
+                            const int32_t *inv_ptr, const int32_t *inv_pos,
+                            const float *luts, const float *gy, const float *gradient_scale,
+                            float *gx, float *gluts, void *ws, size_t ws_bytes,
+                            int B, int I, int N, int k, int O, void *stream);
+
+/* ------------------------------------------------------------------------
+ * RandomLayer + hybrid nodes (node type "hybrid"): thresholded lookup forward (dl_table_sigmoid_fwd,
+ * then dl_dwn_layer_fwd), probabilistic backward.  Replaces the node loop over
+ * hybrid_cuda.forward/.backward (difflut/nodes/cuda/hybrid_cuda_kernel.cu:7-126, 129-243) and
+ * HybridFunctionCPU (difflut/nodes/hybrid_node.py:105-204):
+ *   p[b,n,a]     = prod_j (x_j a_j + (1 - x_j)(1 - a_j)),  x_j = x[b, idx[n,j]] as given
+ *   gluts[n,d,a] = sum_b p[b,n,a] gy[b,n,d]
+ *   gx[b,i]      = sum_{(n,j): idx=i} sum_d gy[b,n,d] sum_a luts[n,d,a] p[b,n,a]
+ *                  (a_j - x_j) / (x_j (1 - x_j) + 1e-8)
+ * computed as dy/dx_j of the multilinear interpolation times q/(q + 1e-8), q = x_j (1 - x_j):
+ * the same value, and like the reference exactly 0 where x_j is 0 or 1.
+ * luts [N,O,L]; gx [B,I] (nullable) and gluts [N,O,L] are overwritten.
+ * ------------------------------------------------------------------------ */
+size_t dl_hybrid_bwd_workspace_bytes(int B, int I, int N, int k, int O);
+int dl_hybrid_layer_bwd(const float *x, const int32_t *idx32,
+                        const int32_t *inv_ptr, const int32_t *inv_pos,
+                        const float *luts, const float *gy, float *gx, float *gluts,
+                        void *ws, size_t ws_bytes,
+                        int B, int I, int N, int k, int O, void *stream);
+
+/* ------------------------------------------------------------------------
  * RandomLayer + Probabilistic nodes, whole layer in one call.
  * Replaces the node loop over probabilistic_cuda.forward/.backward
  * (difflut/nodes/cuda/probabilistic_cuda.cpp:22-49, probabilistic_cuda_kernel.cu:7-307)

@@ -18,6 +18,10 @@ Pin status (see tests/test_oracle.py for the checks):
   hard_mapping .............. golden
   thermometer_* ............. golden thresholds/bits, notebook known answer [0.25,0.5,0.75]
   group_sum ................. golden, reference unit-test values
+  stable_coefficients/backward  integral of the pinned EFD coefficients over beta in [0,1] (1/(h+1) =
+                              int beta^h), literal-loop restatement, k=1 and constant-table cases, histogram sum
+  hybrid_backward ........... autograd of the multilinear interpolation for interior x, per-thread loop form
+                              of the device kernels, exact zeros at x in {0,1}, partition of unity
 No function is left "parity unpinned".
 """
 from __future__ import annotations
@@ -205,6 +209,114 @@ def dwn_layer_backward(x, idx, luts, gy, alpha, beta):
     for d in range(O):
         np.add.at(gl[:, d, :], (np.broadcast_to(n_ar, addr.shape), addr), gy64[b_ar, n_ar, d])
     return gx, gl
+
+
+# ----------------------------------------------------------------------------
+# f1  Gradient-stabilised DWN node       dwn_stable_node.py:113-206, dwn_stable_cuda_kernel.cu:84-172
+# ----------------------------------------------------------------------------
+
+
+def table_sigmoid(raw):
+    """luts = sigmoid(raw_luts) (dwn_stable_node.py:289-295, hybrid_node.py:309-315), float64."""
+    return 1.0 / (1.0 + np.exp(-np.asarray(raw, dtype=np.float64)))
+
+
+def stable_coefficients(luts, scale=1.0):
+    """D[..., l, a] = scale * sum_kappa s(kappa_l) luts[..., kappa] / (popc((a^kappa)&~(1<<l)) + 1).
+
+    The EFD sum with the weight beta^h replaced by 1/(h+1) (dwn_stable_node.py:176-201).
+    `scale` broadcasts against luts.shape[:-1].  luts [..., 2^k] -> D [..., k, 2^k], float64.
+    """
+    luts = np.asarray(luts, dtype=np.float64)
+    L = luts.shape[-1]
+    k = L.bit_length() - 1
+    a = np.arange(L)[:, None]
+    kap = np.arange(L)[None, :]
+    D = np.empty(luts.shape[:-1] + (k, L), dtype=np.float64)
+    for l in range(k):
+        mask = (L - 1) & ~(1 << l)
+        ham = np.vectorize(lambda v: bin(v).count("1"))((a ^ kap) & mask)
+        sgn = np.where((kap >> l) & 1, 1.0, -1.0)
+        D[..., l, :] = luts @ (sgn / (ham + 1.0)).T
+    return D * np.asarray(scale, dtype=np.float64)[..., None, None]
+
+
+def stable_backward(xk, luts, gy, scale):
+    """One node: xk [B,k], luts [O,2^k] (already sigmoid-ed), gy [B,O] -> (gx [B,k], gl [O,2^k]).
+    gl[d, addr_b] += gy[b,d] * scale (dwn_stable_node.py:170-172)."""
+    gy64 = np.asarray(gy, dtype=np.float64)
+    O, L = np.asarray(luts).shape
+    addr = dwn_address(xk)
+    D = stable_coefficients(luts, scale)
+    gx = np.einsum("bd,dlb->bl", gy64, D[:, :, addr])
+    gl = np.zeros((O, L), dtype=np.float64)
+    np.add.at(gl, (slice(None), addr), gy64.T * float(scale))
+    return gx, gl
+
+
+def stable_layer_backward(x, idx, raw_luts, gy, scale):
+    """Layer adjoint down to the raw tables: x [B,I], idx [N,k], raw_luts [N,O,L], gy [B,N,O],
+    scale [N] -> gx [B,I], graw [N,O,L] (float64).  graw = gl * s (1 - s), the sigmoid applied by
+    forward_train outside the autograd Function (dwn_stable_node.py:309-316)."""
+    x = np.asarray(x)
+    luts = table_sigmoid(raw_luts)
+    gy64 = np.asarray(gy, dtype=np.float64)
+    scale = np.broadcast_to(np.asarray(scale, dtype=np.float64), (luts.shape[0],))
+    B, I = x.shape
+    N, O, L = luts.shape
+    addr = dwn_address(gather_forward(x, idx))
+    D = stable_coefficients(luts, scale[:, None])  # [N,O,k,L]
+    n_ar = np.arange(N)[None, :]
+    gm = np.einsum("bnd,bndl->bnl", gy64, D[n_ar, :, :, addr])
+    gx = gather_backward(gm, idx, I)
+    gl = np.zeros((N, O, L), dtype=np.float64)
+    b_ar = np.arange(B)[:, None]
+    for d in range(O):
+        np.add.at(gl[:, d, :], (np.broadcast_to(n_ar, addr.shape), addr), gy64[b_ar, n_ar, d] * scale[None, :])
+    return gx, gl * luts * (1.0 - luts)
+
+
+# ----------------------------------------------------------------------------
+# f1  Hybrid node                        hybrid_node.py:137-204, hybrid_cuda_kernel.cu:38-126
+# ----------------------------------------------------------------------------
+
+HYBRID_EPS = 1e-8  # hybrid_node.py:166
+
+
+def hybrid_backward(xk, luts, gy, dtype=np.float64):
+    """Probabilistic gradients of a thresholded lookup: xk [B,k], luts [O,2^k], gy [B,O] ->
+    (gx [B,k], gl [O,2^k]).  Vectorised form of HybridFunctionCPU.backward: p[b,a] = prod_j
+    (x_j a_j + (1-x_j)(1-a_j)); gl = (p^T gy)^T; gx[b,l] = sum_d gy[b,d] sum_a luts[d,a] p[b,a]
+    (a_l - x_l) / (x_l (1 - x_l) + eps).  Because of eps an input that is exactly 0 or 1 gets a zero
+    gradient, not the one-sided derivative."""
+    x = np.asarray(xk, dtype=dtype)
+    luts = np.asarray(luts, dtype=dtype)
+    gy = np.asarray(gy, dtype=dtype)
+    k = x.shape[1]
+    L = luts.shape[1]
+    combos = np.array([[(a >> j) & 1 for j in range(k)] for a in range(L)], dtype=dtype)
+    xe = x[:, None, :]
+    ae = combos[None, :, :]
+    p = np.prod(xe * ae + (1 - xe) * (1 - ae), axis=2)  # [B,L]
+    gl = (p.T @ gy).T
+    deriv = (ae - xe) / (xe * (1 - xe) + dtype(HYBRID_EPS))  # [B,L,k]
+    weighted = p[:, :, None] * deriv
+    gx = np.einsum("bd,da,bal->bl", gy, luts, weighted)
+    return gx, gl
+
+
+def hybrid_layer_backward(x, idx, raw_luts, gy):
+    """x [B,I], idx [N,k], raw_luts [N,O,L], gy [B,N,O] -> gx [B,I], graw [N,O,L] (float64);
+    graw carries the sigmoid of forward_train (hybrid_node.py:327-332)."""
+    x = np.asarray(x)
+    luts = table_sigmoid(raw_luts)
+    gy = np.asarray(gy, dtype=np.float64)
+    m = gather_forward(x, idx)
+    gm = np.zeros(m.shape, dtype=np.float64)
+    gl = np.zeros(luts.shape, dtype=np.float64)
+    for n in range(luts.shape[0]):
+        gm[:, n], gl[n] = hybrid_backward(m[:, n], luts[n], gy[:, n])
+    return gather_backward(gm, idx, x.shape[1]), gl * luts * (1.0 - luts)
 
 
 # ----------------------------------------------------------------------------

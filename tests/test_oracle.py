@@ -266,3 +266,135 @@ def test_group_sum(golden):
     assert np.array_equal(orc.group_sum(ones, 3, 1.0), np.full((2, 3), 4.0))
     assert np.array_equal(orc.group_sum(ones, 3, 2.0), np.full((2, 3), 2.0))
     assert np.array_equal(orc.group_sum(np.ones((1, 10), np.float32), 4, 1.0), [[3, 3, 3, 1]])  # zero padded
+
+
+# ------------------------------------------------------------------ gradient-stabilised DWN node
+def _stable_literal(xk, luts, gy, scale):
+    """Per-thread loop of the device kernel (dwn_stable_cuda_kernel.cu:84-172), accumulating in Python floats."""
+    B, k = xk.shape
+    O, L = luts.shape
+    gx = np.zeros((B, k))
+    gl = np.zeros((O, L))
+    for b in range(B):
+        addr = sum(1 << i for i in range(k) if xk[b, i] >= 0.5)
+        for d in range(O):
+            gl[d, addr] += float(gy[b, d]) * scale
+        for l in range(k):
+            mask = (L - 1) & ~(1 << l)
+            for d in range(O):
+                tot = 0.0
+                for kap in range(L):
+                    h = bin((addr & mask) ^ (kap & mask)).count("1")
+                    tot += (1.0 if (kap >> l) & 1 else -1.0) * float(luts[d, kap]) / (h + 1.0)
+                gx[b, l] += tot * float(gy[b, d]) * scale
+    return gx, gl
+
+
+def test_stable_coefficients_are_the_beta_integral_of_the_efd_coefficients():
+    """1/(h+1) = integral of beta^h over [0,1]: the stabilised weights are the pinned EFD weights
+    (alpha = 1) integrated over beta; Gauss-Legendre with 4 nodes is exact up to degree 7 > k-1."""
+    rng = np.random.default_rng(5)
+    nodes, weights = np.polynomial.legendre.leggauss(4)
+    for k in (1, 2, 4, 6):
+        luts = rng.random((3, 1 << k))
+        want = sum(w / 2 * orc.efd_coefficients(luts, 1.0, (t + 1) / 2) for t, w in zip(nodes, weights))
+        assert np.allclose(orc.stable_coefficients(luts, 1.7), 1.7 * want, rtol=1e-12, atol=1e-13)
+
+
+def test_stable_backward_special_cases_and_literal_loop():
+    rng = np.random.default_rng(6)
+    for B, k, O in [(7, 3, 2), (5, 1, 1), (4, 4, 1)]:
+        xk = rng.random((B, k)).astype(np.float32)
+        luts = rng.random((O, 1 << k)).astype(np.float32)
+        gy = rng.standard_normal((B, O)).astype(np.float32)
+        gx, gl = orc.stable_backward(xk, luts, gy, 1.25)
+        lx, ll = _stable_literal(xk, luts, gy, 1.25)
+        assert np.allclose(gx, lx, rtol=1e-12, atol=1e-12) and np.allclose(gl, ll, rtol=1e-12, atol=1e-12)
+        assert np.allclose(gl.sum(1), 1.25 * gy.astype(np.float64).sum(0))  # every sample lands in one bin
+        assert np.allclose(orc.stable_backward(xk, np.full_like(luts, 0.3), gy, 1.25)[0], 0.0, atol=1e-15)
+        if k == 1:  # no other input: the plain difference of the two entries
+            assert np.allclose(gx[:, 0], 1.25 * gy[:, 0].astype(np.float64) * (float(luts[0, 1]) - float(luts[0, 0])))
+    # k = 2 by hand: same other bit weighs 1, flipped other bit weighs 1/2
+    luts = np.array([[0.1, 0.4, 0.8, 0.3]])
+    gx, _ = orc.stable_backward(np.array([[0.9, 0.2]], dtype=np.float32), luts, np.array([[2.0]]), 1.0)
+    assert np.allclose(gx, [[2.0 * ((0.4 - 0.1) + (0.3 - 0.8) / 2), 2.0 * ((0.3 - 0.4) + (0.8 - 0.1) / 2)]])
+
+
+def test_stable_layer_equals_per_node_loop_with_sigmoid_chain():
+    rng = np.random.default_rng(7)
+    B, I, N, k, O = 9, 11, 6, 3, 2
+    x = rng.random((B, I)).astype(np.float32)
+    idx = rng.integers(0, I, (N, k))
+    raw = rng.standard_normal((N, O, 1 << k)).astype(np.float32)
+    gy = rng.standard_normal((B, N, O)).astype(np.float32)
+    scale = rng.random(N) + 0.5
+    gx, graw = orc.stable_layer_backward(x, idx, raw, gy, scale)
+    wx = np.zeros((B, I))
+    for n in range(N):
+        s = torch.sigmoid(torch.tensor(raw[n], dtype=torch.float64)).requires_grad_()
+        gxn, gln = orc.stable_backward(x[:, idx[n]], s.detach().numpy(), gy[:, n], scale[n])
+        np.add.at(wx, (slice(None), idx[n]), gxn)
+        t = torch.tensor(raw[n], dtype=torch.float64, requires_grad=True)
+        torch.sigmoid(t).backward(torch.tensor(gln))  # the sigmoid autograd applies outside the Function
+        assert np.allclose(graw[n], t.grad.numpy(), rtol=1e-12, atol=1e-14)
+    assert np.allclose(gx, wx, rtol=1e-12, atol=1e-13)
+
+
+# ------------------------------------------------------------------ hybrid node
+def _hybrid_literal(xk, luts, gy):
+    """Per-thread loops of hybrid_backward_input_kernel / hybrid_backward_lut_kernel
+    (hybrid_cuda_kernel.cu:38-126) in Python floats."""
+    B, k = xk.shape
+    O, L = luts.shape
+    gx = np.zeros((B, k))
+    gl = np.zeros((O, L))
+    for b in range(B):
+        xs = [float(v) for v in xk[b]]
+        for a in range(L):
+            p = 1.0
+            for i in range(k):
+                ai = (a >> i) & 1
+                p *= xs[i] * ai + (1.0 - xs[i]) * (1.0 - ai)
+            for d in range(O):
+                gl[d, a] += p * float(gy[b, d])
+                for l in range(k):
+                    al = (a >> l) & 1
+                    gx[b, l] += p * (al - xs[l]) / (xs[l] * (1.0 - xs[l]) + 1e-8) * float(luts[d, a]) * float(gy[b, d])
+    return gx, gl
+
+
+def test_hybrid_backward_is_the_gradient_of_the_multilinear_interpolation():
+    rng = np.random.default_rng(8)
+    for B, k, O in [(6, 3, 2), (5, 6, 1), (4, 1, 3)]:
+        xk = (0.05 + 0.9 * rng.random((B, k)))
+        luts = rng.random((O, 1 << k))
+        gy = rng.standard_normal((B, O))
+        gx, gl = orc.hybrid_backward(xk, luts, gy)
+        lx, ll = _hybrid_literal(xk, luts, gy)
+        assert np.allclose(gx, lx, rtol=1e-11, atol=1e-12) and np.allclose(gl, ll, rtol=1e-11, atol=1e-12)
+        # interior points: eps only perturbs by <= 1e-8 / (x (1 - x)) relative
+        x = torch.tensor(xk, requires_grad=True)
+        t = torch.tensor(luts, requires_grad=True)
+        combos = torch.tensor([[(a >> j) & 1 for j in range(k)] for a in range(1 << k)], dtype=torch.float64)
+        p = torch.prod(x[:, None, :] * combos + (1 - x[:, None, :]) * (1 - combos), dim=2)
+        (p @ t.T).backward(torch.tensor(gy))
+        assert np.allclose(gx, x.grad.numpy(), rtol=1e-6, atol=1e-9)
+        assert np.allclose(gl, t.grad.numpy(), rtol=1e-12, atol=1e-13)
+        assert np.allclose(gl.sum(1), gy.sum(0))  # the product weights of a sample sum to one
+
+
+def test_hybrid_backward_is_zero_at_binary_inputs():
+    rng = np.random.default_rng(9)
+    xk = rng.integers(0, 2, (8, 4)).astype(np.float32)
+    luts = rng.random((2, 16)).astype(np.float32)
+    gy = rng.standard_normal((8, 2)).astype(np.float32)
+    gx, gl = orc.hybrid_backward(xk, luts, gy)
+    assert np.all(gx == 0.0)  # p * (a_l - x_l) vanishes term by term and the denominator is eps, not 0
+    addr = orc.dwn_address(xk)
+    want = np.zeros((2, 16))
+    np.add.at(want, (slice(None), addr), gy.astype(np.float64).T)
+    assert np.allclose(gl, want)  # at a corner the weights are the indicator of the address
+    mixed = xk.copy()
+    mixed[:, 1] = 0.3
+    gm, _ = orc.hybrid_backward(mixed, luts, gy)
+    assert np.all(gm[:, [0, 2, 3]] == 0.0) and np.all(gm[:, 1] != 0.0)
