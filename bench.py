@@ -114,16 +114,17 @@ def run_stack(args):
     params = [p for layer in layers for p in layer.bank_parameters()]
     opt = torch.optim.Adam(params, lr=1e-3)
     from difflut_amd.layers import DWNStack
-    stack = DWNStack(layers).train()  # same layers; bit-planes / tile-major gradients between them
+    # same layers; thermometer code and activations as bit-planes, tile-major gradients between layers
+    stack = DWNStack(layers, encoder=enc).train()
 
     def step():
         opt.zero_grad(set_to_none=True)
-        h = enc.encode(x)
         if args.layer_by_layer:
+            h = enc.encode(x)
             for layer in layers:
                 h = layer(h)
         else:
-            h = stack(h)
+            h = stack(x)
         loss = torch.nn.functional.cross_entropy(head(h), labels)
         loss.backward()
         opt.step()

@@ -51,6 +51,7 @@ SIGNATURES = {
     "dl_hard_select_fwd": (_I, [_P, _P, _P, _I, _I, _I, _P]),
     "dl_hard_select_bwd": (_I, [_P, _P, _P, _P, _I, _I, _I, _P]),
     "dl_thermometer_encode": (_I, [_P, _P, _P, _I, _I, _I, _P]),
+    "dl_thermometer_planes": (_I, [_P, _P, _P, _I, _I, _I, _P]),
     "dl_group_sum_fwd": (_I, [_P, _P, _I, _I, _I, _F, _P]),
     "dl_group_sum_bwd": (_I, [_P, _P, _I, _I, _I, _F, _P]),
     "dl_profile_enable": (_I, [_I]),

@@ -58,6 +58,46 @@ __global__ __launch_bounds__(256) void thermometer_kernel(const float *__restric
     bits[gid] = x[b * (FB / nbits) + f] > thr[fb] ? 1.0f : 0.0f;  // strict compare
 }
 
+// Thermometer bits as bit-planes for a following DWN layer: word (t, f*nbits + j) holds, in bit r,
+// (x[64t + r][f] > thr[f][j]).  Block = (64 features, batch tile t): the x tile is read row-wise
+// (coalesced) into LDS, then each wavefront takes 16 features with lane = row, one ballot per
+// threshold.  A lane keeps the words whose index is congruent to it and the wavefront stores 64
+// consecutive words at a time.  Rows past B read as "not greater".
+__global__ __launch_bounds__(256) void thermometer_planes_kernel(const float *__restrict__ x, const float *__restrict__ thr,
+                                                                  unsigned long long *__restrict__ planes, int B, int F,
+                                                                  int nbits) {
+    __shared__ float tile[64][65];  // [feature][row]
+    const int t = blockIdx.y, f0 = blockIdx.x * 64;
+    for (int e = threadIdx.x; e < 4096; e += 256) {
+        const int r = e >> 6, c = e & 63;
+        const int b = t * 64 + r;
+        tile[c][r] = (b < B && f0 + c < F) ? x[(size_t)b * F + f0 + c] : -INFINITY;
+    }
+    __syncthreads();
+    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int fbeg = f0 + w * 16, fend = min(F, fbeg + 16);
+    if (fbeg >= fend) return;
+    const int words = (fend - fbeg) * nbits;
+    unsigned long long *out = planes + (size_t)t * F * nbits + (size_t)fbeg * nbits;
+    const float *th = thr + (size_t)fbeg * nbits;
+    float mythr = 0.0f;  // one threshold per lane for the current run of 64 words, handed round below
+    unsigned long long mine = 0;
+    int q = 0;
+    for (int ff = 0; ff < fend - fbeg; ++ff) {
+        const float v = tile[w * 16 + ff][lane];
+        for (int j = 0; j < nbits; ++j, ++q) {
+            const int slot = q & 63;
+            if (slot == 0) mythr = q + lane < words ? th[q + lane] : 0.0f;
+            const float t_q = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mythr), slot));
+            const unsigned long long mask = __ballot(v > t_q);  // strict compare, as the encoder
+            if (slot == lane) mine = mask;
+            if (slot == 63 || q == words - 1) {
+                if (lane <= slot) out[q - slot + lane] = mine;
+            }
+        }
+    }
+}
+
 // One wavefront per (row, group): sum a contiguous run of group_size features.
 __global__ __launch_bounds__(256) void group_sum_fwd_kernel(const float *__restrict__ x, float *__restrict__ y, int B,
                                                              int F, int groups, int gsize, float inv_tau) {
@@ -128,6 +168,17 @@ extern "C" int dl_thermometer_encode(const float *x, const float *thr, float *bi
     if (B <= 0 || F <= 0 || nbits <= 0) return DL_ERR_SHAPE;
     const long long total = (long long)B * F * nbits;
     thermometer_kernel<<<dl_ceil_div(total, 256), 256, 0, (hipStream_t)stream>>>(x, thr, bits, total, F * nbits, nbits);
+    return dl_launch_status();
+}
+
+extern "C" int dl_thermometer_planes(const float *x, const float *thr, void *planes, int B, int F, int nbits,
+                                     void *stream) {
+    if (!x || !thr || !planes) return DL_ERR_NULL;
+    if (B <= 0 || F <= 0 || nbits <= 0) return DL_ERR_SHAPE;
+    hipStream_t s = (hipStream_t)stream;
+    DL_TIMED("thermometer_planes", s,
+             (thermometer_planes_kernel<<<dim3(dl_ceil_div(F, 64), dl_ceil_div(B, 64)), 256, 0, s>>>(
+                 x, thr, (unsigned long long *)planes, B, F, nbits)));
     return dl_launch_status();
 }
 

@@ -1,0 +1,226 @@
+"""Convolutional LUT layer: every output channel is a small tree of LUT layers applied to each patch.
+
+Constructor, configuration object, sub-module layout (`first_layer_chunks`, `trees`, hence the
+state-dict keys) and forward semantics follow difflut/layers/convolutional.py:13-267.  What differs
+is the execution.  The reference loops over chunks of first layers and then over every tree and
+every tree layer, out_channels * tree_depth tiny layer calls per forward.  Here all trees' layers of
+one depth level run as ONE block-diagonal layer call: level l has out_channels * n^(depth-l) nodes,
+tree t's nodes read the columns of tree t only (its index table shifted by t times the level's
+width), and for DWN nodes the levels are chained (bit-planes between levels, tile-major gradients
+back).  The node parameters of a level live in one [nodes, ...] tensor; the per-node Parameters of
+the sub-layers are views of it.
+"""
+import torch
+import torch.nn as nn
+
+from .. import _native, ops
+from ..nodes.node_config import NodeConfig
+from ..registry import register_convolutional_layer
+from .base_layer import LUTLayerMixin, ParameterBank
+from .layer_config import GroupedInputConfig
+from .random_layer import RandomLayer
+
+_BANKED = {"dwn": ("luts",), "probabilistic": ("raw_weights",), "dwn_stable": ("raw_luts", "gradient_scale"),
+           "hybrid": ("raw_luts",)}
+
+
+class ConvolutionConfig:
+    def __init__(self, tree_depth=2, in_channels=None, out_channels=None, receptive_field=5, stride=1, padding=0,
+                 chunk_size=32, seed=42):
+        assert in_channels is not None, "in_channels must be specified"
+        assert out_channels is not None, "out_channels must be specified"
+        self.tree_depth = tree_depth
+        self.in_channels = in_channels
+        self.out_channels = out_channels
+        self.receptive_field = receptive_field
+        self.stride = stride
+        self.padding = padding
+        self.chunk_size = chunk_size
+        self.seed = seed
+
+
+def _pair(v):
+    return (v, v) if isinstance(v, int) else v
+
+
+@register_convolutional_layer("convolutional")
+class ConvolutionalLayer(LUTLayerMixin, nn.Module):
+    def __init__(self, convolution_config, node_type, node_kwargs, layer_type, n_inputs_per_node=6, layer_config=None,
+                 flip_probability=None, grad_stabilization=None, grad_target_std=None, grad_subtract_mean=None,
+                 grad_epsilon=None, grouped_connections=False, ensure_full_coverage=False):
+        super().__init__()
+        self._init_lut_layer_mixin(layer_config, flip_probability, grad_stabilization, grad_target_std,
+                                   grad_subtract_mean, grad_epsilon)
+        cfg = convolution_config
+        self.tree_depth = cfg.tree_depth
+        self.in_channels, self.out_channels = cfg.in_channels, cfg.out_channels
+        self.receptive_field = _pair(cfg.receptive_field)
+        self.input_size = self.in_channels * self.receptive_field[0] * self.receptive_field[1]
+        self.stride, self.padding = _pair(cfg.stride), _pair(cfg.padding)
+        self.node_type, self.layer_type = node_type, layer_type
+        self.n_inputs_per_node = n_inputs_per_node
+        self.seed = cfg.seed
+        self.chunk_size = min(cfg.chunk_size, self.out_channels)
+        # nodes per tree at each level: n^depth, ..., n, 1
+        self.hidden_layers = [n_inputs_per_node ** (self.tree_depth - i) for i in range(self.tree_depth + 1)]
+        grouped = None
+        if grouped_connections:
+            assert self.input_size % self.in_channels == 0, "Input size must be divisible by number of groups."
+            grouped = GroupedInputConfig(n_groups=self.in_channels, input_size=self.input_size,
+                                         output_trees=self.out_channels, luts_per_tree=self.hidden_layers[0],
+                                         bits_per_node=n_inputs_per_node, seed=self.seed,
+                                         ensure_full_coverage=ensure_full_coverage)
+        # sub-modules in the reference's construction order (node parameters draw from the global generator)
+        self.first_layer_chunks = nn.ModuleList()
+        for start in range(0, self.out_channels, self.chunk_size):
+            end = min(start + self.chunk_size, self.out_channels)
+            self.first_layer_chunks.append(layer_type(
+                input_size=self.input_size, output_size=self.hidden_layers[0] * (end - start), node_type=node_type,
+                node_kwargs=node_kwargs, mapping_indices=grouped.get_mapping_indices(start, end) if grouped else None))
+        self.trees = nn.ModuleList()
+        for _ in range(self.out_channels):
+            tree, width = nn.ModuleList(), self.hidden_layers[0]
+            for size in self.hidden_layers[1:]:
+                tree.append(layer_type(input_size=width, output_size=size, node_type=node_type, node_kwargs=node_kwargs))
+                width = size
+            self.trees.append(tree)
+        self.unfold = nn.Unfold(kernel_size=self.receptive_field, padding=self.padding, stride=self.stride)
+        self._kind = self._detect_kind()
+        self._level_banks, self._plans, self._plan_key = [], None, None
+        if self._kind is not None:
+            self._tie_levels()
+
+    # ------------------------------------------------------------------ block-diagonal levels
+    def _sublayers(self):
+        yield from self.first_layer_chunks
+        for tree in self.trees:
+            yield from tree
+
+    def _detect_kind(self):
+        """The fused kind shared by every sub-layer, or None (then the reference's loop runs)."""
+        kinds = set()
+        for layer in self._sublayers():
+            if not isinstance(layer, RandomLayer) or layer.output_dim_per_node != 1:
+                return None
+            kinds.add(layer._fused)
+        kind = kinds.pop() if len(kinds) == 1 else None
+        return kind if kind in _BANKED else None
+
+    def _level_layers(self, level):
+        """Sub-layers of a depth level in column order: level 0 the chunks, level l tree by tree."""
+        return list(self.first_layer_chunks) if level == 0 else [tree[level - 1] for tree in self.trees]
+
+    def _tie_levels(self):
+        self._level_banks = []
+        for level in range(self.tree_depth + 1):
+            nodes = [node for layer in self._level_layers(level) for node in layer.nodes]
+            self._level_banks.append({name: ParameterBank(nodes, name) for name in _BANKED[self._kind]})
+
+    def _apply(self, fn, *args, **kwargs):
+        grads = [{name: bank.flat.grad for name, bank in banks.items()} for banks in self._level_banks]
+        for banks in self._level_banks:
+            for bank in banks.values():
+                bank.flat.grad = None
+        super()._apply(fn, *args, **kwargs)
+        for banks, kept in zip(self._level_banks, grads):
+            for name, bank in banks.items():
+                bank.tie(keep_grad=None if kept[name] is None else fn(kept[name]))
+        self._plans = None
+        return self
+
+    def bank_parameters(self):
+        """One leaf [nodes of the level, ...] per depth level and node parameter (what the fused calls
+        differentiate); hand these to an optimizer instead of the per-node `parameters()`."""
+        return [bank.tensor() for banks in self._level_banks for bank in banks.values()]
+
+    def _level_plans(self, device):
+        tables = [layer._mapping_indices for layer in self._sublayers()]
+        key = (str(device),) + tuple((t.data_ptr(), t._version) for t in tables)
+        if self._plans is None or self._plan_key != key:
+            plans = []
+            for level in range(self.tree_depth + 1):
+                layers = self._level_layers(level)
+                if level == 0:
+                    idx = torch.cat([layer._mapping_indices.to(torch.int32) for layer in layers])
+                    width = self.input_size
+                else:
+                    per_tree = self.hidden_layers[level - 1]
+                    idx = torch.cat([layer._mapping_indices.to(torch.int32) + t * per_tree for t, layer in enumerate(layers)])
+                    width = per_tree * self.out_channels
+                plans.append(ops.MappingPlan(idx.to(device), width))
+            self._plans, self._plan_key = plans, key
+        return self._plans
+
+    def _run_levels(self, patches):
+        """patches [rows, input_size] -> [rows, out_channels] through the depth levels."""
+        plans = self._level_plans(patches.device)
+        banks = [{name: bank.tensor() for name, bank in level.items()} for level in self._level_banks]
+        firsts = [self._level_layers(level)[0].nodes[0] for level in range(self.tree_depth + 1)]
+        kind, h = self._kind, patches
+        if kind == "dwn" and self.training and self.n_inputs_per_node <= ops.FAST_K:
+            scalars = [node.efd_scalars() for node in firsts]
+            return ops.DWNStackFunction.apply(h, None, plans, scalars, *[b["luts"] for b in banks])
+        for plan, bank, node in zip(plans, banks, firsts):
+            if kind == "dwn":
+                if self.training:
+                    h = ops.DWNLayerFunction.apply(h, bank["luts"], plan, *node.efd_scalars())
+                else:
+                    h = ops.dwn_layer_eval(h, bank["luts"].detach(), plan)
+            elif kind == "probabilistic":
+                if self.training:
+                    h = ops.ProbLayerFunction.apply(h, bank["raw_weights"], plan, node.temperature_value())
+                else:
+                    h = ops.prob_layer_eval(h, bank["raw_weights"].detach(), plan, node.temperature_value())
+            elif not self.training:
+                with torch.no_grad():
+                    h = ops.dwn_layer_eval(h, ops.TableSigmoidFunction.apply(bank["raw_luts"]), plan)
+            elif kind == "hybrid":
+                h = ops.HybridLayerFunction.apply(h, ops.TableSigmoidFunction.apply(bank["raw_luts"]), plan)
+            else:
+                h = ops.DWNStableLayerFunction.apply(h, ops.TableSigmoidFunction.apply(bank["raw_luts"]),
+                                                     bank["gradient_scale"].detach(), plan)
+        return h
+
+    def _loop_trees(self, patches):
+        """The reference's loop (convolutional.py:214-242), for sub-layers without a fused kernel."""
+        out = torch.empty(patches.shape[0], self.out_channels, device=patches.device)
+        tree_idx = 0
+        for chunk_idx, chunk in enumerate(self.first_layer_chunks):
+            start = chunk_idx * self.chunk_size
+            count = min(start + self.chunk_size, self.out_channels) - start
+            first = chunk(patches).view(patches.shape[0], count, self.hidden_layers[0])
+            for local in range(count):
+                h = first[:, local, :]
+                for layer in self.trees[tree_idx]:
+                    h = layer(h)
+                out[:, tree_idx] = h.squeeze(-1)
+                tree_idx += 1
+        return out
+
+    # ------------------------------------------------------------------ interface
+    def forward(self, x):
+        _native.require_device(x)
+        batch = x.shape[0]
+        patches = self.unfold(x)  # (batch, channels * kh * kw, positions)
+        positions = patches.shape[2]
+        patches = patches.transpose(1, 2).contiguous().view(-1, self.input_size)
+        if self.training and self.flip_probability > 0.0:
+            patches = self._apply_bit_flip(patches)
+        out = self._run_levels(patches) if self._kind is not None else self._loop_trees(patches)
+        out = out.view(batch, positions, self.out_channels).transpose(1, 2)
+        out_h = (x.shape[2] + 2 * self.padding[0] - self.receptive_field[0]) // self.stride[0] + 1
+        out_w = (x.shape[3] + 2 * self.padding[1] - self.receptive_field[1]) // self.stride[1] + 1
+        out = out.reshape(batch, self.out_channels, out_h, out_w)
+        if self.grad_stabilization != "none" and self.training and out.requires_grad:
+            def hook(grad):
+                return self._apply_gradient_stabilization(grad.reshape(grad.shape[0], -1)).view(grad.shape)
+            out.register_hook(hook)
+        return out
+
+    def __repr__(self):
+        return (f"ConvolutionalLUTLayer(\n  receptive_field={self.receptive_field}, stride={self.stride}, "
+                f"padding={self.padding}\n  in_channels={self.in_channels}, out_channels={self.out_channels}\n"
+                f"  tree_architecture={self.hidden_layers}\n  node_type={self.node_type}, layer_type={self.layer_type}\n"
+                f"  n_inputs_per_node={self.n_inputs_per_node}, tree_depth={self.tree_depth}\n"
+                f"  total_trees={len(self.trees)}, chunk_size={self.chunk_size}, "
+                f"num_chunks={len(self.first_layer_chunks)}\n)")

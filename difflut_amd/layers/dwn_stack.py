@@ -4,6 +4,7 @@ The reference runs a stack layer by layer (`difflut/layers/random_layer.py:306-3
 writing its `[batch, nodes]` fp32 output for the next one to threshold.  The tables, mappings and
 state-dict keys of the wrapped layers are untouched; only the execution of the training forward
 and backward changes (bit-planes between layers, tile-major gradients between layers)."""
+import torch
 import torch.nn as nn
 
 from .. import ops
@@ -17,9 +18,13 @@ class DWNStack(nn.Module):
     with at most 6 inputs and matching widths; anything else (and eval mode) runs the members
     one after the other."""
 
-    def __init__(self, layers):
+    def __init__(self, layers, encoder=None):
+        """`encoder`: a fitted, flattening ThermometerEncoder whose code feeds the first layer; the stack
+        then takes the raw features and equals `layerN(... layer1(encoder.encode(x)))`.  On the chained
+        path the code is never written as a [batch, features * bits] fp32 tensor."""
         super().__init__()
         self.layers = nn.ModuleList(layers)
+        self.encoder = encoder
 
     def _chainable(self):
         width = None
@@ -31,13 +36,31 @@ class DWNStack(nn.Module):
             width = layer.output_size * layer.output_dim_per_node
         return len(self.layers) > 0
 
+    def _fusable_encoder(self, x):
+        from ..encoder.thermometer import ThermometerEncoder
+
+        enc = self.encoder
+        return (isinstance(enc, ThermometerEncoder) and enc.flatten and enc.thresholds is not None and x.dim() == 2
+                and torch.is_tensor(x) and x.shape[1] * enc.num_bits == self.layers[0].input_size)
+
     def forward(self, x):
         if not (self.training and self._chainable()):
+            if self.encoder is not None:
+                x = self.encoder.encode(x)
             for layer in self.layers:
                 x = layer(x)
             return x
-        self.layers[0]._validate_input_dims(x)
+        thresholds = None
+        if self.encoder is not None:
+            if self._fusable_encoder(x):
+                thresholds = self.encoder.thresholds.to(x.device)
+                if x.shape[0] == 0:
+                    raise ValueError(f"BaseLUTLayer requires non-empty batch, got batch_size={x.shape[0]}")
+            else:
+                x = self.encoder.encode(x)
+        if thresholds is None:
+            self.layers[0]._validate_input_dims(x)
         plans = [layer.mapping_plan() for layer in self.layers]
         scalars = [layer.nodes[0].efd_scalars() for layer in self.layers]
         luts = [layer._banks["luts"].tensor() for layer in self.layers]
-        return ops.DWNStackFunction.apply(x, plans, scalars, *luts)
+        return ops.DWNStackFunction.apply(x, thresholds, plans, scalars, *luts)

@@ -139,14 +139,26 @@ class DWNStackFunction(torch.autograd.Function):
     first layer's input gradient, if asked for).  Same arithmetic as calling the layers one by one."""
 
     @staticmethod
-    def forward(ctx, x, plans, scalars, *luts):
-        nat.require_device(x, *luts)
+    def forward(ctx, x, thresholds, plans, scalars, *luts):
+        """`thresholds` [F, nbits] (or None): x is raw data [B, F] and the first layer reads its
+        thermometer code, produced directly as bit-planes; x then gets no gradient (the code is a
+        step function of it)."""
+        nat.require_device(x, thresholds, *luts)
         x = _f32(x)
         luts = tuple(_f32(t) for t in luts)
         B, width = x.shape
         lib = nat.lib()
-        planes = _bytes(lib.dl_dwn_planes_bytes(B, width), x.device)
-        nat.check(lib.dl_dwn_pack_planes(nat.ptr(x), nat.ptr(planes), B, width, nat.stream()))
+        if thresholds is None:
+            planes = _bytes(lib.dl_dwn_planes_bytes(B, width), x.device)
+            nat.check(lib.dl_dwn_pack_planes(nat.ptr(x), nat.ptr(planes), B, width, nat.stream()))
+        else:
+            thr = _f32(thresholds)
+            if thr.dim() != 2 or thr.shape[0] != width:
+                raise RuntimeError(f"thresholds {tuple(thr.shape)} do not match {width} features")
+            nbits = thr.shape[1]
+            planes = _bytes(lib.dl_dwn_planes_bytes(B, width * nbits), x.device)
+            nat.check(lib.dl_thermometer_planes(nat.ptr(x), nat.ptr(thr), nat.ptr(planes), B, width, nbits, nat.stream()))
+            width *= nbits
         saved, dims_all, y = [], [], None
         for l, (plan, lut) in enumerate(zip(plans, luts)):
             N, O, L = lut.shape
@@ -166,6 +178,7 @@ class DWNStackFunction(torch.autograd.Function):
             planes, width = nxt, N * O
         ctx.save_for_backward(*luts, *saved)
         ctx.plans, ctx.scalars, ctx.dims_all = plans, scalars, dims_all
+        ctx.encoded = thresholds is not None
         return y
 
     @staticmethod
@@ -183,7 +196,8 @@ class DWNStackFunction(torch.autograd.Function):
                 gx = torch.empty(lib.dl_dwn_tiled_bytes(B, I) // 4, dtype=torch.float32, device=g.device)
                 gx_tiled = 1
             else:
-                gx = torch.empty((B, I), dtype=torch.float32, device=g.device) if ctx.needs_input_grad[0] else None
+                want = ctx.needs_input_grad[0] and not ctx.encoded
+                gx = torch.empty((B, I), dtype=torch.float32, device=g.device) if want else None
                 gx_tiled = 0
             grads[l] = torch.empty_like(luts[l])
             ws = _bytes(lib.dl_dwn_bwd_workspace_bytes(*dims), g.device)
@@ -192,7 +206,7 @@ class DWNStackFunction(torch.autograd.Function):
                                                  nat.ptr(gx), gx_tiled, nat.ptr(grads[l]), nat.ptr(ws), ws.numel(), *dims,
                                                  nat.stream()))
             g, tiled = gx, gx_tiled
-        return (g, None, None, *grads)
+        return (g, None, None, None, *grads)
 
 
 def dwn_layer_eval(x, luts, plan):

@@ -225,6 +225,11 @@ int dl_hard_select_bwd(const float *gm, const int32_t *inv_ptr, const int32_t *i
  * ------------------------------------------------------------------------ */
 int dl_thermometer_encode(const float *x, const float *thr, float *bits, int B, int F, int nbits,
                           void *stream);
+/* The same comparison written as the bit-planes a chained DWN layer reads (dl_dwn_layer_fwd_planes,
+ * width F*nbits): no counterpart in the reference, which materialises the [B, F*nbits] fp32 tensor
+ * (thermometer.py:108-116) for the first layer to threshold again.  planes: dl_dwn_planes_bytes(B, F*nbits). */
+int dl_thermometer_planes(const float *x, const float *thr, void *planes, int B, int F, int nbits,
+                          void *stream);
 int dl_group_sum_fwd(const float *x, float *y, int B, int F, int groups, float tau, void *stream);
 int dl_group_sum_bwd(const float *gy, float *gx, int B, int F, int groups, float tau, void *stream);
 

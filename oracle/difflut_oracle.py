@@ -20,6 +20,8 @@ Pin status (see tests/test_oracle.py for the checks):
   group_sum ................. golden, reference unit-test values
   stable_coefficients/backward  integral of the pinned EFD coefficients over beta in [0,1] (1/(h+1) =
                               int beta^h), literal-loop restatement, k=1 and constant-table cases, histogram sum
+  conv_unfold/fold .......... torch.nn.functional.unfold/fold (library routines); conv_trees_* are loops over the
+                              pinned layer functions, checked against a hand-built two-tree case
   hybrid_backward ........... autograd of the multilinear interpolation for interior x, per-thread loop form
                               of the device kernels, exact zeros at x in {0,1}, partition of unity
 No function is left "parity unpinned".
@@ -442,3 +444,71 @@ def group_sum(x, k, tau=1.0):
     if F % k:
         x = np.pad(x, ((0, 0), (0, k - F % k)))
     return x.reshape(x.shape[0], k, -1).sum(-1, dtype=np.float32) / np.float32(tau)
+
+
+# ----------------------------------------------------------------------------
+# f4  Convolutional layer                layers/convolutional.py:194-267
+# ----------------------------------------------------------------------------
+
+
+def conv_unfold(x, receptive_field, stride, padding):
+    """x [B,C,H,W] -> patches [B*positions, C*kh*kw] (nn.Unfold, then transpose/flatten, convolutional.py:199-205)."""
+    p = torch.nn.functional.unfold(torch.as_tensor(np.asarray(x)), kernel_size=receptive_field, padding=padding, stride=stride)
+    return p.transpose(1, 2).reshape(-1, p.shape[1]).numpy()
+
+
+def conv_fold(gpatches, shape, receptive_field, stride, padding):
+    """Adjoint of conv_unfold: gpatches [B*positions, C*kh*kw] -> gx [B,C,H,W] (what autograd does for nn.Unfold)."""
+    B, C, H, W = shape
+    g = torch.as_tensor(np.asarray(gpatches))
+    g = g.reshape(B, -1, g.shape[1]).transpose(1, 2)
+    return torch.nn.functional.fold(g, (H, W), kernel_size=receptive_field, padding=padding, stride=stride).numpy()
+
+
+def conv_trees_forward(patches, chunks, trees, hidden0, layer_forward):
+    """The chunk / tree loops of ConvolutionalLayer.forward (convolutional.py:214-242).
+
+    chunks: [(idx, tables)] of the first-layer chunks; trees: per tree [(idx, tables)] of its later layers;
+    layer_forward(x, idx, tables) -> [rows, nodes].  Returns (out [rows, trees], the activations kept for the
+    backward)."""
+    rows = patches.shape[0]
+    out = np.zeros((rows, len(trees)), dtype=np.float32)
+    acts, t = [], 0
+    for idx, tab in chunks:
+        first = layer_forward(patches, idx, tab)
+        count = first.shape[1] // hidden0
+        first = first.reshape(rows, count, hidden0)
+        for local in range(count):
+            h = first[:, local, :]
+            kept = [h]
+            for idx_l, tab_l in trees[t]:
+                h = layer_forward(h, idx_l, tab_l)
+                kept.append(h)
+            out[:, t] = h[:, 0]
+            acts.append(kept)
+            t += 1
+    return out, acts
+
+
+def conv_trees_backward(patches, chunks, trees, hidden0, acts, gout, layer_backward):
+    """Adjoint of conv_trees_forward.  layer_backward(x, idx, tables, gy [rows, nodes]) -> (gx, gtables).
+    Returns (gpatches, chunk table gradients, per-tree table gradients)."""
+    rows = patches.shape[0]
+    gpatches = np.zeros(patches.shape, dtype=np.float64)
+    gchunks, gtrees, t = [], [], 0
+    for idx, tab in chunks:
+        count = np.asarray(tab).shape[0] // hidden0
+        gfirst = np.zeros((rows, count, hidden0), dtype=np.float64)
+        for local in range(count):
+            g = np.asarray(gout)[:, t:t + 1].astype(np.float64)
+            grads = []
+            for (idx_l, tab_l), x_l in zip(reversed(trees[t]), reversed(acts[t][:-1])):
+                g, gt = layer_backward(x_l, idx_l, tab_l, g)
+                grads.append(gt)
+            gtrees.append(list(reversed(grads)))
+            gfirst[:, local, :] = g
+            t += 1
+        gx, gt = layer_backward(patches, idx, tab, gfirst.reshape(rows, -1))
+        gpatches += gx
+        gchunks.append(gt)
+    return gpatches, gchunks, gtrees

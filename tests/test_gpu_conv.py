@@ -1,0 +1,167 @@
+"""GPU parity of the convolutional LUT layer (all trees of a depth level as one block-diagonal layer call)
+against the CPU oracle's chunk / tree loops over the same tables and index tables."""
+import warnings
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import difflut_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+def _build(node_name, depth, in_ch, out_ch, rf, stride, padding, chunk, n=6, grouped=False, seed=42, **node_kw):
+    from difflut_amd import REGISTRY
+    from difflut_amd.layers import ConvolutionConfig
+    from difflut_amd.nodes import NodeConfig
+    from difflut_amd.nodes.utils import uniform_init
+    cfg = ConvolutionConfig(tree_depth=depth, in_channels=in_ch, out_channels=out_ch, receptive_field=rf, stride=stride,
+                            padding=padding, chunk_size=chunk, seed=seed)
+    lo, hi = (-1.0, 2.0) if node_name == "dwn" else (-2.0, 2.0)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        node_cfg = NodeConfig(input_dim=n, output_dim=1, init_fn=uniform_init, init_kwargs={"a": lo, "b": hi}, **node_kw)
+        layer = REGISTRY.get_convolutional_layer("convolutional")(
+            convolution_config=cfg, node_type=REGISTRY.get_node(node_name), node_kwargs=node_cfg,
+            layer_type=REGISTRY.get_layer("random"), n_inputs_per_node=n, grouped_connections=grouped,
+            ensure_full_coverage=grouped)
+    return layer.to(DEV)
+
+
+def _tables(layer, pname):
+    """(chunks, trees) as the oracle wants them: [(idx, tables)] and per tree [(idx, tables)]."""
+    def one(sub):
+        idx = sub._mapping_indices.cpu().numpy().astype(np.int64)
+        tab = np.stack([getattr(node, pname).detach().cpu().numpy() for node in sub.nodes])
+        return idx, tab
+    return [one(c) for c in layer.first_layer_chunks], [[one(l) for l in tree] for tree in layer.trees]
+
+
+def _oracle_fns(kind, scale=1.25):
+    if kind == "dwn":
+        alpha, beta = np.float32(0.5 * 0.75 ** 5), np.float32(0.25 / 0.75)
+        return ("luts", lambda x, i, t: orc.dwn_layer_forward(x, i, t)[:, :, 0],
+                lambda x, i, t, g: orc.dwn_layer_backward(x, i, t, g[:, :, None], alpha, beta))
+    if kind == "probabilistic":
+        return ("raw_weights", lambda x, i, t: orc.prob_layer_forward(x, i, t)[:, :, 0],
+                lambda x, i, t, g: orc.prob_layer_backward(x, i, t, g[:, :, None]))
+    fwd = lambda x, i, t: orc.dwn_layer_forward(x, i, orc.table_sigmoid(t).astype(np.float32))[:, :, 0]
+    if kind == "dwn_stable":
+        return "raw_luts", fwd, lambda x, i, t, g: orc.stable_layer_backward(x, i, t, g[:, :, None], scale)
+    return "raw_luts", fwd, lambda x, i, t, g: orc.hybrid_layer_backward(x, i, t, g[:, :, None])
+
+
+CASES = [  # (kind, depth, in_ch, out_ch, rf, stride, padding, chunk, image)
+    ("dwn", 1, 1, 16, 3, 1, 0, 8, (4, 10, 10)),          # tests/test_layers/test_convolutional_learning.py:186-195
+    ("dwn", 2, 2, 5, 3, 1, 1, 2, (3, 7, 6)),             # ragged last chunk, padding
+    ("dwn", 2, 3, 4, (3, 2), (2, 1), (0, 1), 32, (2, 9, 8)),
+    ("probabilistic", 1, 1, 16, 3, 1, 0, 8, (3, 8, 8)),
+    ("probabilistic", 2, 2, 3, 2, 2, 0, 2, (2, 6, 6)),
+    ("dwn_stable", 2, 2, 4, 3, 1, 0, 3, (2, 6, 7)),
+    ("hybrid", 2, 1, 3, 3, 2, 1, 1, (3, 7, 7)),
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_conv_layer_forward_backward_against_tree_loops(case):
+    kind, depth, in_ch, out_ch, rf, stride, padding, chunk, (B, H, W) = case
+    torch.manual_seed(sum(case[1:4]) + B)
+    layer = _build(kind, depth, in_ch, out_ch, rf, stride, padding, chunk)
+    assert layer._kind == kind
+    layer.train()
+    pname, fwd, bwd = _oracle_fns(kind)
+    rng = np.random.default_rng(H * W + out_ch)
+    x = (0.02 + 0.96 * rng.random((B, in_ch, H, W))).astype(np.float32)
+    xt = torch.tensor(x, device=DEV, requires_grad=True)
+    y = layer(xt)
+    pair = lambda v: (v, v) if isinstance(v, int) else v
+    rf2, st2, pd2 = pair(rf), pair(stride), pair(padding)
+    oh, ow = (H + 2 * pd2[0] - rf2[0]) // st2[0] + 1, (W + 2 * pd2[1] - rf2[1]) // st2[1] + 1
+    assert y.shape == (B, out_ch, oh, ow)
+    chunks, trees = _tables(layer, pname)
+    patches = orc.conv_unfold(x, rf2, st2, pd2)
+    out, acts = orc.conv_trees_forward(patches, chunks, trees, layer.hidden_layers[0], fwd)
+    want = out.reshape(B, oh * ow, out_ch).transpose(0, 2, 1).reshape(B, out_ch, oh, ow)
+    if kind == "dwn":
+        assert np.array_equal(y.detach().cpu().numpy(), want)  # lookups only: bit-exact
+    else:
+        np.testing.assert_allclose(y.detach().cpu().numpy(), want, rtol=1e-5, atol=1e-6)
+    gy = rng.standard_normal(want.shape).astype(np.float32)
+    y.backward(torch.tensor(gy, device=DEV))
+    gout = gy.reshape(B, out_ch, oh * ow).transpose(0, 2, 1).reshape(-1, out_ch)
+    gp, gch, gtr = orc.conv_trees_backward(patches, chunks, trees, layer.hidden_layers[0], acts, gout, bwd)
+    gx = orc.conv_fold(gp, x.shape, rf2, st2, pd2)
+    # gradients pass through up to three levels; terms are O(1): rtol 1e-5 with a floor of 5e-6
+    np.testing.assert_allclose(xt.grad.cpu().numpy(), gx, rtol=1e-5, atol=5e-6)
+    for c, (sub, want_g) in enumerate(zip(layer.first_layer_chunks, gch)):
+        got = np.stack([getattr(node, pname).grad.cpu().numpy() for node in sub.nodes])
+        np.testing.assert_allclose(got, want_g, rtol=1e-5, atol=5e-6, err_msg=f"chunk {c}")
+    for t in (0, out_ch - 1):
+        for l, sub in enumerate(layer.trees[t]):
+            got = np.stack([getattr(node, pname).grad.cpu().numpy() for node in sub.nodes])
+            np.testing.assert_allclose(got, gtr[t][l], rtol=1e-5, atol=5e-6, err_msg=f"tree {t} layer {l}")
+
+
+@pytest.mark.parametrize("kind", ["dwn", "probabilistic", "hybrid"])
+def test_conv_layer_eval_and_state_dict_roundtrip(kind):
+    torch.manual_seed(5)
+    a = _build(kind, 2, 2, 5, 3, 1, 0, 2)
+    b = _build(kind, 2, 2, 5, 3, 1, 0, 2)
+    keys = set(a.state_dict().keys())
+    pname = _oracle_fns(kind)[0]
+    assert {f"first_layer_chunks.0.nodes.0.{pname}", f"first_layer_chunks.2.nodes.35.{pname}",
+            f"trees.4.1.nodes.0.{pname}", "trees.0.0._mapping_indices", "first_layer_chunks.1._mapping_indices"} <= keys
+    b.load_state_dict(a.state_dict())
+    a.eval(); b.eval()
+    x = torch.randint(0, 2, (3, 2, 6, 6), device=DEV).float()
+    with torch.no_grad():
+        ya, yb = a(x), b(x)
+    assert torch.equal(ya, yb) and set(ya.unique().tolist()) <= {0.0, 1.0}
+    # eval semantics level by level: every layer binarises its output
+    chunks, trees = _tables(a, pname)
+    if kind == "dwn":
+        ev = lambda m, i, t: np.stack([orc.dwn_eval_forward(m[:, i[n]], t[n])[:, 0] for n in range(len(t))], 1)
+    elif kind == "probabilistic":
+        ev = lambda m, i, t: np.stack([orc.prob_eval_forward(m[:, i[n]], t[n])[:, 0] for n in range(len(t))], 1)
+    else:
+        ev = lambda m, i, t: np.stack([orc.dwn_eval_forward(m[:, i[n]], orc.table_sigmoid(t[n]).astype(np.float32))[:, 0]
+                                       for n in range(len(t))], 1)
+    patches = orc.conv_unfold(x.cpu().numpy(), (3, 3), (1, 1), (0, 0))
+    out, _ = orc.conv_trees_forward(patches, chunks, trees, 36, ev)
+    assert np.array_equal(ya.cpu().numpy(), out.reshape(3, 16, 5).transpose(0, 2, 1).reshape(3, 5, 4, 4))
+
+
+@pytest.mark.parametrize("seed", [42, 43, 100])
+def test_grouped_connections_cover_every_channel(seed):
+    """tests/test_layers/test_grouped_convolutional_connections.py:25-94: with grouped connections and full
+    coverage the first inputs of the first-layer nodes touch all 64 channels; every node stays inside one channel."""
+    layer = _build("probabilistic", 1, 64, 16, 3, 1, 0, 128, grouped=True, seed=seed)
+    table = layer.first_layer_chunks[0]._mapping_indices.cpu().long()
+    assert (table[:, 0] // 9).unique().numel() == 64
+    assert torch.all((table // 9) == (table[:, :1] // 9))
+    x = torch.rand(2, 64, 8, 8, device=DEV)
+    layer.train()
+    y = layer(x)
+    assert y.shape == (2, 16, 6, 6) and torch.isfinite(y).all()
+
+
+def test_conv_bank_parameters_train_in_place():
+    """An optimizer over bank_parameters() (one tensor per depth level) updates the per-node parameters the
+    state dict shows."""
+    torch.manual_seed(9)
+    layer = _build("dwn", 2, 1, 6, 3, 1, 0, 4)
+    layer.train()
+    banks = layer.bank_parameters()
+    assert [tuple(t.shape) for t in banks] == [(216, 1, 64), (36, 1, 64), (6, 1, 64)]
+    opt = torch.optim.SGD(banks, lr=0.1)
+    before = layer.trees[5][1].nodes[0].luts.detach().clone()
+    x = torch.rand(4, 1, 8, 8, device=DEV)
+    layer(x).sum().backward()
+    assert all(t.grad is not None for t in banks)
+    opt.step()
+    after = layer.state_dict()["trees.5.1.nodes.0.luts"]
+    assert not torch.equal(before, after)
+    assert torch.equal(after, banks[2][5].detach())

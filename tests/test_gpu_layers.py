@@ -366,6 +366,60 @@ def test_dwn_stack_equals_layer_by_layer(shape, input_grad):
     assert torch.equal(stack(x), he)
 
 
+@pytest.mark.parametrize("case", [(130, 37, 4, [60, 20], 6), (64, 784, 4, [2000, 10], 6), (9, 5, 3, [7], 2),
+                                  (300, 70, 1, [33, 40], 5), (65, 17, 9, [50], 4)])
+def test_dwn_stack_with_thermometer_encoder(case):
+    """The stack fed raw features through a fitted thermometer encoder (code written directly as
+    bit-planes) against encode() followed by the layers one by one: outputs bit-exact, table
+    gradients to rtol 1e-5; the planes themselves against the oracle's bits."""
+    REGISTRY, NodeConfig, uniform_init, _ = _api()
+    from difflut_amd import _native as nat
+    from difflut_amd.layers import DWNStack
+    B, F, nbits, widths, k = case
+    torch.manual_seed(B + F)
+    x = torch.rand(B, F, device="cuda")
+    enc = REGISTRY.build_encoder("thermometer", num_bits=nbits).fit(x)
+    layers, width = [], F * nbits
+    for li, n in enumerate(widths):
+        layers.append(REGISTRY.get_layer("random")(width, n, REGISTRY.get_node("dwn"),
+                                                   NodeConfig(input_dim=k, output_dim=1, init_fn=uniform_init,
+                                                              init_kwargs={"a": -1.0, "b": 2.0}), seed=li + 9).cuda())
+        width = n
+    # the planes against the oracle: bit r of word (t, c) is bit c of row 64 t + r
+    lib = nat.lib()
+    planes = torch.zeros(lib.dl_dwn_planes_bytes(B, F * nbits) // 8, dtype=torch.int64, device="cuda")
+    nat.check(lib.dl_thermometer_planes(x.data_ptr(), enc.thresholds.contiguous().data_ptr(), planes.data_ptr(), B, F, nbits,
+                                        nat.stream()))
+    bits = orc.thermometer_encode(x.cpu().numpy(), enc.thresholds.cpu().numpy()).reshape(B, F * nbits)
+    BT = (B + 63) // 64
+    padded = np.zeros((BT * 64, F * nbits), dtype=np.uint64)
+    padded[:B] = bits.astype(np.uint64)
+    want = (padded.reshape(BT, 64, -1) << np.arange(64, dtype=np.uint64)[None, :, None]).sum(1, dtype=np.uint64)
+    got = planes.cpu().numpy().view(np.uint64)[:BT * F * nbits].reshape(BT, F * nbits)
+    assert np.array_equal(got, want)
+    gy = torch.randn(B, widths[-1], device="cuda")
+    h = enc.encode(x)
+    for layer in layers:
+        h = layer(h)
+    h.backward(gy)
+    want_y = h.detach().clone()
+    want_gl = [layer._banks["luts"].flat.grad.clone() for layer in layers]
+    for layer in layers:
+        layer._banks["luts"].flat.grad = None
+    stack = DWNStack(layers, encoder=enc).train()
+    y = stack(x)
+    assert torch.equal(y.detach(), want_y)
+    y.backward(gy)
+    for layer, want_g in zip(layers, want_gl):
+        torch.testing.assert_close(layer._banks["luts"].flat.grad, want_g, rtol=1e-5, atol=1e-6)
+    stack.eval()
+    he = enc.encode(x)
+    for layer in layers:
+        layer.eval()
+        he = layer(he)
+    assert torch.equal(stack(x), he)
+
+
 def test_dwn_layer_step_replays_from_a_hip_graph():
     """The library never allocates or synchronises, and clears buffers with kernels, so a forward +
     backward can be captured once and replayed; every replay is checked against an eager run on

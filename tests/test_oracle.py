@@ -398,3 +398,42 @@ def test_hybrid_backward_is_zero_at_binary_inputs():
     mixed[:, 1] = 0.3
     gm, _ = orc.hybrid_backward(mixed, luts, gy)
     assert np.all(gm[:, [0, 2, 3]] == 0.0) and np.all(gm[:, 1] != 0.0)
+
+
+# ------------------------------------------------------------------ convolutional layer
+def test_conv_unfold_ordering_and_fold_adjoint():
+    """Patch columns are (channel, dy, dx), rows are (image, output position) row-major; fold is the
+    adjoint (<unfold(x), g> = <x, fold(g)>)."""
+    rng = np.random.default_rng(10)
+    x = rng.random((2, 3, 5, 6)).astype(np.float32)
+    p = orc.conv_unfold(x, (3, 2), (1, 2), (1, 0))
+    out_h, out_w = (5 + 2 - 3) // 1 + 1, (6 - 2) // 2 + 1
+    assert p.shape == (2 * out_h * out_w, 3 * 3 * 2)
+    xp = np.pad(x, ((0, 0), (0, 0), (1, 1), (0, 0)))
+    for b, oy, ox, c, dy, dx in [(0, 0, 0, 0, 0, 0), (1, 4, 2, 2, 2, 1), (0, 2, 1, 1, 1, 0)]:
+        assert p[(b * out_h + oy) * out_w + ox, (c * 3 + dy) * 2 + dx] == xp[b, c, oy + dy, ox * 2 + dx]
+    g = rng.standard_normal(p.shape).astype(np.float32)
+    back = orc.conv_fold(g, x.shape, (3, 2), (1, 2), (1, 0))
+    assert np.isclose((p.astype(np.float64) * g).sum(), (x.astype(np.float64) * back).sum(), rtol=1e-6)
+
+
+def test_conv_tree_loops_on_a_hand_built_case():
+    """Two trees of depth 1 with n = 2 in one chunk: tree t reads first-layer columns 2t, 2t+1 only."""
+    rng = np.random.default_rng(11)
+    patches = rng.random((7, 4)).astype(np.float32)
+    idx0 = np.array([[0, 1], [2, 3], [1, 2], [3, 0]])
+    tab0 = rng.random((4, 1, 4)).astype(np.float32)
+    idx1 = np.array([[0, 1]])
+    t1a, t1b = rng.random((1, 1, 4)).astype(np.float32), rng.random((1, 1, 4)).astype(np.float32)
+    fwd = lambda x, idx, tab: orc.dwn_layer_forward(x, idx, tab)[:, :, 0]
+    out, acts = orc.conv_trees_forward(patches, [(idx0, tab0)], [[(idx1, t1a)], [(idx1, t1b)]], 2, fwd)
+    first = fwd(patches, idx0, tab0)
+    assert np.array_equal(out[:, 0], fwd(first[:, 0:2], idx1, t1a)[:, 0])
+    assert np.array_equal(out[:, 1], fwd(first[:, 2:4], idx1, t1b)[:, 0])
+    gout = rng.standard_normal((7, 2)).astype(np.float32)
+    bwd = lambda x, idx, tab, gy: orc.dwn_layer_backward(x, idx, tab, gy[:, :, None], 0.3, 0.4)
+    gp, gch, gtr = orc.conv_trees_backward(patches, [(idx0, tab0)], [[(idx1, t1a)], [(idx1, t1b)]], 2, acts, gout, bwd)
+    ga, gta = bwd(first[:, 0:2], idx1, t1a, gout[:, 0:1])
+    gb, gtb = bwd(first[:, 2:4], idx1, t1b, gout[:, 1:2])
+    wp, wt0 = bwd(patches, idx0, tab0, np.concatenate([ga, gb], 1))
+    assert np.allclose(gp, wp) and np.allclose(gch[0], wt0) and np.allclose(gtr[0][0], gta) and np.allclose(gtr[1][0], gtb)
