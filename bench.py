@@ -44,6 +44,9 @@ WORKLOADS = {
     # the headline layer shape with the two other table-lookup node types
     "stable_k6_b4096_i16384_n8192": (4096, 16384, 8192, 6, 1),
     "hybrid_k6_b4096_i16384_n8192": (4096, 16384, 8192, 6, 1),
+    # convolutional LUT layer through the layer API: (images, in_channels, out_channels, k, O); 28x28 images,
+    # receptive field 5, trees of depth 2
+    "conv_b256_c4_28x28_o32_rf5_d2": (256, 4, 32, 6, 1),
     # whole training step of the deep stack through the layer API: (B, features, first layer width, k, O)
     "dwn_stack_b8192_train_step": (8192, 784, 16000, 6, 1),
 }
@@ -146,6 +149,51 @@ def run_stack(args):
                              "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes_per_step": nbytes},
            "kernel_ms": kernel_times(step, min(args.steps, 5))}
     print(json.dumps(out))
+
+
+def run_conv(args):
+    """ConvolutionalLayer (DWN nodes, trees of depth 2 over 5x5x4 patches of 28x28 images): forward and backward
+    including the input gradient, through the module API."""
+    from difflut_amd import REGISTRY
+    from difflut_amd.layers import ConvolutionConfig
+    from difflut_amd.nodes.node_config import NodeConfig
+
+    dev = torch.device("cuda:0")
+    B, C, T, k, O = WORKLOADS[args.workload]
+    H = W = 28
+    rf, depth = 5, 2
+    torch.manual_seed(0)
+    cfg = ConvolutionConfig(tree_depth=depth, in_channels=C, out_channels=T, receptive_field=rf, stride=1, padding=0,
+                            chunk_size=32, seed=42)
+    layer = REGISTRY.get_convolutional_layer("convolutional")(
+        convolution_config=cfg, node_type=REGISTRY.get_node("dwn"), node_kwargs=NodeConfig(input_dim=k, output_dim=O),
+        layer_type=REGISTRY.get_layer("random"), n_inputs_per_node=k).to(dev).train()
+    x = torch.bernoulli(torch.full((B, C, H, W), 0.5, device=dev)).requires_grad_()
+    out = H - rf + 1
+    gy = torch.randn(B, T, out, out, device=dev)
+    banks = layer.bank_parameters()
+
+    def step():
+        x.grad = None
+        for t in banks:
+            t.grad = None
+        layer(x).backward(gy)
+
+    ms = time_steps(step, args.steps, args.warmup)
+    rows = B * out * out
+    nodes = sum(layer.hidden_layers) * T
+    # compulsory traffic of the convolution as a whole: the image in, its gradient out, the output and its gradient
+    nbytes = 2 * x.numel() * 4 + 2 * gy.numel() * 4 + 4 * nodes * (1 << k) * 4
+    out_d = {"metric": "LUT-node evals/sec fwd+bwd (ConvolutionalLayer, DWN k=6 trees of depth 2, 32 channels, 5x5x4 patches)",
+             "value": rows * nodes / (ms * 1e-3), "unit": "node-evals/s", "ms_per_step": ms, "dtype": "f32",
+             "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+             "vs_baseline": None, "data": "synthetic",
+             "config": {"workload": args.workload, "images": B, "in_channels": C, "out_channels": T, "image": [H, W],
+                        "receptive_field": rf, "tree_depth": depth, "patch_rows": rows, "nodes": nodes},
+             "roofline_step": {"bound": "hbm", "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                               "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes_per_step": nbytes},
+             "kernel_ms": kernel_times(step, min(args.steps, 5))}
+    print(json.dumps(out_d))
 
 
 def run_secondary(args):
@@ -281,6 +329,8 @@ def main():
         raise SystemExit("bench.py needs a ROCm device")
     if args.workload.startswith("dwn_stack"):
         return run_stack(args)
+    if args.workload.startswith("conv"):
+        return run_conv(args)
     if not args.workload.startswith("dwn"):
         return run_secondary(args)
     dev = torch.device("cuda:0")

@@ -52,6 +52,9 @@ SIGNATURES = {
     "dl_hard_select_bwd": (_I, [_P, _P, _P, _P, _I, _I, _I, _P]),
     "dl_thermometer_encode": (_I, [_P, _P, _P, _I, _I, _I, _P]),
     "dl_thermometer_planes": (_I, [_P, _P, _P, _I, _I, _I, _P]),
+    "dl_unfold_rows": (ctypes.c_longlong, [_I] * 9),
+    "dl_unfold": (_I, [_P, _P, _P] + [_I] * 10 + [_P]),
+    "dl_fold": (_I, [_P, _I, _P] + [_I] * 10 + [_P]),
     "dl_group_sum_fwd": (_I, [_P, _P, _I, _I, _I, _F, _P]),
     "dl_group_sum_bwd": (_I, [_P, _P, _I, _I, _I, _F, _P]),
     "dl_profile_enable": (_I, [_I]),

@@ -7,7 +7,8 @@ every tree layer, out_channels * tree_depth tiny layer calls per forward.  Here 
 one depth level run as ONE block-diagonal layer call: level l has out_channels * n^(depth-l) nodes,
 tree t's nodes read the columns of tree t only (its index table shifted by t times the level's
 width), and for DWN nodes the levels are chained (bit-planes between levels, tile-major gradients
-back).  The node parameters of a level live in one [nodes, ...] tensor; the per-node Parameters of
+back) and the patch matrix is only ever written as bit-planes.  Patch extraction and its adjoint are
+the library's own kernels instead of `nn.Unfold` (kept as the `unfold` attribute for inspection).  The node parameters of a level live in one [nodes, ...] tensor; the per-node Parameters of
 the sub-layers are views of it.
 """
 import torch
@@ -151,12 +152,24 @@ class ConvolutionalLayer(LUTLayerMixin, nn.Module):
             self._plans, self._plan_key = plans, key
         return self._plans
 
-    def _run_levels(self, patches):
-        """patches [rows, input_size] -> [rows, out_channels] through the depth levels."""
-        plans = self._level_plans(patches.device)
+    def _geometry(self):
+        return (*self.receptive_field, *self.stride, *self.padding)
+
+    def _chained(self):
+        """DWN trees in training mode run as one chained call that reads the image itself."""
+        return (self._kind == "dwn" and self.training and self.n_inputs_per_node <= ops.FAST_K
+                and self.flip_probability <= 0.0)
+
+    def _run_levels(self, patches, image=None):
+        """patches [rows, input_size] (or, chained, the image batch) -> [rows, out_channels] through the depth levels."""
+        device = patches.device if patches is not None else image.device
+        plans = self._level_plans(device)
         banks = [{name: bank.tensor() for name, bank in level.items()} for level in self._level_banks]
         firsts = [self._level_layers(level)[0].nodes[0] for level in range(self.tree_depth + 1)]
         kind, h = self._kind, patches
+        if image is not None:
+            scalars = [node.efd_scalars() for node in firsts]
+            return ops.DWNStackFunction.apply(image, self._geometry(), plans, scalars, *[b["luts"] for b in banks])
         if kind == "dwn" and self.training and self.n_inputs_per_node <= ops.FAST_K:
             scalars = [node.efd_scalars() for node in firsts]
             return ops.DWNStackFunction.apply(h, None, plans, scalars, *[b["luts"] for b in banks])
@@ -200,16 +213,20 @@ class ConvolutionalLayer(LUTLayerMixin, nn.Module):
     # ------------------------------------------------------------------ interface
     def forward(self, x):
         _native.require_device(x)
+        if x.dim() != 4 or x.shape[1] != self.in_channels:
+            raise ValueError(f"ConvolutionalLayer expects (batch, {self.in_channels}, height, width), got {tuple(x.shape)}")
         batch = x.shape[0]
-        patches = self.unfold(x)  # (batch, channels * kh * kw, positions)
-        positions = patches.shape[2]
-        patches = patches.transpose(1, 2).contiguous().view(-1, self.input_size)
-        if self.training and self.flip_probability > 0.0:
-            patches = self._apply_bit_flip(patches)
-        out = self._run_levels(patches) if self._kind is not None else self._loop_trees(patches)
-        out = out.view(batch, positions, self.out_channels).transpose(1, 2)
         out_h = (x.shape[2] + 2 * self.padding[0] - self.receptive_field[0]) // self.stride[0] + 1
         out_w = (x.shape[3] + 2 * self.padding[1] - self.receptive_field[1]) // self.stride[1] + 1
+        positions = out_h * out_w
+        if self._kind is not None and self._chained():
+            out = self._run_levels(None, image=x)  # patches only ever exist as bit-planes
+        else:
+            patches = ops.UnfoldFunction.apply(x, self._geometry())  # (batch * positions, channels * kh * kw)
+            if self.training and self.flip_probability > 0.0:
+                patches = self._apply_bit_flip(patches)
+            out = self._run_levels(patches) if self._kind is not None else self._loop_trees(patches)
+        out = out.view(batch, positions, self.out_channels).transpose(1, 2)
         out = out.reshape(batch, self.out_channels, out_h, out_w)
         if self.grad_stabilization != "none" and self.training and out.requires_grad:
             def hook(grad):

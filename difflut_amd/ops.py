@@ -91,6 +91,35 @@ class GatherFunction(torch.autograd.Function):
         return gx, None, None
 
 
+# ----------------------------------------------------------------------------- patches of the convolutional layer
+class UnfoldFunction(torch.autograd.Function):
+    """x [B,C,H,W] -> patches [B*OH*OW, C*KH*KW] (nn.Unfold, transposed and flattened as
+    difflut/layers/convolutional.py:199-205 does); backward folds the patch gradients back.
+    `geom` = (KH, KW, SH, SW, PH, PW)."""
+
+    @staticmethod
+    def forward(ctx, x, geom):
+        nat.require_device(x)
+        x = _f32(x)
+        B, C, H, W = x.shape
+        lib = nat.lib()
+        rows = lib.dl_unfold_rows(B, H, W, *geom)
+        if rows <= 0:
+            raise RuntimeError(f"receptive field {geom[:2]} with stride {geom[2:4]}, padding {geom[4:]} does not fit a "
+                               f"{H}x{W} image")
+        patches = torch.empty((rows, C * geom[0] * geom[1]), dtype=torch.float32, device=x.device)
+        nat.check(lib.dl_unfold(nat.ptr(x), nat.ptr(patches), None, B, C, H, W, *geom, nat.stream()))
+        ctx.shape, ctx.geom = (B, C, H, W), geom
+        return patches
+
+    @staticmethod
+    def backward(ctx, gp):
+        gp = _f32(gp)
+        gx = torch.empty(ctx.shape, dtype=torch.float32, device=gp.device)
+        nat.check(nat.lib().dl_fold(nat.ptr(gp), 0, nat.ptr(gx), *ctx.shape, *ctx.geom, nat.stream()))
+        return gx, None
+
+
 # ----------------------------------------------------------------------------- DWN
 class DWNLayerFunction(torch.autograd.Function):
     """y[b, n*O+d] = luts[n,d,addr(b,n)] with the extended-finite-difference backward."""
@@ -139,19 +168,37 @@ class DWNStackFunction(torch.autograd.Function):
     first layer's input gradient, if asked for).  Same arithmetic as calling the layers one by one."""
 
     @staticmethod
-    def forward(ctx, x, thresholds, plans, scalars, *luts):
-        """`thresholds` [F, nbits] (or None): x is raw data [B, F] and the first layer reads its
-        thermometer code, produced directly as bit-planes; x then gets no gradient (the code is a
-        step function of it)."""
+    def forward(ctx, x, source, plans, scalars, *luts):
+        """`source` says what the first layer reads:
+        None                  x [B, I] itself;
+        a tensor [F, nbits]   thermometer thresholds: x is raw data [B, F], its code is produced directly
+                              as bit-planes and x gets no gradient (the code is a step function of it);
+        a tuple (KH, KW, SH, SW, PH, PW)   x is an image batch [B, C, H, W]: the first layer reads its patch
+                              matrix (rows = output positions), again produced directly as bit-planes; the
+                              input gradient is folded back from the tile-major patch gradient."""
+        thresholds = source if torch.is_tensor(source) else None
+        geom = source if isinstance(source, tuple) else None
         nat.require_device(x, thresholds, *luts)
         x = _f32(x)
         luts = tuple(_f32(t) for t in luts)
-        B, width = x.shape
         lib = nat.lib()
-        if thresholds is None:
+        ctx.image = None
+        if geom is not None:
+            Bi, C, H, W = x.shape
+            B = int(lib.dl_unfold_rows(Bi, H, W, *geom))
+            if B <= 0:
+                raise RuntimeError(f"receptive field {geom[:2]} with stride {geom[2:4]}, padding {geom[4:]} does not fit "
+                                   f"a {H}x{W} image")
+            width = C * geom[0] * geom[1]
+            planes = _bytes(lib.dl_dwn_planes_bytes(B, width), x.device)
+            nat.check(lib.dl_unfold(nat.ptr(x), None, nat.ptr(planes), Bi, C, H, W, *geom, nat.stream()))
+            ctx.image = ((Bi, C, H, W), geom)
+        elif thresholds is None:
+            B, width = x.shape
             planes = _bytes(lib.dl_dwn_planes_bytes(B, width), x.device)
             nat.check(lib.dl_dwn_pack_planes(nat.ptr(x), nat.ptr(planes), B, width, nat.stream()))
         else:
+            B, width = x.shape
             thr = _f32(thresholds)
             if thr.dim() != 2 or thr.shape[0] != width:
                 raise RuntimeError(f"thresholds {tuple(thr.shape)} do not match {width} features")
@@ -197,8 +244,13 @@ class DWNStackFunction(torch.autograd.Function):
                 gx_tiled = 1
             else:
                 want = ctx.needs_input_grad[0] and not ctx.encoded
-                gx = torch.empty((B, I), dtype=torch.float32, device=g.device) if want else None
-                gx_tiled = 0
+                gx_tiled = 1 if ctx.image is not None else 0
+                if not want:
+                    gx = None
+                elif gx_tiled:
+                    gx = torch.empty(lib.dl_dwn_tiled_bytes(B, I) // 4, dtype=torch.float32, device=g.device)
+                else:
+                    gx = torch.empty((B, I), dtype=torch.float32, device=g.device)
             grads[l] = torch.empty_like(luts[l])
             ws = _bytes(lib.dl_dwn_bwd_workspace_bytes(*dims), g.device)
             nat.check(lib.dl_dwn_layer_bwd_tiled(nat.ptr(saved[l]), nat.ptr(plan.inv_ptr), nat.ptr(plan.inv_pos),
@@ -206,6 +258,11 @@ class DWNStackFunction(torch.autograd.Function):
                                                  nat.ptr(gx), gx_tiled, nat.ptr(grads[l]), nat.ptr(ws), ws.numel(), *dims,
                                                  nat.stream()))
             g, tiled = gx, gx_tiled
+        if ctx.image is not None and g is not None:
+            shape, geom = ctx.image
+            gimg = torch.empty(shape, dtype=torch.float32, device=g.device)
+            nat.check(lib.dl_fold(nat.ptr(g), 1, nat.ptr(gimg), *shape, *geom, nat.stream()))
+            g = gimg
         return (g, None, None, None, *grads)
 
 

@@ -234,6 +234,25 @@ int dl_group_sum_fwd(const float *x, float *y, int B, int F, int groups, float t
 int dl_group_sum_bwd(const float *gy, float *gx, int B, int F, int groups, float tau, void *stream);
 
 /* ------------------------------------------------------------------------
+ * Convolutional LUT layer: patch extraction and its adjoint.
+ * Replaces nn.Unfold + transpose + contiguous + view in ConvolutionalLayer.forward
+ * (difflut/layers/convolutional.py:199-205) and what autograd does for them in the backward.
+ *   x [B,C,H,W];  rows r = (b, oy, ox) row-major, OH = (H + 2 PH - KH) / SH + 1 (OW alike);
+ *   columns c = (ch, dy, dx) row-major;  patches[r][c] = x[b, ch, oy SH + dy - PH, ox SW + dx - PW], 0 outside.
+ * dl_unfold writes `patches` [rows, C KH KW] fp32 (nullable) and/or `planes` (nullable): the same matrix
+ * as the bit-planes of (value >= 0.5) that dl_dwn_layer_fwd_planes reads (dl_dwn_planes_bytes(rows, C KH KW));
+ * the bit-plane form has no counterpart in the reference.  dl_fold sums a gradient of the patch matrix,
+ * row-major or (tiled) tile-major [rows/64][C KH KW][64] as dl_dwn_layer_bwd_tiled writes it, back into
+ * gx [B,C,H,W] (overwritten; fixed summation order).  C KH KW <= 4096.  dl_unfold_rows returns B OH OW (0 if
+ * the geometry is invalid).
+ * ------------------------------------------------------------------------ */
+long long dl_unfold_rows(int B, int H, int W, int KH, int KW, int SH, int SW, int PH, int PW);
+int dl_unfold(const float *x, float *patches, void *planes, int B, int C, int H, int W,
+              int KH, int KW, int SH, int SW, int PH, int PW, void *stream);
+int dl_fold(const float *gpatches, int tiled, float *gx, int B, int C, int H, int W,
+            int KH, int KW, int SH, int SW, int PH, int PW, void *stream);
+
+/* ------------------------------------------------------------------------
  * Per-kernel timing.  No counterpart in the reference (it has no tracing at all).
  * After dl_profile_enable(1) every kernel launched by the entry points above is
  * bracketed by HIP events on its stream (at most 64 kernels between two reads).

@@ -54,6 +54,59 @@ def _oracle_fns(kind, scale=1.25):
     return "raw_luts", fwd, lambda x, i, t, g: orc.hybrid_layer_backward(x, i, t, g[:, :, None])
 
 
+GEOMS = [  # (B, C, H, W), (KH, KW, SH, SW, PH, PW)
+    ((2, 3, 5, 6), (3, 2, 1, 2, 1, 0)),
+    ((3, 1, 10, 10), (3, 3, 1, 1, 0, 0)),
+    ((1, 4, 28, 28), (5, 5, 1, 1, 0, 0)),
+    ((5, 2, 9, 7), (2, 3, 2, 3, 1, 2)),
+    ((70, 1, 4, 4), (4, 4, 1, 1, 0, 0)),   # one row per image
+    ((2, 2, 6, 6), (1, 1, 1, 1, 0, 0)),
+]
+
+
+@pytest.mark.parametrize("case", GEOMS)
+def test_unfold_rows_planes_and_fold(case):
+    """Patch matrix bit-exact against torch's unfold (CPU), its bit-planes against the packed oracle bits,
+    and the fold of row-major and tile-major gradients against torch's fold."""
+    from difflut_amd import _native as nat
+    from difflut_amd import ops
+    shape, geom = case
+    rng = np.random.default_rng(sum(shape) + sum(geom))
+    x = rng.random(shape).astype(np.float32)
+    want = orc.conv_unfold(x, geom[0:2], geom[2:4], geom[4:6])
+    xt = torch.tensor(x, device=DEV, requires_grad=True)
+    patches = ops.UnfoldFunction.apply(xt, geom)
+    assert np.array_equal(patches.detach().cpu().numpy(), want)
+    rows, cols = want.shape
+    lib = nat.lib()
+    assert lib.dl_unfold_rows(shape[0], shape[2], shape[3], *geom) == rows
+    planes = torch.zeros(lib.dl_dwn_planes_bytes(rows, cols) // 8, dtype=torch.int64, device=DEV)
+    nat.check(lib.dl_unfold(xt.data_ptr(), None, planes.data_ptr(), *shape, *geom, nat.stream()))
+    BT = (rows + 63) // 64
+    bits = np.zeros((BT * 64, cols), dtype=np.uint64)
+    bits[:rows] = (want >= 0.5).astype(np.uint64)
+    packed = (bits.reshape(BT, 64, cols) << np.arange(64, dtype=np.uint64)[None, :, None]).sum(1, dtype=np.uint64)
+    assert np.array_equal(planes.cpu().numpy().view(np.uint64)[:BT * cols].reshape(BT, cols), packed)
+    g = rng.standard_normal(want.shape).astype(np.float32)
+    patches.backward(torch.tensor(g, device=DEV))
+    folded = orc.conv_fold(g, shape, geom[0:2], geom[2:4], geom[4:6])
+    np.testing.assert_allclose(xt.grad.cpu().numpy(), folded, rtol=1e-6, atol=1e-6)  # <= KH*KW terms per pixel
+    tiled = np.zeros((BT * 64, cols), dtype=np.float32)
+    tiled[:rows] = g
+    tiled = np.ascontiguousarray(tiled.reshape(BT, 64, cols).transpose(0, 2, 1))
+    gx = torch.empty(shape, device=DEV)
+    nat.check(lib.dl_fold(torch.tensor(tiled, device=DEV).data_ptr(), 1, gx.data_ptr(), *shape, *geom, nat.stream()))
+    assert torch.equal(gx, xt.grad)  # same terms in the same order
+
+
+def test_unfold_rejects_bad_geometry():
+    from difflut_amd import ops
+    with pytest.raises(RuntimeError):
+        ops.UnfoldFunction.apply(torch.rand(1, 1, 3, 3, device=DEV), (5, 5, 1, 1, 0, 0))
+    with pytest.raises(RuntimeError):
+        ops.UnfoldFunction.apply(torch.rand(1, 1, 3, 3), (3, 3, 1, 1, 0, 0))  # CPU tensor
+
+
 CASES = [  # (kind, depth, in_ch, out_ch, rf, stride, padding, chunk, image)
     ("dwn", 1, 1, 16, 3, 1, 0, 8, (4, 10, 10)),          # tests/test_layers/test_convolutional_learning.py:186-195
     ("dwn", 2, 2, 5, 3, 1, 1, 2, (3, 7, 6)),             # ragged last chunk, padding

@@ -67,6 +67,26 @@ def test_dwn_layer_forward_backward(shape):
     np.testing.assert_allclose(lt.grad.cpu().numpy(), gl, rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("shape", [(33000, 50, 300, 6, 1), (40000, 7, 40, 2, 1)])
+def test_dwn_backward_few_inputs_many_rows(shape):
+    """Few inputs read by many nodes over many rows (the shape of the first level of a convolutional layer:
+    CSR lists of ~36 entries per input, hundreds of batch tiles) against the C restatement on all rows."""
+    B, I, N, k, O = shape
+    ops = _ops()
+    x, idx, luts, gy = make_case(sum(shape) % 1000, *shape)
+    plan = ops.MappingPlan(dev(idx, torch.int32), I)
+    alpha, beta = 0.5 * 0.75 ** (k - 1), 1.0 / 3.0
+    xt = dev(x).requires_grad_()
+    lt = dev(luts).requires_grad_()
+    y = ops.DWNLayerFunction.apply(xt, lt, plan, alpha, beta)
+    y.backward(dev(gy.reshape(B, N * O)))
+    assert np.array_equal(y.detach().cpu().numpy(), c_oracle.dwn_layer_forward(x, idx, luts).reshape(B, N * O))
+    wx, wl = c_oracle.dwn_layer_backward(x, idx, luts, gy, alpha, beta)
+    # up to N*k/I (~36) terms of size alpha*|gy|*|D| per input: rtol 1e-5, floor 5e-6
+    np.testing.assert_allclose(xt.grad.cpu().numpy(), wx, rtol=1e-5, atol=5e-6)
+    np.testing.assert_allclose(lt.grad.cpu().numpy(), wl, rtol=1e-5, atol=2e-4)  # ~B/2^k terms per bin
+
+
 def test_dwn_threshold_is_inclusive_and_exact_at_half():
     ops = _ops()
     x = np.array([[0.5, 0.49999997, 0.50000006, 0.0, 1.0, -3.0]], dtype=np.float32)
