@@ -29,3 +29,12 @@ def golden():
 
     path = os.path.join(ROOT, "tests", "golden", "reference_vectors.npz")
     return dict(np.load(path, allow_pickle=False))
+
+
+@pytest.fixture(scope="session")
+def golden_next():
+    """Vectors of the node types and layers added later (tests/golden/make_golden_next.py)."""
+    import numpy as np
+
+    path = os.path.join(ROOT, "tests", "golden", "reference_vectors_next.npz")
+    return dict(np.load(path, allow_pickle=False))

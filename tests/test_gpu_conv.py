@@ -218,3 +218,35 @@ def test_conv_bank_parameters_train_in_place():
     after = layer.state_dict()["trees.5.1.nodes.0.luts"]
     assert not torch.equal(before, after)
     assert torch.equal(after, banks[2][5].detach())
+
+
+def test_conv_layer_against_reference_vectors(golden_next):
+    """The reference layer's own state dict loaded into this layer; outputs, input gradient, every table
+    gradient and the eval outputs against what the reference's CPU path produced (tests/golden)."""
+    from difflut_amd.layers import ConvolutionalLayer, ConvolutionConfig, RandomLayer
+    from difflut_amd.nodes import DWNNode, NodeConfig
+
+    g = golden_next
+    cfg = ConvolutionConfig(tree_depth=2, in_channels=2, out_channels=3, receptive_field=2, stride=1, padding=0,
+                            chunk_size=2, seed=42)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        layer = ConvolutionalLayer(cfg, DWNNode, NodeConfig(input_dim=2, output_dim=1), RandomLayer, n_inputs_per_node=2)
+    state = {k[len("conv_state."):]: torch.tensor(v) for k, v in g.items() if k.startswith("conv_state.")}
+    layer.load_state_dict(state)
+    layer = layer.to(DEV).train()
+    x = torch.tensor(g["conv_x"], device=DEV, requires_grad=True)
+    y = layer(x)
+    assert np.array_equal(y.detach().cpu().numpy(), g["conv_y"])
+    y.backward(torch.tensor(g["conv_gy"], device=DEV))
+    np.testing.assert_allclose(x.grad.cpu().numpy(), g["conv_gx"], rtol=1e-5, atol=2e-6)
+    checked = 0
+    for name, param in layer.named_parameters():
+        want = g.get(f"conv_grad.{name}")
+        if want is not None and want.shape != ():
+            np.testing.assert_allclose(param.grad.cpu().numpy(), want, rtol=1e-5, atol=2e-6, err_msg=name)
+            checked += 1
+    assert checked == 12 + 6 + 3
+    layer.eval()
+    with torch.no_grad():
+        assert np.array_equal(layer(torch.tensor(g["conv_eval_x"], device=DEV)).cpu().numpy(), g["conv_eval_y"])

@@ -312,3 +312,30 @@ def test_full_size_properties_stable_and_hybrid_k6_b4096_n8192():
         _, gx0, _ = run(torch.full_like(luts, 0.3), gy)
         assert gx0.abs().max().item() <= 2e-5  # constant table: every difference vanishes
         assert torch.isfinite(gx).all() and gx.abs().max().item() > 0
+
+
+@pytest.mark.parametrize("name,kind", [("dwn_stable", "stable"), ("hybrid", "hybrid")])
+@pytest.mark.parametrize("tag", ["k6o1", "k3o2"])
+def test_nodes_against_reference_vectors(golden_next, name, kind, tag):
+    """Same inputs the reference's own CPU path was run on (tests/golden): training output, gradients down to
+    the raw tables, eval output."""
+    REGISTRY, _, _, _ = _api()
+    g = golden_next
+    raw = g[f"{kind}_{tag}_raw"]
+    O, L = raw.shape
+    kw = {"gradient_scale": 1.6} if kind == "stable" else {}
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        node = REGISTRY.get_node(name)(input_dim=L.bit_length() - 1, output_dim=O, **kw)
+    with torch.no_grad():
+        node.raw_luts.copy_(torch.tensor(raw))
+    node = node.to(DEV).train()
+    xt = dev(g[f"{kind}_{tag}_x"]).requires_grad_()
+    y = node(xt)
+    np.testing.assert_allclose(y.detach().cpu().numpy(), g[f"{kind}_{tag}_y"], rtol=3e-7, atol=1e-8)  # sigmoid: 2 ulp
+    y.backward(dev(g[f"{kind}_{tag}_gy"]))
+    np.testing.assert_allclose(xt.grad.cpu().numpy(), g[f"{kind}_{tag}_gx"], rtol=2e-5, atol=2e-6)
+    np.testing.assert_allclose(node.raw_luts.grad.cpu().numpy(), g[f"{kind}_{tag}_graw"], rtol=2e-5, atol=2e-6)
+    node.eval()
+    with torch.no_grad():
+        assert np.array_equal(node(dev(g[f"{kind}_{tag}_eval_x"])).cpu().numpy(), g[f"{kind}_{tag}_eval_y"])

@@ -157,3 +157,83 @@ def test_residual_initialiser_known_answer(golden):
                           init_kwargs={"node_type": "probabilistic", "noise_factor": 0.0, "logit_clarity": 5.0,
                                        "input_dim": 3})
     assert p.raw_weights[:, 0].tolist() == [-5, 5, -5, 5, -5, 5, -5, 5]
+
+
+def test_stable_and_hybrid_nodes_consume_the_generator_like_the_reference(golden_next):
+    """Same constructor calls in the same order as the script that wrote the vectors: default `raw_luts`
+    (randn * 0.1), initialised tables, inputs and the generator position afterwards all agree."""
+    from difflut_amd.nodes import DWNStableNode, HybridNode
+    from difflut_amd.nodes.utils import uniform_init
+
+    g = golden_next
+    torch.manual_seed(21)
+    for cls, kind in ((DWNStableNode, "stable"), (HybridNode, "hybrid")):
+        for tag, B, k, O in (("k6o1", 12, 6, 1), ("k3o2", 9, 3, 2)):
+            kw = {"gradient_scale": 1.6} if kind == "stable" else {}
+            node = cls(input_dim=k, output_dim=O, use_cuda=False, **kw)
+            assert np.array_equal(node.raw_luts.detach().numpy(), g[f"{kind}_{tag}_default_raw"])
+            node = cls(input_dim=k, output_dim=O, use_cuda=False, init_fn=uniform_init, init_kwargs={"a": -2.0, "b": 2.0}, **kw)
+            assert np.array_equal(node.raw_luts.detach().numpy(), g[f"{kind}_{tag}_raw"])
+            assert tuple(node.raw_luts.shape) == (O, 2 ** k)
+            if kind == "stable":
+                assert abs(float(node.gradient_scale) - 1.6) < 1e-7 and isinstance(node.gradient_scale, torch.nn.Parameter)
+            else:
+                assert np.array_equal(node.binary_combinations.numpy()[5][:3], [1.0, 0.0, 1.0])  # input 0 = LSB
+            x = 0.02 + 0.96 * torch.rand(B, k)
+            assert np.array_equal(x.numpy(), g[f"{kind}_{tag}_x"])
+            torch.randn(B, O); torch.randint(0, 2, (B, k))
+    assert np.array_equal(torch.rand(3).numpy(), g["next_rand_after_nodes"])
+
+
+@pytest.mark.parametrize("tag,cover", [("cover", True), ("nocover", False)])
+def test_grouped_input_mapping_matches_reference(golden_next, tag, cover):
+    from difflut_amd.layers import GroupedInputConfig
+
+    g = golden_next
+    torch.manual_seed(77)
+    cfg = GroupedInputConfig(n_groups=4, input_size=36, output_trees=5, luts_per_tree=6, bits_per_node=6, seed=42,
+                             ensure_full_coverage=cover)
+    assert np.array_equal(cfg.mapping_indices.numpy(), g[f"grouped_{tag}_table"])
+    assert np.array_equal(cfg.get_mapping_indices(1, 3).numpy(), g[f"grouped_{tag}_chunk_1_3"])
+    assert np.array_equal(torch.rand(2).numpy(), g[f"grouped_{tag}_next_rand"])
+    groups = cfg.mapping_indices // 9
+    assert torch.all(groups == groups[:, :1])  # a node stays inside one group
+    if cover:
+        assert sorted(groups[:28, 0].tolist()) == sorted(list(range(4)) * 7)  # dealt out as permutations
+
+
+def test_convolutional_layer_construction_matches_reference(golden_next):
+    """Sub-module layout, state-dict keys, index tables and per-node tables of a seeded layer."""
+    from difflut_amd import REGISTRY
+    from difflut_amd.layers import ConvolutionalLayer, ConvolutionConfig, RandomLayer
+    from difflut_amd.nodes import DWNNode, NodeConfig, ProbabilisticNode
+    from difflut_amd.nodes.utils import uniform_init
+
+    g = golden_next
+    assert REGISTRY.get_convolutional_layer("convolutional") is ConvolutionalLayer
+    torch.manual_seed(31)
+    cfg = ConvolutionConfig(tree_depth=2, in_channels=2, out_channels=3, receptive_field=2, stride=1, padding=0,
+                            chunk_size=2, seed=42)
+    layer = ConvolutionalLayer(cfg, DWNNode, NodeConfig(input_dim=2, output_dim=1, init_fn=uniform_init,
+                                                        init_kwargs={"a": -1.0, "b": 2.0}), RandomLayer, n_inputs_per_node=2)
+    want = {k[len("conv_state."):]: v for k, v in g.items() if k.startswith("conv_state.")}
+    state = layer.state_dict()
+    assert set(state) == set(want)
+    for name, value in want.items():
+        assert np.array_equal(state[name].numpy(), value), name
+    assert layer.hidden_layers == [4, 2, 1] and len(layer.first_layer_chunks) == 2 and len(layer.trees) == 3
+    assert [tuple(t.shape) for t in layer.bank_parameters()] == [(12, 1, 4), (6, 1, 4), (3, 1, 4)]
+    assert np.array_equal(torch.rand(4, 2, 4, 4)[:2].numpy(), g["conv_x"])  # generator position after construction
+    with pytest.raises(RuntimeError):
+        layer(torch.rand(2, 2, 4, 4))  # CPU tensors are refused
+    torch.manual_seed(32)
+    gcfg = ConvolutionConfig(tree_depth=1, in_channels=4, out_channels=5, receptive_field=3, stride=1, padding=0,
+                             chunk_size=2, seed=43)
+    glayer = ConvolutionalLayer(gcfg, ProbabilisticNode, NodeConfig(input_dim=6, output_dim=1), RandomLayer,
+                                n_inputs_per_node=6, grouped_connections=True, ensure_full_coverage=True)
+    for c, chunk in enumerate(glayer.first_layer_chunks):
+        assert np.array_equal(chunk._mapping_indices.numpy(), g[f"gconv_chunk{c}_idx"])
+    assert np.array_equal(glayer.trees[0][0]._mapping_indices.numpy(), g["gconv_tree0_idx"])
+    assert np.array_equal(glayer.trees[4][0]._mapping_indices.numpy(), g["gconv_tree4_idx"])
+    assert np.array_equal(glayer.first_layer_chunks[0].nodes[0].raw_weights.detach().numpy(), g["gconv_first_raw"])
+    assert np.array_equal(glayer.trees[4][0].nodes[0].raw_weights.detach().numpy(), g["gconv_last_raw"])

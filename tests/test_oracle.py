@@ -437,3 +437,47 @@ def test_conv_tree_loops_on_a_hand_built_case():
     gb, gtb = bwd(first[:, 2:4], idx1, t1b, gout[:, 1:2])
     wp, wt0 = bwd(patches, idx0, tab0, np.concatenate([ga, gb], 1))
     assert np.allclose(gp, wp) and np.allclose(gch[0], wt0) and np.allclose(gtr[0][0], gta) and np.allclose(gtr[1][0], gtb)
+
+
+# ------------------------------------------------------------------ reference numbers for the later node types
+@pytest.mark.parametrize("kind", ["stable", "hybrid"])
+@pytest.mark.parametrize("tag", ["k6o1", "k3o2"])
+def test_stable_and_hybrid_match_reference(golden_next, kind, tag):
+    g = golden_next
+    x, raw, gy = g[f"{kind}_{tag}_x"], g[f"{kind}_{tag}_raw"], g[f"{kind}_{tag}_gy"]
+    luts = orc.table_sigmoid(raw)
+    assert np.allclose(orc.dwn_forward(x, luts.astype(np.float32)), g[f"{kind}_{tag}_y"], rtol=1e-6, atol=1e-7)
+    idx = np.arange(x.shape[1])[None]
+    if kind == "stable":
+        gx, graw = orc.stable_layer_backward(x, idx, raw[None], gy[:, None, :], 1.6)
+    else:
+        gx, graw = orc.hybrid_layer_backward(x, idx, raw[None], gy[:, None, :])
+    assert np.allclose(gx, g[f"{kind}_{tag}_gx"], rtol=2e-5, atol=2e-6)      # the reference accumulates in fp32
+    assert np.allclose(graw[0], g[f"{kind}_{tag}_graw"], rtol=2e-5, atol=2e-6)
+    ev = orc.dwn_eval_forward(g[f"{kind}_{tag}_eval_x"], luts.astype(np.float32))
+    assert np.array_equal(ev, g[f"{kind}_{tag}_eval_y"])
+
+
+def test_conv_loops_match_reference_layer(golden_next):
+    """The oracle's chunk / tree loops on the reference layer's own tables and index tables."""
+    g = golden_next
+    state = {k[len("conv_state."):]: v for k, v in g.items() if k.startswith("conv_state.")}
+    def sub(prefix):
+        n = 1 + max(int(k.split(".")[len(prefix.split(".")) + 1]) for k in state if k.startswith(prefix + ".nodes."))
+        return state[prefix + "._mapping_indices"].astype(np.int64), np.stack([state[f"{prefix}.nodes.{i}.luts"] for i in range(n)])
+    chunks = [sub(f"first_layer_chunks.{c}") for c in range(2)]
+    trees = [[sub(f"trees.{t}.{l}") for l in range(2)] for t in range(3)]
+    alpha, beta = float(state["trees.0.0.nodes.0.alpha"]), float(state["trees.0.0.nodes.0.beta"])
+    x = g["conv_x"]
+    patches = orc.conv_unfold(x, (2, 2), (1, 1), (0, 0))
+    fwd = lambda m, i, t: orc.dwn_layer_forward(m, i, t)[:, :, 0]
+    out, acts = orc.conv_trees_forward(patches, chunks, trees, 4, fwd)
+    y = out.reshape(2, 9, 3).transpose(0, 2, 1).reshape(2, 3, 3, 3)
+    assert np.array_equal(y, g["conv_y"])
+    gout = g["conv_gy"].reshape(2, 3, 9).transpose(0, 2, 1).reshape(-1, 3)
+    bwd = lambda m, i, t, gy: orc.dwn_layer_backward(m, i, t, gy[:, :, None], alpha, beta)
+    gp, gch, gtr = orc.conv_trees_backward(patches, chunks, trees, 4, acts, gout, bwd)
+    assert np.allclose(orc.conv_fold(gp, x.shape, (2, 2), (1, 1), (0, 0)), g["conv_gx"], rtol=1e-5, atol=1e-6)
+    assert np.allclose(gch[1][3], g["conv_grad.first_layer_chunks.1.nodes.3.luts"], rtol=1e-5, atol=1e-6)
+    assert np.allclose(gtr[2][1][0], g["conv_grad.trees.2.1.nodes.0.luts"], rtol=1e-5, atol=1e-6)
+    assert np.allclose(gtr[0][0][1], g["conv_grad.trees.0.0.nodes.1.luts"], rtol=1e-5, atol=1e-6)
