@@ -237,3 +237,33 @@ def test_convolutional_layer_construction_matches_reference(golden_next):
     assert np.array_equal(glayer.trees[4][0]._mapping_indices.numpy(), g["gconv_tree4_idx"])
     assert np.array_equal(glayer.first_layer_chunks[0].nodes[0].raw_weights.detach().numpy(), g["gconv_first_raw"])
     assert np.array_equal(glayer.trees[4][0].nodes[0].raw_weights.detach().numpy(), g["gconv_last_raw"])
+
+
+def test_argument_checks_of_the_later_entry_points_need_no_gpu():
+    """Null pointers, bad sizes and unsupported geometries are refused before anything is launched."""
+    from difflut_amd import _native as nat
+
+    lib = nat.lib()
+    one = ctypes.c_void_p(64)  # any non-null value: the checks below fail before it is dereferenced
+    assert lib.dl_unfold(None, one, None, 1, 1, 4, 4, 2, 2, 1, 1, 0, 0, None) == -1
+    assert lib.dl_unfold(one, None, None, 1, 1, 4, 4, 2, 2, 1, 1, 0, 0, None) == -1        # no output asked for
+    assert lib.dl_unfold(one, one, None, 1, 1, 4, 4, 5, 5, 1, 1, 0, 0, None) == -2         # window larger than image
+    assert lib.dl_unfold(one, one, None, 1, 1, 4, 4, 2, 2, 0, 1, 0, 0, None) == -2         # zero stride
+    assert lib.dl_unfold(one, one, None, 1, 64, 20, 20, 9, 9, 1, 1, 0, 0, None) == -3      # 5184 columns > 4096
+    assert lib.dl_fold(None, 0, one, 1, 1, 4, 4, 2, 2, 1, 1, 0, 0, None) == -1
+    assert lib.dl_unfold_rows(3, 28, 28, 5, 5, 1, 1, 0, 0) == 3 * 24 * 24
+    assert lib.dl_unfold_rows(3, 28, 28, 5, 5, 2, 2, 2, 2) == 3 * 14 * 14
+    assert lib.dl_unfold_rows(3, 4, 4, 5, 5, 1, 1, 0, 0) == 0
+    assert lib.dl_table_sigmoid_fwd(one, one, 0, None) == -2 and lib.dl_table_sigmoid_fwd(None, one, 8, None) == -1
+    assert lib.dl_table_sigmoid_bwd(one, None, one, 8, None) == -1
+    assert lib.dl_dwn_stable_layer_bwd(None, one, one, one, one, one, one, None, one, one, one, 1 << 30,
+                                       64, 8, 4, 2, 1, None) == -1                          # no gradient scale
+    assert lib.dl_dwn_stable_layer_bwd(None, one, one, one, one, one, one, one, one, one, one, 0,
+                                       64, 8, 4, 2, 1, None) == -4                          # workspace too small
+    assert lib.dl_hybrid_layer_bwd(one, one, one, one, one, one, one, one, one, 0, 64, 8, 4, 2, 1, None) == -4
+    assert lib.dl_hybrid_layer_bwd(one, one, one, one, one, one, one, one, one, 1 << 30, 64, 8, 4, 0, 1, None) == -2
+    assert lib.dl_thermometer_planes(one, None, one, 4, 4, 2, None) == -1
+    assert lib.dl_thermometer_planes(one, one, one, 4, 0, 2, None) == -2
+    dims = (4096, 16384, 8192, 6, 1)
+    assert lib.dl_hybrid_bwd_workspace_bytes(*dims) < lib.dl_prob_bwd_workspace_bytes(*dims)
+    assert lib.dl_hybrid_bwd_workspace_bytes(*dims) >= 4096 * (16384 + 8192 + 6 * 8192) * 4
