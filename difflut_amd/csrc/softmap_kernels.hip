@@ -118,6 +118,11 @@ struct SoftmapArgs {
     int inner_count, outer_count, col_tiles, red_chunk;
     const unsigned short *Eb;  // precision 1: bf16 softmax numerators [M][I]
     const float *rs;           // precision 1: 1 / row sum [M]
+    // precision 1: operands rounded to bf16 once, in the layout their product reads
+    const unsigned short *xb;   // x [B][I]                      (forward A operand)
+    const unsigned *xp;         // x pairs [ceil(B/2)][I]: (x[2p][i], x[2p+1][i])   (gW B operand)
+    const unsigned short *gms;  // gm[b][o] / sum[o], [B][M]     (gx A operand)
+    const unsigned *gmp;        // gm pairs [ceil(B/2)][M]       (gW A operand)
 };
 
 // MODE 0: forward   rows=b cols=o red=i   A = x[b,i]  (red contiguous)   B = S[o,i] (red contiguous)
@@ -377,8 +382,9 @@ static void softmap_launch(const SoftmapArgs &g, hipStream_t s) {
 // written once, rounded to bf16, by the row-statistics pass (301 MB for the 48000 x 3136 case, kept
 // with the statistics for the backward); 1/sum stays a per-row fp32 factor that is applied to the
 // forward output, to the gm operand of the gx product and in the gW epilogue.  x and gm are rounded
-// to bf16 (nearest even) while they are staged.  A lane feeds the MFMA eight consecutive k of one
-// row, so LDS holds a stage row-major, As[row][32 k] with 16 bytes of padding per row.
+// to bf16 (nearest even) once per call by a packing pass (softmap_pack_bf16), into the layout the
+// staging code copies to LDS unchanged.  A lane feeds the MFMA eight consecutive k of one row, so LDS
+// holds a stage row-major, As[row][32 k] with 16 bytes of padding per row.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
@@ -430,6 +436,29 @@ __global__ __launch_bounds__(256) void softmap_rowstats_bf16(const float *__rest
     if (lane == 0) { mxs[row] = mx; rss[row] = 1.0f / sum; }
 }
 
+// Operands of the bf16 products, rounded once (nearest even) into the layout the staging code copies:
+// row-major bf16 for an operand that is contiguous along the reduction, and (k, k+1) pairs for one that is
+// contiguous along the rows/columns (an MFMA lane wants consecutive k next to each other).
+// src [R][C] fp32 -> rows [R][C] bf16 (optionally scaled per column) and/or pairs [ceil(R/2)][C] u32.
+__global__ __launch_bounds__(256) void softmap_pack_bf16(const float *__restrict__ src, const float *__restrict__ colscale,
+                                                          unsigned short *__restrict__ rows, unsigned *__restrict__ pairs,
+                                                          int R, int C) {
+    const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+    const int RP = (R + 1) / 2;
+    if (e >= (long long)RP * C) return;
+    const int c = (int)(e % C);
+    const int rp = (int)(e / C);
+    const float v0 = src[(size_t)(2 * rp) * C + c];
+    const float v1 = 2 * rp + 1 < R ? src[(size_t)(2 * rp + 1) * C + c] : 0.0f;
+    if (pairs) pairs[e] = softmap_pk_bf16(v0, v1);
+    if (rows) {
+        const float f = colscale ? colscale[c] : 1.0f;
+        const unsigned pk = softmap_pk_bf16(v0 * f, v1 * f);
+        rows[(size_t)(2 * rp) * C + c] = (unsigned short)(pk & 0xffffu);
+        if (2 * rp + 1 < R) rows[(size_t)(2 * rp + 1) * C + c] = (unsigned short)(pk >> 16);
+    }
+}
+
 template <int MODE, bool EDGE>
 __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *lds, int rt, int ct, int zc) {
     constexpr int KC = SB_K;
@@ -449,51 +478,52 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
 
-    // ---- A operand, fp32 in memory (x; gm scaled by 1/sum of its column in the gx product; gm).
-    // red-contiguous: float4 along k, 8 per row, rows a_o + 32 p.  row-contiguous: float4 along the
-    // rows for one k; piece p holds k = 2 a_o + (p & 1) + 16 (p >> 1), so pieces 2j and 2j+1 are
-    // neighbours in k and go to LDS as packed pairs.
-    float4 pa[4];
-    float4 ars[2];  // gx product: 1/sum of the four k of pieces {0,1} and {2,3}
-    const int a_q = A_RED_CONTIG ? (tid & 7) : (tid & 31), a_o = A_RED_CONTIG ? (tid >> 3) : (tid >> 5);
+    // ---- A operand, bf16 in memory (softmap_pack_bf16): two 16-byte pieces per thread and stage.
+    // red-contiguous (x rows; gm / sum rows): 8 consecutive k of row a_o + 64 p, copied as they are.
+    // row-contiguous (gW: gm pairs): the pair kp = a_o + 8 p of rows 4 a_q .. 4 a_q + 3.
+    uint4 pa[2];
+    const int a_q = A_RED_CONTIG ? (tid & 3) : (tid & 31), a_o = A_RED_CONTIG ? (tid >> 2) : (tid >> 5);
+    const unsigned short *__restrict__ arow = MODE == 0 ? g.xb : g.gms;
     const int lda = MODE == 0 ? I : M;
-    auto k_of = [](int o, int p) { return 2 * o + (p & 1) + 16 * (p >> 1); };
-    auto in_a = [&](int row, int k) -> float {
-        if (row >= R || k >= k_end) return 0.0f;
-        if (MODE == 0) return x[(size_t)row * I + k];
-        if (MODE == 1) return gm[(size_t)row * M + k] * rs[k];
-        return gm[(size_t)k * M + row];
-    };
+    const int kp_end = (k_end + 1) / 2;
     auto fetch_a = [&](int p, int k0) __attribute__((always_inline)) {
         if (A_RED_CONTIG) {
-            const int row = r0 + a_o + 32 * p, k = k0 + a_q * 4;
-            if (EDGE) pa[p] = make_float4(in_a(row, k), in_a(row, k + 1), in_a(row, k + 2), in_a(row, k + 3));
-            else {
-                pa[p] = *reinterpret_cast<const float4 *>((MODE == 0 ? x : gm) + (size_t)row * lda + k);
-                if (MODE == 1 && (p & 1) == 0) ars[p >> 1] = *reinterpret_cast<const float4 *>(rs + k);
+            const int row = r0 + a_o + 64 * p, k = k0 + a_q * 8;
+            if (EDGE) {
+                unsigned w[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const unsigned lo = (row < R && k + 2 * j < k_end) ? arow[(size_t)row * lda + k + 2 * j] : 0u;
+                    const unsigned hi = (row < R && k + 2 * j + 1 < k_end) ? arow[(size_t)row * lda + k + 2 * j + 1] : 0u;
+                    w[j] = lo | (hi << 16);
+                }
+                pa[p] = make_uint4(w[0], w[1], w[2], w[3]);
+            } else {
+                pa[p] = *reinterpret_cast<const uint4 *>(arow + (size_t)row * lda + k);
             }
         } else {
-            const int k = k0 + k_of(a_o, p), row = r0 + a_q * 4;
-            if (EDGE) pa[p] = make_float4(in_a(row, k), in_a(row + 1, k), in_a(row + 2, k), in_a(row + 3, k));
-            else pa[p] = *reinterpret_cast<const float4 *>(gm + (size_t)k * M + row);
+            const int kp = (k0 >> 1) + a_o + 8 * p, row = r0 + a_q * 4;
+            if (EDGE) {
+                unsigned w[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) w[j] = (kp < kp_end && row + j < R) ? g.gmp[(size_t)kp * M + row + j] : 0u;
+                pa[p] = make_uint4(w[0], w[1], w[2], w[3]);
+            } else {
+                pa[p] = *reinterpret_cast<const uint4 *>(g.gmp + (size_t)kp * M + row);
+            }
         }
     };
     auto commit_a = [&](int p, int buf) __attribute__((always_inline)) {
         char *Ab = As + buf * STAGE;
+        const uint4 v = make_uint4(pa[p].x, pa[p].y, pa[p].z, pa[p].w);
         if (A_RED_CONTIG) {
-            float4 v = make_float4(pa[p].x, pa[p].y, pa[p].z, pa[p].w);
-            if (!EDGE && MODE == 1) {
-                const float4 f = ars[p >> 1];
-                v.x *= f.x; v.y *= f.y; v.z *= f.z; v.w *= f.w;
-            }
-            *reinterpret_cast<uint2 *>(Ab + (a_o + 32 * p) * SB_LD + a_q * 8) =
-                make_uint2(softmap_pk_bf16(v.x, v.y), softmap_pk_bf16(v.z, v.w));
-        } else if (p & 1) {
-            char *d = Ab + (a_q * 4) * SB_LD + k_of(a_o, p - 1) * 2;
-            *reinterpret_cast<unsigned *>(d) = softmap_pk_bf16(pa[p - 1].x, pa[p].x);
-            *reinterpret_cast<unsigned *>(d + SB_LD) = softmap_pk_bf16(pa[p - 1].y, pa[p].y);
-            *reinterpret_cast<unsigned *>(d + 2 * SB_LD) = softmap_pk_bf16(pa[p - 1].z, pa[p].z);
-            *reinterpret_cast<unsigned *>(d + 3 * SB_LD) = softmap_pk_bf16(pa[p - 1].w, pa[p].w);
+            *reinterpret_cast<uint4 *>(Ab + (a_o + 64 * p) * SB_LD + a_q * 16) = v;
+        } else {
+            char *d = Ab + (a_q * 4) * SB_LD + (a_o + 8 * p) * 4;
+            *reinterpret_cast<unsigned *>(d) = v.x;
+            *reinterpret_cast<unsigned *>(d + SB_LD) = v.y;
+            *reinterpret_cast<unsigned *>(d + 2 * SB_LD) = v.z;
+            *reinterpret_cast<unsigned *>(d + 3 * SB_LD) = v.w;
         }
     };
 
@@ -501,9 +531,9 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
     //  MODE 0: exp2((W[o, k] - max[o]) * scale) from the fp32 W, red-contiguous, four float4 pieces like
     //          the A operand (the bf16 copy E would be read in half cache lines per stage here)
     //  MODE 1: E[k, i] bf16, column-contiguous: rows 2 kp and 2 kp + 1, 8 columns each -> packed pairs
-    //  MODE 2: x[k, i] fp32, column-contiguous: as the A operand
+    //  MODE 2: x pairs [kp, i], column-contiguous: as the A operand of that mode
     uint4 pe[2];
-    float4 pb[MODE == 1 ? 1 : 4];
+    float4 pb[MODE == 0 ? 4 : 1];
     float bmx[4];  // MODE 0: row maxima of the W rows this thread stages
     const int e_q = tid & 15, e_o = tid >> 4;
     const int b_q = MODE == 0 ? (tid & 7) : (tid & 31), b_o = MODE == 0 ? (tid >> 3) : (tid >> 5);
@@ -535,10 +565,15 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
                 pe[p] = *reinterpret_cast<const uint4 *>(Eb + (size_t)k * I + col);
             }
         } else {
-            const int k = k0 + k_of(b_o, p), col = c0 + b_q * 4;
-            auto xv = [&](int kk, int cc) -> float { return (kk < k_end && cc < C) ? x[(size_t)kk * I + cc] : 0.0f; };
-            if (EDGE) pb[p] = make_float4(xv(k, col), xv(k, col + 1), xv(k, col + 2), xv(k, col + 3));
-            else pb[p] = *reinterpret_cast<const float4 *>(x + (size_t)k * I + col);
+            const int kp = (k0 >> 1) + b_o + 8 * p, col = c0 + b_q * 4;
+            if (EDGE) {
+                unsigned w[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) w[j] = (kp < kp_end && col + j < C) ? g.xp[(size_t)kp * I + col + j] : 0u;
+                pe[p] = make_uint4(w[0], w[1], w[2], w[3]);
+            } else {
+                pe[p] = *reinterpret_cast<const uint4 *>(g.xp + (size_t)kp * I + col);
+            }
         }
     };
     auto commit_b = [&](int p, int buf) __attribute__((always_inline)) {
@@ -562,24 +597,26 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
                     *reinterpret_cast<unsigned *>(d + j * SB_LD) = v;
                 }
             }
-        } else if (p & 1) {
-            char *d = Bb + (b_q * 4) * SB_LD + k_of(b_o, p - 1) * 2;
-            *reinterpret_cast<unsigned *>(d) = softmap_pk_bf16(pb[p - 1].x, pb[p].x);
-            *reinterpret_cast<unsigned *>(d + SB_LD) = softmap_pk_bf16(pb[p - 1].y, pb[p].y);
-            *reinterpret_cast<unsigned *>(d + 2 * SB_LD) = softmap_pk_bf16(pb[p - 1].z, pb[p].z);
-            *reinterpret_cast<unsigned *>(d + 3 * SB_LD) = softmap_pk_bf16(pb[p - 1].w, pb[p].w);
+        } else {
+            char *d = Bb + (b_q * 4) * SB_LD + (b_o + 8 * p) * 4;
+            *reinterpret_cast<unsigned *>(d) = pe[p].x;
+            *reinterpret_cast<unsigned *>(d + SB_LD) = pe[p].y;
+            *reinterpret_cast<unsigned *>(d + 2 * SB_LD) = pe[p].z;
+            *reinterpret_cast<unsigned *>(d + 3 * SB_LD) = pe[p].w;
         }
     };
     // pieces handled after the first (h = 0) and the second (h = 1) half of a stage's MFMAs
     // (the two rows of a MODE 1 pair travel together in the second half: they are packed in one go)
     auto fetch_half = [&](int h, int k0) __attribute__((always_inline)) {
-        fetch_a(2 * h, k0); fetch_a(2 * h + 1, k0);
-        if (MODE != 1) { fetch_b(2 * h, k0); fetch_b(2 * h + 1, k0); }
+        fetch_a(h, k0);
+        if (MODE == 0) { fetch_b(2 * h, k0); fetch_b(2 * h + 1, k0); }
+        else if (MODE == 2) fetch_b(h, k0);
         else if (h == 1) { fetch_b(0, k0); fetch_b(1, k0); }
     };
     auto commit_half = [&](int h, int buf) __attribute__((always_inline)) {
-        commit_a(2 * h, buf); commit_a(2 * h + 1, buf);
-        if (MODE != 1) { commit_b(2 * h, buf); commit_b(2 * h + 1, buf); }
+        commit_a(h, buf);
+        if (MODE == 0) { commit_b(2 * h, buf); commit_b(2 * h + 1, buf); }
+        else if (MODE == 2) commit_b(h, buf);
         else if (h == 1) commit_b(1, buf);
     };
 
@@ -678,8 +715,9 @@ __global__ __launch_bounds__(256, 3) void softmap_mfma_bf16(SoftmapArgs g) {
     const int R = MODE == 2 ? g.M : g.B, C = MODE == 0 ? g.M : g.I;
     const int KD = MODE == 0 ? g.I : (MODE == 1 ? g.M : g.B);
     const int k_begin = zc * g.red_chunk, k_end = min(KD, k_begin + g.red_chunk);
+    // whole tiles and stages, and rows of the bf16 operands that start on 16-byte boundaries
     const bool inside = (rt + 1) * SM_T <= R && (ct + 1) * SM_T <= C && (k_end - k_begin) % SB_K == 0 &&
-                        g.red_chunk % 4 == 0 && g.I % 8 == 0 && g.M % 4 == 0;
+                        g.red_chunk % 8 == 0 && g.I % 8 == 0 && g.M % 8 == 0;
     if (inside) softmap_tile_bf16<MODE, false>(g, lds, rt, ct, zc);
     else softmap_tile_bf16<MODE, true>(g, lds, rt, ct, zc);
 }
@@ -718,27 +756,47 @@ extern "C" size_t dl_soft_map_saved_bytes(int B, int I, int M, int precision) {
     return softmap_stats_bytes(M) + (precision == 1 ? dl_align256((size_t)M * I * sizeof(unsigned short)) : 0);
 }
 
+// workspace: r [M], the partial gx products, and for bf16 operands the packed copies of x and gm
+static inline size_t softmap_r_bytes(int M) { return dl_align256((size_t)M * sizeof(float)); }
+static inline size_t softmap_part_bytes(int B, int I, int M, int precision) {
+    return dl_align256((size_t)softmap_gx_chunks(B, I, M, precision) * B * I * sizeof(float));
+}
+static inline size_t softmap_rows_bytes(int R, int C) { return dl_align256((size_t)R * C * sizeof(unsigned short)); }
+static inline size_t softmap_pairs_bytes(int R, int C) { return dl_align256((size_t)((R + 1) / 2) * C * sizeof(unsigned)); }
 extern "C" size_t dl_soft_map_workspace_bytes(int B, int I, int M, int precision) {
     if (B <= 0 || I <= 0 || M <= 0) return 256;
-    return dl_align256((size_t)M * sizeof(float)) +
-           dl_align256((size_t)softmap_gx_chunks(B, I, M, precision) * B * I * sizeof(float));
+    size_t bytes = softmap_r_bytes(M) + softmap_part_bytes(B, I, M, precision);
+    if (precision == 1)
+        bytes += softmap_rows_bytes(B, I) + softmap_pairs_bytes(B, I) + softmap_rows_bytes(B, M) + softmap_pairs_bytes(B, M);
+    return bytes;
+}
+static void softmap_pack(const float *src, const float *colscale, unsigned short *rows, unsigned *pairs, int R, int C,
+                         hipStream_t s) {
+    const long long total = (long long)((R + 1) / 2) * C;
+    DL_TIMED("softmap_pack_bf16", s,
+             (softmap_pack_bf16<<<dl_ceil_div(total, 256), 256, 0, s>>>(src, colscale, rows, pairs, R, C)));
 }
 
 extern "C" int dl_soft_map_fwd(const float *x, const float *W, float tau, float *m, float *stats, void *ws,
                                size_t ws_bytes, int B, int I, int M, int precision, void *stream) {
-    (void)ws; (void)ws_bytes;
     if (!x || !W || !m || !stats) return DL_ERR_NULL;
     int rc = softmap_check(B, I, M, precision);
     if (rc) return rc;
     if (!(tau > 0.0f)) return DL_ERR_SHAPE;
+    if (precision == 1 && !ws) return DL_ERR_NULL;
+    if (precision == 1 && ws_bytes < dl_soft_map_workspace_bytes(B, I, M, precision)) return DL_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
     const float inv_tau = 1.0f / tau, scale = SM_LOG2E / tau;
     SoftmapArgs g{x, W, stats, nullptr, nullptr, scale, inv_tau, m, B, I, M,
-                  dl_ceil_div(B, SM_T), dl_ceil_div(M, SM_T), 1, dl_ceil_div(I, 4) * 4, nullptr, nullptr};
+                  dl_ceil_div(B, SM_T), dl_ceil_div(M, SM_T), 1, dl_ceil_div(I, 8) * 8, nullptr, nullptr,
+                  nullptr, nullptr, nullptr, nullptr};
     if (precision == 1) {
         unsigned short *Eb = (unsigned short *)((char *)stats + softmap_stats_bytes(M));
         DL_TIMED("softmap_rowstats_bf16", s,
                  (softmap_rowstats_bf16<<<dl_ceil_div(M, 4), 256, 0, s>>>(W, scale, stats, stats + M, Eb, M, I)));
+        unsigned short *xb = (unsigned short *)((char *)ws + softmap_r_bytes(M) + softmap_part_bytes(B, I, M, precision));
+        softmap_pack(x, nullptr, xb, nullptr, B, I, s);
+        g.xb = xb;
         g.Eb = Eb;
         g.rs = stats + M;
         DL_TIMED("softmap_bf16_fwd", s, (softmap_launch_bf16<0>(g, s)));
@@ -760,7 +818,7 @@ extern "C" int dl_soft_map_bwd(const float *x, const float *W, float tau, const 
     hipStream_t s = (hipStream_t)stream;
     const float inv_tau = 1.0f / tau, scale = SM_LOG2E / tau;
     float *r = (float *)ws;
-    float *part = (float *)((char *)ws + dl_align256((size_t)M * sizeof(float)));
+    float *part = (float *)((char *)ws + softmap_r_bytes(M));
     const int chunks = softmap_gx_chunks(B, I, M, precision);
     int red_chunk = dl_ceil_div(M, chunks);
     red_chunk = dl_ceil_div(red_chunk, 32) * 32;  // whole stages, so float4 loads stay aligned
@@ -768,8 +826,19 @@ extern "C" int dl_soft_map_bwd(const float *x, const float *W, float tau, const 
     const unsigned short *Eb = precision == 1 ? (const unsigned short *)((const char *)stats + softmap_stats_bytes(M)) : nullptr;
     const float *rs = precision == 1 ? stats + M : nullptr;
     DL_TIMED("softmap_rowdot", s, (softmap_rowdot<<<dl_ceil_div(M, 32), 256, 0, s>>>(gm, m, r, B, M)));
+    unsigned *xp = nullptr, *gmp = nullptr;
+    unsigned short *gms = nullptr;
+    if (precision == 1) {
+        char *w = (char *)ws + softmap_r_bytes(M) + softmap_part_bytes(B, I, M, precision) + softmap_rows_bytes(B, I);
+        xp = (unsigned *)w; w += softmap_pairs_bytes(B, I);
+        gms = (unsigned short *)w; w += softmap_rows_bytes(B, M);
+        gmp = (unsigned *)w;
+        softmap_pack(x, nullptr, nullptr, xp, B, I, s);
+        softmap_pack(gm, rs, gms, gmp, B, M, s);
+    }
     const SoftmapArgs ggx{x, W, stats, gm, nullptr, scale, inv_tau, used_chunks > 1 ? part : gx, B, I, M,
-                          dl_ceil_div(B, SM_T), col_tiles * used_chunks, col_tiles, red_chunk, Eb, rs};
+                          dl_ceil_div(B, SM_T), col_tiles * used_chunks, col_tiles, red_chunk, Eb, rs,
+                          nullptr, xp, gms, gmp};
     if (precision == 1) DL_TIMED("softmap_bf16_gx", s, (softmap_launch_bf16<1>(ggx, s)));
     else DL_TIMED("softmap_mfma_gx", s, (softmap_launch<1, SM_K>(ggx, s)));
     if (used_chunks > 1)
@@ -777,7 +846,8 @@ extern "C" int dl_soft_map_bwd(const float *x, const float *W, float tau, const 
                  (softmap_reduce_chunks<<<dl_ceil_div((long long)B * I, 256), 256, 0, s>>>(part, gx, (long long)B * I,
                                                                                          used_chunks)));
     const SoftmapArgs ggw{x, W, stats, gm, r, scale, inv_tau, gW, B, I, M,
-                          col_tiles, dl_ceil_div(M, SM_T), 1, dl_ceil_div(B, 4) * 4, Eb, rs};
+                          col_tiles, dl_ceil_div(M, SM_T), 1, dl_ceil_div(B, 8) * 8, Eb, rs,
+                          nullptr, xp, gms, gmp};
     if (precision == 1) DL_TIMED("softmap_bf16_gw", s, (softmap_launch_bf16<2>(ggw, s)));
     else DL_TIMED("softmap_mfma_gw", s, (softmap_launch<2, SM_K>(ggw, s)));
     return dl_launch_status();
