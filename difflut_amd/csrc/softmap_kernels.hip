@@ -120,9 +120,9 @@ struct SoftmapArgs {
     const float *rs;           // precision 1: 1 / row sum [M]
     // precision 1: operands rounded to bf16 once, in the layout their product reads
     const unsigned short *xb;   // x [B][I]                      (forward A operand)
-    const unsigned *xp;         // x pairs [ceil(B/2)][I]: (x[2p][i], x[2p+1][i])   (gW B operand)
+    const uint4 *x8;            // x in blocks of 8 batch rows: [ceil(B/8)][I] x 8 bf16   (gW B operand)
     const unsigned short *gms;  // gm[b][o] / sum[o], [B][M]     (gx A operand)
-    const unsigned *gmp;        // gm pairs [ceil(B/2)][M]       (gW A operand)
+    const uint4 *gm8;           // gm in blocks of 8 batch rows: [ceil(B/8)][M] x 8 bf16  (gW A operand)
 };
 
 // MODE 0: forward   rows=b cols=o red=i   A = x[b,i]  (red contiguous)   B = S[o,i] (red contiguous)
@@ -437,25 +437,30 @@ __global__ __launch_bounds__(256) void softmap_rowstats_bf16(const float *__rest
 }
 
 // Operands of the bf16 products, rounded once (nearest even) into the layout the staging code copies:
-// row-major bf16 for an operand that is contiguous along the reduction, and (k, k+1) pairs for one that is
-// contiguous along the rows/columns (an MFMA lane wants consecutive k next to each other).
-// src [R][C] fp32 -> rows [R][C] bf16 (optionally scaled per column) and/or pairs [ceil(R/2)][C] u32.
+// row-major bf16 for an operand that is contiguous along the reduction; for one that is contiguous
+// along the rows / columns of the product (the reduction runs over its rows) blocks of 8 consecutive
+// reduction steps per element, because an MFMA lane wants 8 consecutive k side by side - the
+// transposition happens here, through coalesced accesses, and not as bank-conflicting LDS stores.
+// src [R][C] fp32 -> rows [R][C] bf16 (optionally scaled per column) and/or blocks [ceil(R/8)][C] x 8 bf16.
 __global__ __launch_bounds__(256) void softmap_pack_bf16(const float *__restrict__ src, const float *__restrict__ colscale,
-                                                          unsigned short *__restrict__ rows, unsigned *__restrict__ pairs,
+                                                          unsigned short *__restrict__ rows, uint4 *__restrict__ blocks,
                                                           int R, int C) {
     const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
-    const int RP = (R + 1) / 2;
-    if (e >= (long long)RP * C) return;
+    const int RB = (R + 7) / 8;
+    if (e >= (long long)RB * C) return;
     const int c = (int)(e % C);
-    const int rp = (int)(e / C);
-    const float v0 = src[(size_t)(2 * rp) * C + c];
-    const float v1 = 2 * rp + 1 < R ? src[(size_t)(2 * rp + 1) * C + c] : 0.0f;
-    if (pairs) pairs[e] = softmap_pk_bf16(v0, v1);
+    const int rb = (int)(e / C);
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = 8 * rb + i < R ? src[(size_t)(8 * rb + i) * C + c] : 0.0f;
+    if (blocks)
+        blocks[e] = make_uint4(softmap_pk_bf16(v[0], v[1]), softmap_pk_bf16(v[2], v[3]), softmap_pk_bf16(v[4], v[5]),
+                               softmap_pk_bf16(v[6], v[7]));
     if (rows) {
         const float f = colscale ? colscale[c] : 1.0f;
-        const unsigned pk = softmap_pk_bf16(v0 * f, v1 * f);
-        rows[(size_t)(2 * rp) * C + c] = (unsigned short)(pk & 0xffffu);
-        if (2 * rp + 1 < R) rows[(size_t)(2 * rp + 1) * C + c] = (unsigned short)(pk >> 16);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (8 * rb + i < R) rows[(size_t)(8 * rb + i) * C + c] = (unsigned short)(softmap_pk_bf16(v[i] * f, 0.0f) & 0xffffu);
     }
 }
 
@@ -480,12 +485,13 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
 
     // ---- A operand, bf16 in memory (softmap_pack_bf16): two 16-byte pieces per thread and stage.
     // red-contiguous (x rows; gm / sum rows): 8 consecutive k of row a_o + 64 p, copied as they are.
-    // row-contiguous (gW: gm pairs): the pair kp = a_o + 8 p of rows 4 a_q .. 4 a_q + 3.
+    // row-contiguous (gW: gm in blocks of 8 k): k-block a_q (= my wavefront) of row a_o + 64 p, so a
+    // wavefront reads 64 consecutive rows = 1 KB and stores them to 64 consecutive LDS rows.
     uint4 pa[2];
-    const int a_q = A_RED_CONTIG ? (tid & 3) : (tid & 31), a_o = A_RED_CONTIG ? (tid >> 2) : (tid >> 5);
+    const int a_q = A_RED_CONTIG ? (tid & 3) : (tid >> 6), a_o = A_RED_CONTIG ? (tid >> 2) : (tid & 63);
     const unsigned short *__restrict__ arow = MODE == 0 ? g.xb : g.gms;
     const int lda = MODE == 0 ? I : M;
-    const int kp_end = (k_end + 1) / 2;
+    const int kb_end = (k_end + 7) / 8;
     auto fetch_a = [&](int p, int k0) __attribute__((always_inline)) {
         if (A_RED_CONTIG) {
             const int row = r0 + a_o + 64 * p, k = k0 + a_q * 8;
@@ -502,36 +508,22 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
                 pa[p] = *reinterpret_cast<const uint4 *>(arow + (size_t)row * lda + k);
             }
         } else {
-            const int kp = (k0 >> 1) + a_o + 8 * p, row = r0 + a_q * 4;
-            if (EDGE) {
-                unsigned w[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) w[j] = (kp < kp_end && row + j < R) ? g.gmp[(size_t)kp * M + row + j] : 0u;
-                pa[p] = make_uint4(w[0], w[1], w[2], w[3]);
-            } else {
-                pa[p] = *reinterpret_cast<const uint4 *>(g.gmp + (size_t)kp * M + row);
-            }
+            const int kb = (k0 >> 3) + a_q, row = r0 + a_o + 64 * p;
+            if (EDGE) pa[p] = (kb < kb_end && row < R) ? g.gm8[(size_t)kb * M + row] : make_uint4(0u, 0u, 0u, 0u);
+            else pa[p] = g.gm8[(size_t)kb * M + row];
         }
     };
     auto commit_a = [&](int p, int buf) __attribute__((always_inline)) {
         char *Ab = As + buf * STAGE;
         const uint4 v = make_uint4(pa[p].x, pa[p].y, pa[p].z, pa[p].w);
-        if (A_RED_CONTIG) {
-            *reinterpret_cast<uint4 *>(Ab + (a_o + 64 * p) * SB_LD + a_q * 16) = v;
-        } else {
-            char *d = Ab + (a_q * 4) * SB_LD + (a_o + 8 * p) * 4;
-            *reinterpret_cast<unsigned *>(d) = v.x;
-            *reinterpret_cast<unsigned *>(d + SB_LD) = v.y;
-            *reinterpret_cast<unsigned *>(d + 2 * SB_LD) = v.z;
-            *reinterpret_cast<unsigned *>(d + 3 * SB_LD) = v.w;
-        }
+        *reinterpret_cast<uint4 *>(Ab + (a_o + 64 * p) * SB_LD + a_q * 16) = v;  // both forms: 8 k of one row
     };
 
     // ---- B operand
     //  MODE 0: exp2((W[o, k] - max[o]) * scale) from the fp32 W, red-contiguous, four float4 pieces like
     //          the A operand (the bf16 copy E would be read in half cache lines per stage here)
     //  MODE 1: E[k, i] bf16, column-contiguous: rows 2 kp and 2 kp + 1, 8 columns each -> packed pairs
-    //  MODE 2: x pairs [kp, i], column-contiguous: as the A operand of that mode
+    //  MODE 2: x in blocks of 8 k, column-contiguous: as the A operand of that mode
     uint4 pe[2];
     float4 pb[MODE == 0 ? 4 : 1];
     float bmx[4];  // MODE 0: row maxima of the W rows this thread stages
@@ -565,15 +557,9 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
                 pe[p] = *reinterpret_cast<const uint4 *>(Eb + (size_t)k * I + col);
             }
         } else {
-            const int kp = (k0 >> 1) + b_o + 8 * p, col = c0 + b_q * 4;
-            if (EDGE) {
-                unsigned w[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) w[j] = (kp < kp_end && col + j < C) ? g.xp[(size_t)kp * I + col + j] : 0u;
-                pe[p] = make_uint4(w[0], w[1], w[2], w[3]);
-            } else {
-                pe[p] = *reinterpret_cast<const uint4 *>(g.xp + (size_t)kp * I + col);
-            }
+            const int kb = (k0 >> 3) + (tid >> 6), col = c0 + (tid & 63) + 64 * p;
+            if (EDGE) pe[p] = (kb < kb_end && col < C) ? g.x8[(size_t)kb * I + col] : make_uint4(0u, 0u, 0u, 0u);
+            else pe[p] = g.x8[(size_t)kb * I + col];
         }
     };
     auto commit_b = [&](int p, int buf) __attribute__((always_inline)) {
@@ -598,11 +584,8 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
                 }
             }
         } else {
-            char *d = Bb + (b_q * 4) * SB_LD + (b_o + 8 * p) * 4;
-            *reinterpret_cast<unsigned *>(d) = pe[p].x;
-            *reinterpret_cast<unsigned *>(d + SB_LD) = pe[p].y;
-            *reinterpret_cast<unsigned *>(d + 2 * SB_LD) = pe[p].z;
-            *reinterpret_cast<unsigned *>(d + 3 * SB_LD) = pe[p].w;
+            *reinterpret_cast<uint4 *>(Bb + ((tid & 63) + 64 * p) * SB_LD + (tid >> 6) * 16) =
+                make_uint4(pe[p].x, pe[p].y, pe[p].z, pe[p].w);
         }
     };
     // pieces handled after the first (h = 0) and the second (h = 1) half of a stage's MFMAs
@@ -672,6 +655,43 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
             rowst[tid * 2 + 1] = g.r[row];
         }
         __syncthreads();
+        if (!EDGE) {
+            // Interior tiles: a wavefront's 64 x 64 block of G goes through LDS 32 rows at a time, so that
+            // a lane owns four consecutive columns of a row: 8-byte loads of the numerators, 16-byte stores of
+            // gW in runs of 256 bytes per row (the accumulator layout itself gives 2-byte loads and 4-byte
+            // stores in runs of 128).  Each wavefront uses its own LDS region; no block barrier is needed.
+            constexpr int TS = 68;  // floats per staged row: 64 + 4, keeps 16-byte alignment
+            float *stg = reinterpret_cast<float *>(lds) + 2 * SM_T + wave * (32 * TS);
+            const int rr = lane >> 4, c4 = (lane & 15) * 4;
+#pragma clang loop unroll(disable)
+            for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const floatx16 a = i == 0 ? (j == 0 ? acc[0][0] : acc[0][1]) : (j == 0 ? acc[1][0] : acc[1][1]);
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        stg[(8 * (v >> 2) + 4 * (lane >> 5) + (v & 3)) * TS + j * 32 + (lane & 31)] = a[v];
+                }
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int it = 0; it < 8; ++it) {
+                    const int lr = wm + i * 32 + it * 4 + rr;
+                    const size_t at = (size_t)(r0 + lr) * I + c0 + wn + c4;
+                    const float4 gv = *reinterpret_cast<const float4 *>(stg + (it * 4 + rr) * TS + c4);
+                    const uint2 e = *reinterpret_cast<const uint2 *>(Eb + at);
+                    const float f = rowst[lr * 2] * g.inv_tau, rv = rowst[lr * 2 + 1];
+                    float4 o;
+                    o.x = __uint_as_float(e.x << 16) * f * (gv.x - rv);
+                    o.y = __uint_as_float(e.x & 0xffff0000u) * f * (gv.y - rv);
+                    o.z = __uint_as_float(e.y << 16) * f * (gv.z - rv);
+                    o.w = __uint_as_float(e.y & 0xffff0000u) * f * (gv.w - rv);
+                    *reinterpret_cast<float4 *>(dst + at) = o;
+                }
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+            }
+        } else {
         // rolled on purpose (see the fp32 kernel): gW = S (G - r) / tau with S = E / sum
 #pragma clang loop unroll(disable)
         for (int ij = 0; ij < 4; ++ij) {
@@ -682,11 +702,12 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
             for (int v = 0; v < 16; ++v) {
                 const int lr = wm + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
                 const int row = r0 + lr;
-                if (!EDGE || (row < R && col < C)) {
+                if (row < R && col < C) {
                     const float sv = softmap_bf16_f32(Eb[(size_t)row * I + col]) * rowst[lr * 2];
                     dst[(size_t)row * C + col] = sv * (a[v] - rowst[lr * 2 + 1]) * g.inv_tau;
                 }
             }
+        }
         }
     } else {
 #pragma unroll
@@ -762,19 +783,19 @@ static inline size_t softmap_part_bytes(int B, int I, int M, int precision) {
     return dl_align256((size_t)softmap_gx_chunks(B, I, M, precision) * B * I * sizeof(float));
 }
 static inline size_t softmap_rows_bytes(int R, int C) { return dl_align256((size_t)R * C * sizeof(unsigned short)); }
-static inline size_t softmap_pairs_bytes(int R, int C) { return dl_align256((size_t)((R + 1) / 2) * C * sizeof(unsigned)); }
+static inline size_t softmap_blocks_bytes(int R, int C) { return dl_align256((size_t)((R + 7) / 8) * C * sizeof(uint4)); }
 extern "C" size_t dl_soft_map_workspace_bytes(int B, int I, int M, int precision) {
     if (B <= 0 || I <= 0 || M <= 0) return 256;
     size_t bytes = softmap_r_bytes(M) + softmap_part_bytes(B, I, M, precision);
     if (precision == 1)
-        bytes += softmap_rows_bytes(B, I) + softmap_pairs_bytes(B, I) + softmap_rows_bytes(B, M) + softmap_pairs_bytes(B, M);
+        bytes += softmap_rows_bytes(B, I) + softmap_blocks_bytes(B, I) + softmap_rows_bytes(B, M) + softmap_blocks_bytes(B, M);
     return bytes;
 }
-static void softmap_pack(const float *src, const float *colscale, unsigned short *rows, unsigned *pairs, int R, int C,
+static void softmap_pack(const float *src, const float *colscale, unsigned short *rows, uint4 *blocks, int R, int C,
                          hipStream_t s) {
-    const long long total = (long long)((R + 1) / 2) * C;
+    const long long total = (long long)((R + 7) / 8) * C;
     DL_TIMED("softmap_pack_bf16", s,
-             (softmap_pack_bf16<<<dl_ceil_div(total, 256), 256, 0, s>>>(src, colscale, rows, pairs, R, C)));
+             (softmap_pack_bf16<<<dl_ceil_div(total, 256), 256, 0, s>>>(src, colscale, rows, blocks, R, C)));
 }
 
 extern "C" int dl_soft_map_fwd(const float *x, const float *W, float tau, float *m, float *stats, void *ws,
@@ -826,19 +847,19 @@ extern "C" int dl_soft_map_bwd(const float *x, const float *W, float tau, const 
     const unsigned short *Eb = precision == 1 ? (const unsigned short *)((const char *)stats + softmap_stats_bytes(M)) : nullptr;
     const float *rs = precision == 1 ? stats + M : nullptr;
     DL_TIMED("softmap_rowdot", s, (softmap_rowdot<<<dl_ceil_div(M, 32), 256, 0, s>>>(gm, m, r, B, M)));
-    unsigned *xp = nullptr, *gmp = nullptr;
+    uint4 *x8 = nullptr, *gm8 = nullptr;
     unsigned short *gms = nullptr;
     if (precision == 1) {
         char *w = (char *)ws + softmap_r_bytes(M) + softmap_part_bytes(B, I, M, precision) + softmap_rows_bytes(B, I);
-        xp = (unsigned *)w; w += softmap_pairs_bytes(B, I);
+        x8 = (uint4 *)w; w += softmap_blocks_bytes(B, I);
         gms = (unsigned short *)w; w += softmap_rows_bytes(B, M);
-        gmp = (unsigned *)w;
-        softmap_pack(x, nullptr, nullptr, xp, B, I, s);
-        softmap_pack(gm, rs, gms, gmp, B, M, s);
+        gm8 = (uint4 *)w;
+        softmap_pack(x, nullptr, nullptr, x8, B, I, s);
+        softmap_pack(gm, rs, gms, gm8, B, M, s);
     }
     const SoftmapArgs ggx{x, W, stats, gm, nullptr, scale, inv_tau, used_chunks > 1 ? part : gx, B, I, M,
                           dl_ceil_div(B, SM_T), col_tiles * used_chunks, col_tiles, red_chunk, Eb, rs,
-                          nullptr, xp, gms, gmp};
+                          nullptr, x8, gms, gm8};
     if (precision == 1) DL_TIMED("softmap_bf16_gx", s, (softmap_launch_bf16<1>(ggx, s)));
     else DL_TIMED("softmap_mfma_gx", s, (softmap_launch<1, SM_K>(ggx, s)));
     if (used_chunks > 1)
@@ -847,7 +868,7 @@ extern "C" int dl_soft_map_bwd(const float *x, const float *W, float tau, const 
                                                                                          used_chunks)));
     const SoftmapArgs ggw{x, W, stats, gm, r, scale, inv_tau, gW, B, I, M,
                           col_tiles, dl_ceil_div(M, SM_T), 1, dl_ceil_div(B, 8) * 8, Eb, rs,
-                          nullptr, xp, gms, gmp};
+                          nullptr, x8, gms, gm8};
     if (precision == 1) DL_TIMED("softmap_bf16_gw", s, (softmap_launch_bf16<2>(ggw, s)));
     else DL_TIMED("softmap_mfma_gw", s, (softmap_launch<2, SM_K>(ggw, s)));
     return dl_launch_status();
