@@ -574,7 +574,10 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
             if (p == 1) {
                 const unsigned ra[4] = {pe[0].x, pe[0].y, pe[0].z, pe[0].w};
                 const unsigned rb[4] = {pe[1].x, pe[1].y, pe[1].z, pe[1].w};
-                char *d = Bb + (e_q * 8) * SB_LD + (2 * e_o) * 2;
+                // rows 8 e_q + j of the stage: 8 rows apart is a multiple of 32 banks whatever the (16-byte
+                // aligned) row stride, so the 16-byte block a pair lands in is XOR-ed with (row / 8) % 4;
+                // the MFMA reads below undo it
+                char *d = Bb + (e_q * 8) * SB_LD + ((((e_o >> 2) ^ (e_q & 3)) << 2) | (e_o & 3)) * 4;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const unsigned a = ra[j >> 1], b = rb[j >> 1];
@@ -622,13 +625,17 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
     auto stage = [&](int s, auto do_commit, auto do_fetch) __attribute__((always_inline)) {
         const int cur = s & 1;
         const char *Ab = As + cur * STAGE + (wm + l32) * SB_LD + kh * 16;
-        const char *Bb = Bs + cur * STAGE + (wn + l32) * SB_LD + kh * 16;
+        const char *Bb = Bs + cur * STAGE + (wn + l32) * SB_LD;
+        // k-block kh + 2 kk of my B row; MODE 1 stores it swizzled by (row / 8) % 4 (rows wn + l32 and + 32
+        // share that value: wn and 32 are multiples of 32)
+        const int bsw = MODE == 1 ? ((l32 >> 3) & 3) : 0;
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
+            const int bo = ((kh + 2 * kk) ^ bsw) * 16;
             const bf16x8 a0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(Ab + kk * 32));
             const bf16x8 a1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(Ab + 32 * SB_LD + kk * 32));
-            const bf16x8 b0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(Bb + kk * 32));
-            const bf16x8 b1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(Bb + 32 * SB_LD + kk * 32));
+            const bf16x8 b0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(Bb + bo));
+            const bf16x8 b1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(Bb + 32 * SB_LD + bo));
             acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b0, acc[0][0], 0, 0, 0);
             acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b1, acc[0][1], 0, 0, 0);
             acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b0, acc[1][0], 0, 0, 0);
