@@ -520,28 +520,31 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
     };
 
     // ---- B operand
-    //  MODE 0: exp2((W[o, k] - max[o]) * scale) from the fp32 W, red-contiguous, four float4 pieces like
-    //          the A operand (the bf16 copy E would be read in half cache lines per stage here)
+    //  MODE 0: E[o, k] bf16, red-contiguous: 8 consecutive k of column (= row of W) b_o + 64 p, copied as
+    //          they are, like the A operand
     //  MODE 1: E[k, i] bf16, column-contiguous: rows 2 kp and 2 kp + 1, 8 columns each -> packed pairs
     //  MODE 2: x in blocks of 8 k, column-contiguous: as the A operand of that mode
     uint4 pe[2];
-    float4 pb[MODE == 0 ? 4 : 1];
-    float bmx[4];  // MODE 0: row maxima of the W rows this thread stages
     const int e_q = tid & 15, e_o = tid >> 4;
-    const int b_q = MODE == 0 ? (tid & 7) : (tid & 31), b_o = MODE == 0 ? (tid >> 3) : (tid >> 5);
+    const int b_q = tid & 3, b_o = tid >> 2;  // MODE 0
     auto eb = [&](int o, int i) -> unsigned {  // predicated scalar access, bits of E[o,i]
         return (o < M && i < I) ? (unsigned)Eb[(size_t)o * I + i] : 0u;
     };
-    if (MODE == 0) {
-#pragma unroll
-        for (int p = 0; p < 4; ++p) bmx[p] = g.stats[min(c0 + b_o + 32 * p, C - 1)];
-    }
     auto fetch_b = [&](int p, int k0) __attribute__((always_inline)) {
         if (MODE == 0) {
-            const int col = c0 + b_o + 32 * p, k = k0 + b_q * 4;
-            auto wv = [&](int kk) -> float { return (col < C && kk < k_end) ? g.W[(size_t)col * I + kk] : -INFINITY; };
-            if (EDGE) pb[p] = make_float4(wv(k), wv(k + 1), wv(k + 2), wv(k + 3));
-            else pb[p] = *reinterpret_cast<const float4 *>(g.W + (size_t)col * I + k);
+            const int col = c0 + b_o + 64 * p, k = k0 + b_q * 8;
+            if (EDGE) {
+                unsigned wv[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const unsigned lo = k + 2 * j < k_end ? eb(col, k + 2 * j) : 0u;
+                    const unsigned hi = k + 2 * j + 1 < k_end ? eb(col, k + 2 * j + 1) : 0u;
+                    wv[j] = lo | (hi << 16);
+                }
+                pe[p] = make_uint4(wv[0], wv[1], wv[2], wv[3]);
+            } else {
+                pe[p] = *reinterpret_cast<const uint4 *>(Eb + (size_t)col * I + k);
+            }
         } else if (MODE == 1) {
             const int k = k0 + 2 * e_o + p, col = c0 + e_q * 8;  // p = 0, 1: the two rows of the pair
             if (EDGE) {
@@ -565,11 +568,7 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
     auto commit_b = [&](int p, int buf) __attribute__((always_inline)) {
         char *Bb = Bs + buf * STAGE;
         if (MODE == 0) {
-            // exp2(-inf) = 0 covers the predicated path's padding
-            const float e0 = softmap_e(pb[p].x, bmx[p], g.scale), e1 = softmap_e(pb[p].y, bmx[p], g.scale);
-            const float e2 = softmap_e(pb[p].z, bmx[p], g.scale), e3 = softmap_e(pb[p].w, bmx[p], g.scale);
-            *reinterpret_cast<uint2 *>(Bb + (b_o + 32 * p) * SB_LD + b_q * 8) =
-                make_uint2(softmap_pk_bf16(e0, e1), softmap_pk_bf16(e2, e3));
+            *reinterpret_cast<uint4 *>(Bb + (b_o + 64 * p) * SB_LD + b_q * 16) = make_uint4(pe[p].x, pe[p].y, pe[p].z, pe[p].w);
         } else if (MODE == 1) {
             if (p == 1) {
                 const unsigned ra[4] = {pe[0].x, pe[0].y, pe[0].z, pe[0].w};
@@ -595,14 +594,12 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
     // (the two rows of a MODE 1 pair travel together in the second half: they are packed in one go)
     auto fetch_half = [&](int h, int k0) __attribute__((always_inline)) {
         fetch_a(h, k0);
-        if (MODE == 0) { fetch_b(2 * h, k0); fetch_b(2 * h + 1, k0); }
-        else if (MODE == 2) fetch_b(h, k0);
+        if (MODE != 1) fetch_b(h, k0);
         else if (h == 1) { fetch_b(0, k0); fetch_b(1, k0); }
     };
     auto commit_half = [&](int h, int buf) __attribute__((always_inline)) {
         commit_a(h, buf);
-        if (MODE == 0) { commit_b(2 * h, buf); commit_b(2 * h + 1, buf); }
-        else if (MODE == 2) commit_b(h, buf);
+        if (MODE != 1) commit_b(h, buf);
         else if (h == 1) commit_b(1, buf);
     };
 
