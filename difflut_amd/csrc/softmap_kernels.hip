@@ -312,7 +312,43 @@ __device__ __forceinline__ void softmap_tile(const SoftmapArgs &g, float *sm_lds
         }
         __syncthreads();
     }
-    if (MODE == 2) {
+    if (MODE == 2 && !EDGE) {
+        // Interior tiles: a wavefront's 64 x 64 block of G goes through LDS 32 rows at a time, so that a
+        // lane owns four consecutive columns of a row: 16-byte loads of W and 16-byte stores of gW in runs
+        // of 256 bytes per row (the accumulator layout itself gives 4-byte accesses in runs of 128).
+        // Each wavefront uses its own LDS region behind the row statistics; no block barrier is needed.
+        constexpr int TS = 68;  // floats per staged row: 64 + 4, keeps 16-byte alignment
+        float *stg = rowst + 4 * SM_T + (tid >> 6) * (32 * TS);
+        const int rr = lane >> 4, c4 = (lane & 15) * 4;
+#pragma clang loop unroll(disable)
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const floatx16 a = i == 0 ? (j == 0 ? acc[0][0] : acc[0][1]) : (j == 0 ? acc[1][0] : acc[1][1]);
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    stg[(8 * (v >> 2) + 4 * (lane >> 5) + (v & 3)) * TS + j * 32 + (lane & 31)] = a[v];
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int it = 0; it < 8; ++it) {
+                const int lr = wm + i * 32 + it * 4 + rr;
+                const size_t at = (size_t)(r0 + lr) * I + c0 + wn + c4;
+                const float4 gv = *reinterpret_cast<const float4 *>(stg + (it * 4 + rr) * TS + c4);
+                const float4 wv = *reinterpret_cast<const float4 *>(W + at);
+                const float mx = rowst[lr * 4], f = rowst[lr * 4 + 1] * g.inv_tau, rv = rowst[lr * 4 + 2];
+                float4 o;
+                o.x = softmap_e(wv.x, mx, scale) * f * (gv.x - rv);
+                o.y = softmap_e(wv.y, mx, scale) * f * (gv.y - rv);
+                o.z = softmap_e(wv.z, mx, scale) * f * (gv.z - rv);
+                o.w = softmap_e(wv.w, mx, scale) * f * (gv.w - rv);
+                *reinterpret_cast<float4 *>(dst + at) = o;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
+    } else if (MODE == 2) {
         // one 32x32 sub-tile per trip of a loop that is kept rolled: unrolled, the scheduler puts all
         // 64 W loads in flight at once and the registers that costs push the staging buffers of
         // the main loop into scratch memory
@@ -369,7 +405,10 @@ __global__ __launch_bounds__(256, 3) void softmap_mfma(SoftmapArgs g) {
 template <int MODE, int KC>
 static void softmap_launch(const SoftmapArgs &g, hipStream_t s) {
     constexpr int LDA = MODE != 2 ? SM_LD_T : SM_LD_V, LDB = MODE == 0 ? SM_LD_T : SM_LD_V;
-    constexpr int lds_bytes = 2 * KC * (LDA + LDB) * (int)sizeof(float);
+    // the gW epilogue re-uses the stages: row statistics (4 floats per tile row) + 32 x 68 floats per wavefront
+    constexpr int stage_bytes = 2 * KC * (LDA + LDB) * (int)sizeof(float);
+    constexpr int epi_bytes = MODE == 2 ? (4 * SM_T + 4 * 32 * 68) * (int)sizeof(float) : 0;
+    constexpr int lds_bytes = stage_bytes > epi_bytes ? stage_bytes : epi_bytes;
     if (lds_bytes > 65536)
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&softmap_mfma<MODE, KC>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
