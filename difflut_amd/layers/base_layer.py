@@ -214,7 +214,11 @@ class BaseLUTLayer(ABC, LUTLayerMixin, nn.Module):
         optimizer instead of `parameters()` (N small tensors) makes its step one kernel per tensor;
         both see the same memory.  Call after the layer is on its device: `.to()` re-creates the leaves."""
         banks = [bank.tensor() for bank in self._banks.values()]
-        own = [p for name, p in self.named_parameters() if not name.startswith("nodes.")]
+        # the layer's own parameters: everything outside `nodes` (not a walk over the N node modules)
+        own = [p for p in self._parameters.values() if p is not None]
+        for name, child in self.named_children():
+            if name != "nodes":
+                own.extend(child.parameters())
         return banks + own
 
     def _run_nodes(self, x, plan):
