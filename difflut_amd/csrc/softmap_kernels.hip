@@ -423,12 +423,19 @@ static void softmap_launch(const SoftmapArgs &g, hipStream_t s) {
 // forward output, to the gm operand of the gx product and in the gW epilogue.  x and gm are rounded
 // to bf16 (nearest even) once per call by a packing pass (softmap_pack_bf16), into the layout the
 // staging code copies to LDS unchanged.  A lane feeds the MFMA eight consecutive k of one row, so LDS
-// holds a stage row-major, As[row][32 k] with 16 bytes of padding per row.
+// holds a stage row-major, As[row][32 k], unpadded and XOR-swizzled in units of 16 bytes.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
 #define SB_K 32   // reduction depth per stage
-#define SB_LD 80  // bytes per LDS row
+#define SB_LD 64  // bytes per LDS row: 32 k, no padding
+// Rows are unpadded, so two consecutive rows fill the 32 banks exactly; the 16-byte block (8 k) of a row
+// sits at position block ^ softmap_swz(row).  Eight consecutive rows then put a given logical block on
+// eight different bank groups: the 16-byte stores of a stage (consecutive lanes = the blocks of two
+// consecutive rows) and the 16-byte MFMA operand reads (consecutive lanes = consecutive rows, one logical
+// block) are both free of bank conflicts.  The second term separates rows 16 apart for the one stage
+// that is written transposed, 4 bytes at a time.
+__device__ __forceinline__ int softmap_swz(int row) { return ((row >> 1) ^ (row >> 4)) & 3; }
 
 __device__ __forceinline__ unsigned softmap_pk_bf16(float lo, float hi) {
     const floatx2 v = {lo, hi};
@@ -555,7 +562,8 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
     auto commit_a = [&](int p, int buf) __attribute__((always_inline)) {
         char *Ab = As + buf * STAGE;
         const uint4 v = make_uint4(pa[p].x, pa[p].y, pa[p].z, pa[p].w);
-        *reinterpret_cast<uint4 *>(Ab + (a_o + 64 * p) * SB_LD + a_q * 16) = v;  // both forms: 8 k of one row
+        const int row = a_o + 64 * p;  // both forms: 8 k of one row
+        *reinterpret_cast<uint4 *>(Ab + row * SB_LD + ((a_q ^ softmap_swz(row)) << 4)) = v;
     };
 
     // ---- B operand
@@ -607,25 +615,29 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
     auto commit_b = [&](int p, int buf) __attribute__((always_inline)) {
         char *Bb = Bs + buf * STAGE;
         if (MODE == 0) {
-            *reinterpret_cast<uint4 *>(Bb + (b_o + 64 * p) * SB_LD + b_q * 16) = make_uint4(pe[p].x, pe[p].y, pe[p].z, pe[p].w);
+            const int row = b_o + 64 * p;
+            *reinterpret_cast<uint4 *>(Bb + row * SB_LD + ((b_q ^ softmap_swz(row)) << 4)) = make_uint4(pe[p].x, pe[p].y, pe[p].z, pe[p].w);
         } else if (MODE == 1) {
             if (p == 1) {
                 const unsigned ra[4] = {pe[0].x, pe[0].y, pe[0].z, pe[0].w};
                 const unsigned rb[4] = {pe[1].x, pe[1].y, pe[1].z, pe[1].w};
-                // rows 8 e_q + j of the stage: 8 rows apart is a multiple of 32 banks whatever the (16-byte
-                // aligned) row stride, so the 16-byte block a pair lands in is XOR-ed with (row / 8) % 4;
-                // the MFMA reads below undo it
-                char *d = Bb + (e_q * 8) * SB_LD + ((((e_o >> 2) ^ (e_q & 3)) << 2) | (e_o & 3)) * 4;
+                // The pair (k, k+1) = dword e_o of rows 8 e_q + j, j = 0..7.  Lanes that differ in e_q are 8
+                // rows apart, i.e. on the same banks but for the swizzle; to use both halves of the banks in
+                // every store, lanes with odd e_q walk their columns in the order j ^ 1.
+                const int odd = e_q & 1;
+                const unsigned sel_lo = 0x05040100u, sel_hi = 0x07060302u;  // low / high halves of the two rows
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const unsigned a = ra[j >> 1], b = rb[j >> 1];
-                    // low halves (even column) or high halves (odd column) of the two rows -> (k, k+1)
-                    const unsigned v = (j & 1) ? __builtin_amdgcn_perm(b, a, 0x07060302u) : __builtin_amdgcn_perm(b, a, 0x05040100u);
-                    *reinterpret_cast<unsigned *>(d + j * SB_LD) = v;
+                for (int st = 0; st < 8; ++st) {
+                    const int j = st ^ odd;  // j >> 1 == st >> 1: same source registers for every lane
+                    const unsigned a = ra[st >> 1], b = rb[st >> 1];
+                    const unsigned v = __builtin_amdgcn_perm(b, a, (j & 1) ? sel_hi : sel_lo);
+                    const int row = e_q * 8 + j;
+                    *reinterpret_cast<unsigned *>(Bb + row * SB_LD + ((((e_o >> 2) ^ softmap_swz(row)) << 2) | (e_o & 3)) * 4) = v;
                 }
             }
         } else {
-            *reinterpret_cast<uint4 *>(Bb + ((tid & 63) + 64 * p) * SB_LD + (tid >> 6) * 16) =
+            const int row = (tid & 63) + 64 * p;
+            *reinterpret_cast<uint4 *>(Bb + row * SB_LD + (((tid >> 6) ^ softmap_swz(row)) << 4)) =
                 make_uint4(pe[p].x, pe[p].y, pe[p].z, pe[p].w);
         }
     };
@@ -660,18 +672,17 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
     const int kh = lane >> 5, l32 = lane & 31;
     auto stage = [&](int s, auto do_commit, auto do_fetch) __attribute__((always_inline)) {
         const int cur = s & 1;
-        const char *Ab = As + cur * STAGE + (wm + l32) * SB_LD + kh * 16;
+        const char *Ab = As + cur * STAGE + (wm + l32) * SB_LD;
         const char *Bb = Bs + cur * STAGE + (wn + l32) * SB_LD;
-        // k-block kh + 2 kk of my B row; MODE 1 stores it swizzled by (row / 8) % 4 (rows wn + l32 and + 32
-        // share that value: wn and 32 are multiples of 32)
-        const int bsw = MODE == 1 ? ((l32 >> 3) & 3) : 0;
+        // k-block kh + 2 kk of my rows, at its swizzled position; rows 32 apart differ in the swizzle by 2
+        const int swa = softmap_swz(wm + l32), swb = softmap_swz(wn + l32);
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
-            const int bo = ((kh + 2 * kk) ^ bsw) * 16;
-            const bf16x8 a0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(Ab + kk * 32));
-            const bf16x8 a1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(Ab + 32 * SB_LD + kk * 32));
-            const bf16x8 b0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(Bb + bo));
-            const bf16x8 b1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(Bb + 32 * SB_LD + bo));
+            const int blk = kh + 2 * kk;
+            const bf16x8 a0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(Ab + ((blk ^ swa) << 4)));
+            const bf16x8 a1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(Ab + 32 * SB_LD + ((blk ^ swa ^ 2) << 4)));
+            const bf16x8 b0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(Bb + ((blk ^ swb) << 4)));
+            const bf16x8 b1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(Bb + 32 * SB_LD + ((blk ^ swb ^ 2) << 4)));
             acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b0, acc[0][0], 0, 0, 0);
             acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b1, acc[0][1], 0, 0, 0);
             acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b0, acc[1][0], 0, 0, 0);
@@ -770,7 +781,7 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
 
 template <int MODE>
 __global__ __launch_bounds__(256, 3) void softmap_mfma_bf16(SoftmapArgs g) {
-    __shared__ __align__(16) char lds[4 * SM_T * SB_LD];
+    __shared__ __align__(16) char lds[MODE == 2 ? (2 * SM_T + 4 * 32 * 68) * 4 : 4 * SM_T * SB_LD];  // gW: its epilogue's staging
     int inner, outer;
     if (!dl_xcd_map(g.inner_count, g.outer_count, inner, outer)) return;
     const int rt = MODE == 2 ? outer : inner;
