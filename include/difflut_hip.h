@@ -202,6 +202,8 @@ int dl_prob_layer_eval(const float *x, const int32_t *idx32, const float *raw_w,
 /* size of `stats`: what the forward keeps for the backward (row maximum and 1/sum; with
  * precision 1 also the bf16 softmax numerators, M*I*2 bytes) */
 size_t dl_soft_map_saved_bytes(int B, int I, int M, int precision);
+/* scratch of either direction (one size for both): the backward's r [M] and partial gx products and,
+ * with precision 1, the bf16 copies of x and gm.  The forward only needs it with precision 1. */
 size_t dl_soft_map_workspace_bytes(int B, int I, int M, int precision);
 int dl_soft_map_fwd(const float *x, const float *W, float tau, float *m, float *stats,
                     void *ws, size_t ws_bytes, int B, int I, int M, int precision, void *stream);
