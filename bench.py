@@ -196,6 +196,23 @@ def run_conv(args):
     print(json.dumps(out_d))
 
 
+def maybe_graph(step, args):
+    """With --graph: the step's launches captured once (after warm-up, on a side stream as torch requires) and
+    replayed; the library never allocates, synchronises or uses memset nodes, so a step is capturable as it is."""
+    if not getattr(args, "graph", False):
+        return step
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    return graph.replay
+
+
 def run_secondary(args):
     """Probabilistic layer (k=4, 1024 x 4096 -> 4096 nodes), DWN-stable and hybrid layers at the headline shape, and
     soft connectivity (512 x 3136 -> 48000 rows), all through the C ABI."""
@@ -205,7 +222,6 @@ def run_secondary(args):
 
     lib = nat.lib()
     dev = torch.device("cuda:0")
-    stream = torch.cuda.current_stream().cuda_stream
     B, I, N, k, O = WORKLOADS[args.workload]
     torch.manual_seed(0)
     if args.workload.startswith("prob"):
@@ -220,12 +236,12 @@ def run_secondary(args):
 
         def step():
             nat.check(lib.dl_prob_layer_fwd(x.data_ptr(), plan.idx32.data_ptr(), raw.data_ptr(), 1.0, y.data_ptr(),
-                                            saved.data_ptr(), saved.numel(), *dims, stream))
+                                            saved.data_ptr(), saved.numel(), *dims, nat.stream()))
             nat.check(lib.dl_prob_layer_bwd(x.data_ptr(), saved.data_ptr(), plan.idx32.data_ptr(), plan.inv_ptr.data_ptr(),
                                             plan.inv_pos.data_ptr(), raw.data_ptr(), 1.0, gy.data_ptr(), gx.data_ptr(),
-                                            graw.data_ptr(), ws.data_ptr(), ws.numel(), *dims, stream))
+                                            graw.data_ptr(), ws.data_ptr(), ws.numel(), *dims, nat.stream()))
 
-        ms = time_steps(step, args.steps, args.warmup)
+        ms = time_steps(maybe_graph(step, args), args.steps, args.warmup)
         nbytes = 5 * B * I * 4 + 3 * N * (1 << k) * O * 4 + 2 * N * k * 2  # x, y, gy, x again, gx; tables r, r, grad
         flops = 320 * B * N
         out = {"metric": "LUT-node evals/sec fwd+bwd (Probabilistic k=4, B=1024, 4096 nodes)", "value": B * N / (ms * 1e-3),
@@ -250,21 +266,21 @@ def run_secondary(args):
                              lib.dl_hybrid_bwd_workspace_bytes(*dims)), dtype=torch.uint8, device=dev)
 
         def step():
-            nat.check(lib.dl_table_sigmoid_fwd(raw.data_ptr(), luts.data_ptr(), count, stream))
+            nat.check(lib.dl_table_sigmoid_fwd(raw.data_ptr(), luts.data_ptr(), count, nat.stream()))
             nat.check(lib.dl_dwn_layer_fwd(x.data_ptr(), plan.idx32.data_ptr(), luts.data_ptr(), y.data_ptr(),
-                                           saved.data_ptr(), ws.data_ptr(), ws.numel(), *dims, stream))
+                                           saved.data_ptr(), ws.data_ptr(), ws.numel(), *dims, nat.stream()))
             if stable:
                 nat.check(lib.dl_dwn_stable_layer_bwd(None, saved.data_ptr(), plan.idx32.data_ptr(), plan.inv_ptr.data_ptr(),
                                                       plan.inv_pos.data_ptr(), luts.data_ptr(), gy.data_ptr(),
                                                       scale.data_ptr(), gx.data_ptr(), gl.data_ptr(), ws.data_ptr(),
-                                                      ws.numel(), *dims, stream))
+                                                      ws.numel(), *dims, nat.stream()))
             else:
                 nat.check(lib.dl_hybrid_layer_bwd(x.data_ptr(), plan.idx32.data_ptr(), plan.inv_ptr.data_ptr(),
                                                   plan.inv_pos.data_ptr(), luts.data_ptr(), gy.data_ptr(), gx.data_ptr(),
-                                                  gl.data_ptr(), ws.data_ptr(), ws.numel(), *dims, stream))
-            nat.check(lib.dl_table_sigmoid_bwd(gl.data_ptr(), luts.data_ptr(), graw.data_ptr(), count, stream))
+                                                  gl.data_ptr(), ws.data_ptr(), ws.numel(), *dims, nat.stream()))
+            nat.check(lib.dl_table_sigmoid_bwd(gl.data_ptr(), luts.data_ptr(), graw.data_ptr(), count, nat.stream()))
 
-        ms = time_steps(step, args.steps, args.warmup)
+        ms = time_steps(maybe_graph(step, args), args.steps, args.warmup)
         fwd_b, bwd_b, _ = algorithmic_bytes(B, I, N, k, O)  # same tensors cross HBM as for the DWN node
         nbytes = fwd_b + bwd_b
         name = "DWN-stable" if stable else "hybrid"
@@ -285,12 +301,12 @@ def run_secondary(args):
 
         def step():
             nat.check(lib.dl_soft_map_fwd(x.data_ptr(), W.data_ptr(), 1.0, m.data_ptr(), stats.data_ptr(), ws.data_ptr(),
-                                          ws.numel(), B, I, M, precision, stream))
+                                          ws.numel(), B, I, M, precision, nat.stream()))
             nat.check(lib.dl_soft_map_bwd(x.data_ptr(), W.data_ptr(), 1.0, m.data_ptr(), stats.data_ptr(), gm.data_ptr(),
                                           gx.data_ptr(), gW.data_ptr(), ws.data_ptr(), ws.numel(), B, I, M, precision,
-                                          stream))
+                                          nat.stream()))
 
-        ms = time_steps(step, args.steps, args.warmup)
+        ms = time_steps(maybe_graph(step, args), args.steps, args.warmup)
         flops = 3 * 2.0 * B * I * M
         peak = 157.3 if precision == 0 else 2500.0
         out = {"metric": "soft-connectivity contraction fwd+bwd (x[512,3136] . softmax(W[48000,3136])^T)",
@@ -299,7 +315,8 @@ def run_secondary(args):
                "roofline_step": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
                                  "frac": flops / (ms * 1e-3) / 1e12 / peak, "algorithmic_flops_per_step": flops}}
     out.update({"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
-                "vs_baseline": None, "data": "synthetic", "config": {"workload": args.workload},
+                "vs_baseline": None, "data": "synthetic",
+                "config": {"workload": args.workload, "launch": "hip graph replay" if args.graph else "direct"},
                 "kernel_ms": kernel_times(step, min(args.steps, 10))})
     print(json.dumps(out))
 
@@ -314,6 +331,8 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=4096, help="batch rows of the workload the CPU baseline runs")
     ap.add_argument("--precision", type=int, default=0, help="soft-connectivity workload: 0 fp32, 1 bf16 operands")
     ap.add_argument("--layer-by-layer", action="store_true", help="stack workload: call the layers one by one")
+    ap.add_argument("--graph", action="store_true",
+                    help="C-ABI workloads other than the default: replay the step from a captured HIP graph")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no collective); run with --gpus 1",
