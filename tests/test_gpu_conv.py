@@ -250,3 +250,31 @@ def test_conv_layer_against_reference_vectors(golden_next):
     layer.eval()
     with torch.no_grad():
         assert np.array_equal(layer(torch.tensor(g["conv_eval_x"], device=DEV)).cpu().numpy(), g["conv_eval_y"])
+
+
+@pytest.mark.parametrize("kind", ["dwn", "hybrid"])
+def test_conv_layer_with_grouped_connections_against_tree_loops(kind):
+    """Grouped first-layer connections (every node inside one channel) through the fused levels."""
+    torch.manual_seed(13)
+    B, in_ch, H, W, out_ch = 3, 4, 7, 7, 5
+    layer = _build(kind, 2, in_ch, out_ch, 3, 1, 0, 2, grouped=True, seed=7)
+    layer.train()
+    pname, fwd, bwd = _oracle_fns(kind)
+    table = layer.first_layer_chunks[0]._mapping_indices.cpu().long()
+    assert torch.all((table // 9) == (table[:, :1] // 9))
+    rng = np.random.default_rng(14)
+    x = (0.02 + 0.96 * rng.random((B, in_ch, H, W))).astype(np.float32)
+    xt = torch.tensor(x, device=DEV, requires_grad=True)
+    y = layer(xt)
+    chunks, trees = _tables(layer, pname)
+    patches = orc.conv_unfold(x, (3, 3), (1, 1), (0, 0))
+    out, acts = orc.conv_trees_forward(patches, chunks, trees, layer.hidden_layers[0], fwd)
+    want = out.reshape(B, 25, out_ch).transpose(0, 2, 1).reshape(B, out_ch, 5, 5)
+    np.testing.assert_allclose(y.detach().cpu().numpy(), want, rtol=1e-6, atol=1e-7)
+    gy = rng.standard_normal(want.shape).astype(np.float32)
+    y.backward(torch.tensor(gy, device=DEV))
+    gout = gy.reshape(B, out_ch, 25).transpose(0, 2, 1).reshape(-1, out_ch)
+    gp, gch, _ = orc.conv_trees_backward(patches, chunks, trees, layer.hidden_layers[0], acts, gout, bwd)
+    np.testing.assert_allclose(xt.grad.cpu().numpy(), orc.conv_fold(gp, x.shape, (3, 3), (1, 1), (0, 0)), rtol=1e-5, atol=5e-6)
+    got = np.stack([getattr(node, pname).grad.cpu().numpy() for node in layer.first_layer_chunks[2].nodes])
+    np.testing.assert_allclose(got, gch[2], rtol=1e-5, atol=5e-6)
