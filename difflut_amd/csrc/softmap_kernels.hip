@@ -100,14 +100,35 @@ __global__ __launch_bounds__(256) void softmap_rowdot(const float *__restrict__ 
     }
 }
 
-// out[e] = sum over chunks of part[chunk][e], fixed order
+// out[e] = sum over chunks of part[chunk][e], fixed order; VEC = 4 when total is a multiple of 4
+template <int VEC>
 __global__ __launch_bounds__(256) void softmap_reduce_chunks(const float *__restrict__ part, float *__restrict__ out,
                                                               long long total, int chunks) {
-    const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long e = ((long long)blockIdx.x * 256 + threadIdx.x) * VEC;
     if (e >= total) return;
-    float acc = 0.0f;
-    for (int c = 0; c < chunks; ++c) acc += part[(size_t)c * total + e];
-    out[e] = acc;
+    if (VEC == 4) {
+        float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        int c = 0;
+        for (; c + 4 <= chunks; c += 4) {  // four independent loads in flight, added in chunk order
+            const float4 p0 = *reinterpret_cast<const float4 *>(part + (size_t)c * total + e);
+            const float4 p1 = *reinterpret_cast<const float4 *>(part + (size_t)(c + 1) * total + e);
+            const float4 p2 = *reinterpret_cast<const float4 *>(part + (size_t)(c + 2) * total + e);
+            const float4 p3 = *reinterpret_cast<const float4 *>(part + (size_t)(c + 3) * total + e);
+            acc.x += p0.x; acc.y += p0.y; acc.z += p0.z; acc.w += p0.w;
+            acc.x += p1.x; acc.y += p1.y; acc.z += p1.z; acc.w += p1.w;
+            acc.x += p2.x; acc.y += p2.y; acc.z += p2.z; acc.w += p2.w;
+            acc.x += p3.x; acc.y += p3.y; acc.z += p3.z; acc.w += p3.w;
+        }
+        for (; c < chunks; ++c) {
+            const float4 p = *reinterpret_cast<const float4 *>(part + (size_t)c * total + e);
+            acc.x += p.x; acc.y += p.y; acc.z += p.z; acc.w += p.w;
+        }
+        *reinterpret_cast<float4 *>(out + e) = acc;
+    } else {
+        float acc = 0.0f;
+        for (int c = 0; c < chunks; ++c) acc += part[(size_t)c * total + e];
+        out[e] = acc;
+    }
 }
 
 struct SoftmapArgs {
@@ -916,10 +937,15 @@ extern "C" int dl_soft_map_bwd(const float *x, const float *W, float tau, const 
                           nullptr, x8, gms, gm8};
     if (precision == 1) DL_TIMED("softmap_bf16_gx", s, (softmap_launch_bf16<1>(ggx, s)));
     else DL_TIMED("softmap_mfma_gx", s, (softmap_launch<1, SM_K>(ggx, s)));
-    if (used_chunks > 1)
-        DL_TIMED("softmap_reduce_chunks", s,
-                 (softmap_reduce_chunks<<<dl_ceil_div((long long)B * I, 256), 256, 0, s>>>(part, gx, (long long)B * I,
-                                                                                         used_chunks)));
+    if (used_chunks > 1) {
+        const long long total = (long long)B * I;
+        if (total % 4 == 0 && ((uintptr_t)gx & 15) == 0)
+            DL_TIMED("softmap_reduce_chunks", s,
+                     (softmap_reduce_chunks<4><<<dl_ceil_div(total / 4, 256), 256, 0, s>>>(part, gx, total, used_chunks)));
+        else
+            DL_TIMED("softmap_reduce_chunks", s,
+                     (softmap_reduce_chunks<1><<<dl_ceil_div(total, 256), 256, 0, s>>>(part, gx, total, used_chunks)));
+    }
     const SoftmapArgs ggw{x, W, stats, gm, r, scale, inv_tau, gW, B, I, M,
                           col_tiles, dl_ceil_div(M, SM_T), 1, dl_ceil_div(B, 8) * 8, Eb, rs,
                           nullptr, x8, gms, gm8};
