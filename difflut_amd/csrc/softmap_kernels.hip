@@ -503,6 +503,52 @@ __global__ __launch_bounds__(256) void softmap_rowstats_bf16(const float *__rest
     if (lane == 0) { mxs[row] = mx; rss[row] = 1.0f / sum; }
 }
 
+// Row statistics with the row held in registers (rows of up to 256 * NV floats, I a multiple of 4): W is
+// read once - the two-sweep kernels above fetch it twice, the second sweep does not stay in cache when
+// every wavefront of the chip streams its own 12 KB row.  One wavefront per row; BF16 also writes the bf16
+// numerators and sums the rounded values, exactly as softmap_rowstats_bf16 does.
+template <int NV, bool BF16>
+__global__ __launch_bounds__(256) void softmap_rowstats_regs(const float *__restrict__ W, float scale, float *__restrict__ out_a,
+                                                              float *__restrict__ out_b, unsigned short *__restrict__ Eb,
+                                                              int M, int I) {
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= M) return;
+    const float4 *w4 = reinterpret_cast<const float4 *>(W + (size_t)row * I);
+    const int n4 = I >> 2;
+    float4 v[NV];
+#pragma unroll
+    for (int q = 0; q < NV; ++q) {
+        const int i = lane + 64 * q;
+        v[q] = i < n4 ? w4[i] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int q = 0; q < NV; ++q) mx = fmaxf(mx, fmaxf(fmaxf(v[q].x, v[q].y), fmaxf(v[q].z, v[q].w)));
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+    float sum = 0.0f;
+#pragma unroll
+    for (int q = 0; q < NV; ++q) {
+        const int i = lane + 64 * q;
+        // exp2(-inf) = 0: the padding adds nothing
+        const float e0 = softmap_e(v[q].x, mx, scale), e1 = softmap_e(v[q].y, mx, scale);
+        const float e2 = softmap_e(v[q].z, mx, scale), e3 = softmap_e(v[q].w, mx, scale);
+        if (BF16) {
+            const unsigned lo = softmap_pk_bf16(e0, e1), hi = softmap_pk_bf16(e2, e3);
+            sum += (__uint_as_float(lo << 16) + __uint_as_float(lo & 0xffff0000u)) +
+                   (__uint_as_float(hi << 16) + __uint_as_float(hi & 0xffff0000u));
+            if (i < n4) *reinterpret_cast<uint2 *>(Eb + (size_t)row * I + 4 * i) = make_uint2(lo, hi);
+        } else {
+            sum += (e0 + e1) + (e2 + e3);
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+    if (lane == 0) {
+        if (BF16) { out_a[row] = mx; out_b[row] = 1.0f / sum; }
+        else { out_a[2 * row] = mx; out_a[2 * row + 1] = 1.0f / sum; }
+    }
+}
+
 // Operands of the bf16 products, rounded once (nearest even) into the layout the staging code copies:
 // row-major bf16 for an operand that is contiguous along the reduction; for one that is contiguous
 // along the rows / columns of the product (the reduction runs over its rows) blocks of 8 consecutive
@@ -873,6 +919,20 @@ static void softmap_pack(const float *src, const float *colscale, unsigned short
              (softmap_pack_bf16<<<dl_ceil_div(total, 256), 256, 0, s>>>(src, colscale, rows, blocks, R, C)));
 }
 
+// rows that fit a wavefront's registers are read once; longer or unaligned rows take the two-sweep kernels
+template <bool BF16>
+static void softmap_stats_launch(const float *W, float scale, float *a, float *b, unsigned short *Eb, int M, int I,
+                                 hipStream_t s) {
+    const int grid = dl_ceil_div(M, 4), n4 = I >> 2;
+    const bool regs = I % 4 == 0 && n4 <= 1024 && ((uintptr_t)W & 15) == 0;
+    const char *name = BF16 ? "softmap_rowstats_bf16" : "softmap_rowstats";
+    if (regs && n4 <= 256) DL_TIMED(name, s, (softmap_rowstats_regs<4, BF16><<<grid, 256, 0, s>>>(W, scale, a, b, Eb, M, I)));
+    else if (regs && n4 <= 512) DL_TIMED(name, s, (softmap_rowstats_regs<8, BF16><<<grid, 256, 0, s>>>(W, scale, a, b, Eb, M, I)));
+    else if (regs) DL_TIMED(name, s, (softmap_rowstats_regs<16, BF16><<<grid, 256, 0, s>>>(W, scale, a, b, Eb, M, I)));
+    else if (BF16) DL_TIMED(name, s, (softmap_rowstats_bf16<<<grid, 256, 0, s>>>(W, scale, a, b, Eb, M, I)));
+    else DL_TIMED(name, s, (softmap_rowstats<<<grid, 256, 0, s>>>(W, scale, a, M, I)));
+}
+
 extern "C" int dl_soft_map_fwd(const float *x, const float *W, float tau, float *m, float *stats, void *ws,
                                size_t ws_bytes, int B, int I, int M, int precision, void *stream) {
     if (!x || !W || !m || !stats) return DL_ERR_NULL;
@@ -888,8 +948,7 @@ extern "C" int dl_soft_map_fwd(const float *x, const float *W, float tau, float 
                   nullptr, nullptr, nullptr, nullptr};
     if (precision == 1) {
         unsigned short *Eb = (unsigned short *)((char *)stats + softmap_stats_bytes(M));
-        DL_TIMED("softmap_rowstats_bf16", s,
-                 (softmap_rowstats_bf16<<<dl_ceil_div(M, 4), 256, 0, s>>>(W, scale, stats, stats + M, Eb, M, I)));
+        softmap_stats_launch<true>(W, scale, stats, stats + M, Eb, M, I, s);
         unsigned short *xb = (unsigned short *)((char *)ws + softmap_r_bytes(M) + softmap_part_bytes(B, I, M, precision));
         softmap_pack(x, nullptr, xb, nullptr, B, I, s);
         g.xb = xb;
@@ -897,7 +956,7 @@ extern "C" int dl_soft_map_fwd(const float *x, const float *W, float tau, float 
         g.rs = stats + M;
         DL_TIMED("softmap_bf16_fwd", s, (softmap_launch_bf16<0>(g, s)));
     } else {
-        DL_TIMED("softmap_rowstats", s, (softmap_rowstats<<<dl_ceil_div(M, 4), 256, 0, s>>>(W, scale, stats, M, I)));
+        softmap_stats_launch<false>(W, scale, stats, nullptr, nullptr, M, I, s);
         DL_TIMED("softmap_mfma_fwd", s, (softmap_launch<0, SM_K>(g, s)));
     }
     return dl_launch_status();
