@@ -584,7 +584,7 @@ __device__ __forceinline__ void softmap_tile_bf16(const SoftmapArgs &g, char *ld
     constexpr int STAGE = SM_T * SB_LD;  // bytes of one operand stage
     char *const As = lds;                // [2][128][SB_LD]
     char *const Bs = lds + 2 * STAGE;
-    const float *__restrict__ x = g.x, *__restrict__ gm = g.gm, *__restrict__ rs = g.rs;
+    const float *__restrict__ rs = g.rs;
     const unsigned short *__restrict__ Eb = g.Eb;
     const int B = g.B, I = g.I, M = g.M;
     const int R = MODE == 2 ? M : B, C = MODE == 0 ? M : I;
