@@ -521,7 +521,8 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT,
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int r = 0; r < DWN_WI; ++r)
-            if (wbeg + r < iend) gx[((size_t)t * I + i0 + wbeg + r) * 64 + lane] = tile[wbeg + r][lane];
+            if (wbeg + r < iend)  // streamed past the L2, which holds the rows the gather re-reads
+                __builtin_nontemporal_store(tile[wbeg + r][lane], &gx[((size_t)t * I + i0 + wbeg + r) * 64 + lane]);
         return;
     }
     __syncthreads();
