@@ -401,8 +401,8 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
 // bwd_gx: one block per (64-input slab, 64-row batch tile), 256 threads, lane = batch row.  A wavefront
 // owns 16 consecutive inputs, i.e. one contiguous run of CSR entries.  The run is read 64 entries
 // at a time into registers (one entry per lane: node, slot, local input), then replayed 8 entries
-// per step with wave-uniform addressing; the 8 x 3 vector loads of the next step are requested
-// before the current step is evaluated.  The entries of one input are consecutive, so its sum is
+// per step with wave-uniform addressing: the 8 x 3 vector loads of a step are requested together,
+// then evaluated.  The entries of one input are consecutive, so its sum is
 // kept in a register and written to the LDS tile once, in CSR order (reproducible sums).
 #define DWN_IS 64
 #define DWN_WI (DWN_IS / 4)  // inputs per wavefront
@@ -505,13 +505,12 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT,
                 acc += term;
             }
         };
-        Group A, Bq;
-        request(0, A);
-        for (int s0 = 0; s0 < cnt; s0 += 2 * DWN_EG) {
-            if (s0 + DWN_EG < cnt) request(s0 + DWN_EG, Bq);
-            evaluate(A);
-            if (s0 + 2 * DWN_EG < cnt) request(s0 + 2 * DWN_EG, A);
-            if (s0 + DWN_EG < cnt) evaluate(Bq);
+        // one group in flight per wavefront: the other resident wavefronts cover its latency, and a
+        // second group in registers measured slower (fewer wavefronts fit)
+        Group G;
+        for (int s0 = 0; s0 < cnt; s0 += DWN_EG) {
+            request(s0, G);
+            evaluate(G);
         }
     }
     if (cur >= 0) tile[wbeg + cur][lane] = acc;
