@@ -118,7 +118,7 @@ def run_stack(args):
     opt = torch.optim.Adam(params, lr=1e-3)
     from difflut_amd.layers import DWNStack
     # same layers; thermometer code and activations as bit-planes, tile-major gradients between layers
-    stack = DWNStack(layers, encoder=enc).train()
+    stack = DWNStack(layers, encoder=enc, head=head).train()
 
     def step():
         opt.zero_grad(set_to_none=True)
@@ -126,9 +126,10 @@ def run_stack(args):
             h = enc.encode(x)
             for layer in layers:
                 h = layer(h)
+            logits = head(h)
         else:
-            h = stack(x)
-        loss = torch.nn.functional.cross_entropy(head(h), labels)
+            logits = stack(x)  # the last layer sums per group itself
+        loss = torch.nn.functional.cross_entropy(logits, labels)
         loss.backward()
         opt.step()
 

@@ -101,13 +101,20 @@ __global__ __launch_bounds__(256) void dwn_pack_planes(const float *__restrict__
 #define DWN_WC (DWN_TC / DWN_FW)      // columns per wavefront
 #define DWN_CG 4                      // columns per group
 // CHAIN: the variant for chained layers, which can also (or only) emit the columns as bit-planes.
-template <int K, bool O1, bool CHAIN = false>
+// GSUM: the variant under a GroupSum head.  Instead of y it writes, per row, the sums of the tile's columns
+// that fall into each group the tile touches (at most DWN_GS_SLOTS of them):
+// partial[(column tile * slots + slot)][row], slot = group - first group of the tile; dwn_group_finish
+// adds the tiles of a group in a fixed order.
+#define DWN_GS_SLOTS 4
+template <int K, bool O1, bool CHAIN = false, bool GSUM = false>
 __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restrict__ planes, const int *__restrict__ idx32,
                                                                const float *__restrict__ luts, float *__restrict__ y,
                                                                uint8_t *__restrict__ addrT, u64 *__restrict__ planes_out,
-                                                               int B, int I, int N, int O, int BT) {
+                                                               int B, int I, int N, int O, int BT, int gsize = 1,
+                                                               int slots = 1) {
     __shared__ float tile[DWN_TC][65];  // [column][row]
     __shared__ u64 plane_tile[CHAIN ? DWN_TC : 1];  // thresholded outputs of the tile's columns, one bit per row
+    __shared__ float gpart[GSUM ? DWN_FW : 1][GSUM ? DWN_GS_SLOTS : 1][64];  // [wavefront][slot][row]
     constexpr int L = 1 << K;
     constexpr int NIDX = (DWN_WC * K + 63) / 64;  // index registers per lane
     const int NO = N * O;
@@ -177,6 +184,30 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
         const int rows = min(64, B - t * 64);  // rows past B read as 0, like the planes packed from x
         const u64 valid = rows == 64 ? ~0ull : ((1ull << rows) - 1ull);
         planes_out[(size_t)t * NO + c0 + threadIdx.x] = plane_tile[threadIdx.x] & valid;
+    }
+    if (GSUM) {
+        // wavefront w adds columns w, w + 8, ... of the tile for its row (lane), one running sum per slot
+        const int g0 = c0 / gsize;
+        float acc[DWN_GS_SLOTS];
+#pragma unroll
+        for (int sl = 0; sl < DWN_GS_SLOTS; ++sl) acc[sl] = 0.0f;
+        for (int cc = wave; cc < cend; cc += DWN_FW) {
+            const int sl = (c0 + cc) / gsize - g0;  // wave-uniform
+            const float v = tile[cc][lane];
+#pragma unroll
+            for (int q = 0; q < DWN_GS_SLOTS; ++q) acc[q] += (q == sl) ? v : 0.0f;
+        }
+#pragma unroll
+        for (int sl = 0; sl < DWN_GS_SLOTS; ++sl) gpart[wave][sl][lane] = acc[sl];
+        __syncthreads();
+        if ((int)threadIdx.x < 64 * slots) {
+            const int sl = threadIdx.x >> 6;
+            float sum = 0.0f;
+#pragma unroll
+            for (int w = 0; w < DWN_FW; ++w) sum += gpart[w][sl][lane];
+            y[((size_t)ctile * slots + sl) * ((size_t)BT * 64) + t * 64 + lane] = sum;  // y = the partial sums here
+        }
+        return;
     }
     if (CHAIN && !y) return;
     for (int e = threadIdx.x; e < 64 * DWN_TC; e += 64 * DWN_FW) {
@@ -302,11 +333,14 @@ __device__ __forceinline__ int dwn_quad_xor(int v) {
 }
 // IN_T: gy arrives tile-major already ([B/64][N*O][64], e.g. the input gradient a following layer
 // wrote in that form); only the histogram is left to do.
-template <bool WRITE_T, bool IN_T = false>
+// GROUPS: gy is the gradient of a GroupSum head, [B][groups]: column c takes gy[b][c / gsize] * inv_tau,
+// so the [B, N*O] gradient of the layer's output is never written.
+template <bool WRITE_T, bool IN_T = false, bool GROUPS = false>
 __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__restrict__ gy, const uint8_t *__restrict__ addrT,
                                                                float *__restrict__ gyT, float *__restrict__ gluts,
                                                                int B, int NO, int O, int L, int BP, int BT,
-                                                               int tiles_per_chunk) {
+                                                               int tiles_per_chunk, int groups = 0, int gsize = 1,
+                                                               float inv_tau = 1.0f) {
     __shared__ float tile[64][DWN_HC + 1];       // [row][column]
     __shared__ float hist[DWN_HC][65];           // [column][bin]
     __shared__ uint8_t atile[DWN_HC][64 + 4];    // [column][row] addresses
@@ -332,6 +366,15 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
             if (IN_T) {  // 16 threads x 16 B = the 256 contiguous bytes of one column
                 if (tc + 16 * p < cend)
                     pre[p] = *reinterpret_cast<const float4 *>(gy + ((size_t)t * NO + c0 + tc + 16 * p) * 64 + tr);
+            } else if (GROUPS) {
+                if (b < B) {
+                    const float *src = gy + (size_t)b * groups;
+                    const int c = c0 + q * 4;
+                    if (q * 4 + 0 < cend) pre[p].x = src[(c + 0) / gsize] * inv_tau;
+                    if (q * 4 + 1 < cend) pre[p].y = src[(c + 1) / gsize] * inv_tau;
+                    if (q * 4 + 2 < cend) pre[p].z = src[(c + 2) / gsize] * inv_tau;
+                    if (q * 4 + 3 < cend) pre[p].w = src[(c + 3) / gsize] * inv_tau;
+                }
             } else if (b < B) {
                 const float *src = gy + (size_t)b * NO + c0 + q * 4;
                 if (vec4) {
@@ -571,9 +614,18 @@ extern "C" size_t dl_dwn_bwd_workspace_bytes(int B, int I, int N, int k, int O) 
 
 template <int K>
 static void dwn_launch_lookup(const u64 *planes, const int *idx32, const float *luts, float *y, uint8_t *addrT,
-                              u64 *planes_out, int B, int I, int N, int O, hipStream_t s) {
+                              u64 *planes_out, int B, int I, int N, int O, hipStream_t s, int gsize = 0, int slots = 0) {
     const int BT = dwn_bt(B);
     const int grid = dl_xcd_grid(dl_ceil_div((long long)N * O, DWN_TC), BT);
+    if (gsize > 0) {  // y holds the per-tile group sums
+        if (O == 1)
+            DL_TIMED("dwn_lookup_fwd", s, (dwn_lookup_fwd<K, true, false, true><<<grid, 64 * DWN_FW, 0, s>>>(
+                                              planes, idx32, luts, y, addrT, nullptr, B, I, N, O, BT, gsize, slots)));
+        else
+            DL_TIMED("dwn_lookup_fwd", s, (dwn_lookup_fwd<K, false, false, true><<<grid, 64 * DWN_FW, 0, s>>>(
+                                              planes, idx32, luts, y, addrT, nullptr, B, I, N, O, BT, gsize, slots)));
+        return;
+    }
 #define DWN_LOOKUP(O1_, CHAIN_)                                                                                        \
     DL_TIMED("dwn_lookup_fwd", s,                                                                                      \
              (dwn_lookup_fwd<K, O1_, CHAIN_><<<grid, 64 * DWN_FW, 0, s>>>(planes, idx32, luts, y, addrT, planes_out, B, I, \
@@ -631,9 +683,14 @@ static void dwn_launch_gx(const float *gyT, const uint8_t *addrT, const float *D
 // gx row-major [B, I] or (gx_tiled) tile-major [B/64][I][64]
 // scale == null: EFD weights alpha * beta^h; otherwise the stabilised weights scale[n] / (h + 1),
 // which also multiply the table gradient
+struct DwnGroupHead {
+    int groups, gsize;
+    float inv_tau;
+};
 static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos, const float *luts,
                              const float *gy, int gy_tiled, float alpha, float beta, const float *scale, float *gx,
-                             int gx_tiled, float *gluts, void *ws, int B, int I, int N, int k, int O, hipStream_t s) {
+                             int gx_tiled, float *gluts, void *ws, int B, int I, int N, int k, int O, hipStream_t s,
+                             const DwnGroupHead *head = nullptr) {
     const long long NO = (long long)N * O;
     const int L = 1 << k;
     const uint8_t *addrT = (const uint8_t *)saved;
@@ -657,7 +714,15 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
                  (dwn_efd_table<<<dl_ceil_div(NO, 4), 256, 0, s>>>(luts, D, gluts, (int)NO, k, alpha, beta, sform ? 1 : 0)));
     else
         dl_fill_zero(gluts, NO * L, s);
-    if (gy_tiled)
+    if (head && gx)
+        DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<true, false, true><<<hgrid, 256, 0, s>>>(
+                                                  gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc, head->groups,
+                                                  head->gsize, head->inv_tau)));
+    else if (head)
+        DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<false, false, true><<<hgrid, 256, 0, s>>>(
+                                                  gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc, head->groups,
+                                                  head->gsize, head->inv_tau)));
+    else if (gy_tiled)
         DL_TIMED("dwn_bwd_hist_tiled", s, (dwn_bwd_transpose_hist<false, true><<<hgrid, 256, 0, s>>>(
                                               gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc)));
     else if (gx)
@@ -776,6 +841,76 @@ extern "C" int dl_dwn_layer_fwd_planes(const void *planes_in, const int32_t *idx
         default: dwn_launch_lookup<6>(planes, idx32, luts, y, addrT, po, B, I, N, O, s); break;
     }
     return dl_launch_status();
+}
+
+// ---- GroupSum head on the last layer of a chain
+// logits[b][g] = inv_tau * (sum of the per-tile partial sums of group g, tiles in ascending order)
+__global__ __launch_bounds__(256) void dwn_group_finish(const float *__restrict__ partial, float *__restrict__ logits, int B,
+                                                         int BP, int F, int groups, int gsize, int slots, float inv_tau) {
+    const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (e >= (long long)B * groups) return;
+    const int g = (int)(e / B), b = (int)(e % B);
+    const int c_lo = g * gsize, c_hi = min(F, c_lo + gsize);
+    float sum = 0.0f;
+    if (c_lo < c_hi)
+        for (int ct = c_lo / DWN_TC; ct <= (c_hi - 1) / DWN_TC; ++ct)
+            sum += partial[((size_t)ct * slots + (g - (ct * DWN_TC) / gsize)) * BP + b];
+    logits[(size_t)b * groups + g] = sum * inv_tau;
+}
+// groups the columns of one tile can touch, and the size of a group (features padded up to groups * gsize)
+static inline int dwn_group_size(int F, int groups) { return (F + groups - 1) / groups; }
+static inline int dwn_group_slots(int gsize) { return (DWN_TC - 1) / gsize + 2; }
+
+extern "C" size_t dl_dwn_groups_workspace_bytes(int B, int N, int O, int groups) {
+    if (B <= 0 || N <= 0 || O <= 0 || groups <= 0) return 256;
+    const long long F = (long long)N * O;
+    const int slots = dwn_group_slots(dwn_group_size((int)F, groups));
+    return dl_align256((size_t)dl_ceil_div(F, DWN_TC) * slots * dwn_bt(B) * 64 * sizeof(float));
+}
+
+extern "C" int dl_dwn_layer_fwd_planes_groups(const void *planes_in, const int32_t *idx32, const float *luts, float *logits,
+                                              void *saved, void *ws, size_t ws_bytes, int B, int I, int N, int k, int O,
+                                              int groups, float tau, void *stream) {
+    if (!planes_in || !idx32 || !luts || !logits || !saved || !ws) return DL_ERR_NULL;
+    int rc = dwn_check(B, I, N, k, O);
+    if (rc) return rc;
+    if (groups <= 0 || !(tau > 0.0f)) return DL_ERR_SHAPE;
+    if (!dwn_fast(N, k, O)) return DL_ERR_UNSUPPORTED;
+    const int F = N * O, gsize = dwn_group_size(F, groups), slots = dwn_group_slots(gsize);
+    if (slots > DWN_GS_SLOTS) return DL_ERR_UNSUPPORTED;  // groups narrower than half a column tile
+    if (ws_bytes < dl_dwn_groups_workspace_bytes(B, N, O, groups)) return DL_ERR_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    const u64 *planes = (const u64 *)planes_in;
+    uint8_t *addrT = (uint8_t *)saved;
+    float *partial = (float *)ws;
+    switch (k) {
+        case 1: dwn_launch_lookup<1>(planes, idx32, luts, partial, addrT, nullptr, B, I, N, O, s, gsize, slots); break;
+        case 2: dwn_launch_lookup<2>(planes, idx32, luts, partial, addrT, nullptr, B, I, N, O, s, gsize, slots); break;
+        case 3: dwn_launch_lookup<3>(planes, idx32, luts, partial, addrT, nullptr, B, I, N, O, s, gsize, slots); break;
+        case 4: dwn_launch_lookup<4>(planes, idx32, luts, partial, addrT, nullptr, B, I, N, O, s, gsize, slots); break;
+        case 5: dwn_launch_lookup<5>(planes, idx32, luts, partial, addrT, nullptr, B, I, N, O, s, gsize, slots); break;
+        default: dwn_launch_lookup<6>(planes, idx32, luts, partial, addrT, nullptr, B, I, N, O, s, gsize, slots); break;
+    }
+    DL_TIMED("dwn_group_finish", s,
+             (dwn_group_finish<<<dl_ceil_div((long long)B * groups, 256), 256, 0, s>>>(partial, logits, B, dwn_bt(B) * 64, F,
+                                                                                     groups, gsize, slots, 1.0f / tau)));
+    return dl_launch_status();
+}
+
+extern "C" int dl_dwn_layer_bwd_groups(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos, const float *luts,
+                                       const float *glogits, int groups, float tau, float alpha, float beta, float *gx,
+                                       int gx_tiled, float *gluts, void *ws, size_t ws_bytes, int B, int I, int N, int k,
+                                       int O, void *stream) {
+    if (!saved || !luts || !glogits || !gluts || !ws) return DL_ERR_NULL;
+    if (gx && (!inv_ptr || !inv_pos)) return DL_ERR_NULL;
+    int rc = dwn_check(B, I, N, k, O);
+    if (rc) return rc;
+    if (groups <= 0 || !(tau > 0.0f)) return DL_ERR_SHAPE;
+    if (!dwn_fast(N, k, O)) return DL_ERR_UNSUPPORTED;
+    if (ws_bytes < dl_dwn_bwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
+    const DwnGroupHead head = {groups, dwn_group_size(N * O, groups), 1.0f / tau};
+    return dwn_backward_fast(saved, inv_ptr, inv_pos, luts, glogits, 0, alpha, beta, nullptr, gx, gx_tiled, gluts, ws, B, I, N,
+                             k, O, (hipStream_t)stream, &head);
 }
 
 extern "C" int dl_dwn_layer_bwd_tiled(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos,

@@ -169,10 +169,10 @@ class ConvolutionalLayer(LUTLayerMixin, nn.Module):
         kind, h = self._kind, patches
         if image is not None:
             scalars = [node.efd_scalars() for node in firsts]
-            return ops.DWNStackFunction.apply(image, self._geometry(), plans, scalars, *[b["luts"] for b in banks])
+            return ops.DWNStackFunction.apply(image, self._geometry(), plans, scalars, None, *[b["luts"] for b in banks])
         if kind == "dwn" and self.training and self.n_inputs_per_node <= ops.FAST_K:
             scalars = [node.efd_scalars() for node in firsts]
-            return ops.DWNStackFunction.apply(h, None, plans, scalars, *[b["luts"] for b in banks])
+            return ops.DWNStackFunction.apply(h, None, plans, scalars, None, *[b["luts"] for b in banks])
         for plan, bank, node in zip(plans, banks, firsts):
             if kind == "dwn":
                 if self.training:

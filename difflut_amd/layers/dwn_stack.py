@@ -18,13 +18,27 @@ class DWNStack(nn.Module):
     with at most 6 inputs and matching widths; anything else (and eval mode) runs the members
     one after the other."""
 
-    def __init__(self, layers, encoder=None):
+    def __init__(self, layers, encoder=None, head=None):
         """`encoder`: a fitted, flattening ThermometerEncoder whose code feeds the first layer; the stack
         then takes the raw features and equals `layerN(... layer1(encoder.encode(x)))`.  On the chained
-        path the code is never written as a [batch, features * bits] fp32 tensor."""
+        path the code is never written as a [batch, features * bits] fp32 tensor.
+        `head`: a GroupSum applied to the last layer's output (`head(layerN(...))`); on the chained path the
+        last layer sums its columns per group itself and its [batch, nodes] output is never written."""
         super().__init__()
         self.layers = nn.ModuleList(layers)
         self.encoder = encoder
+        self.head = head
+
+    def _fusable_head(self):
+        from ..utils.modules import GroupSum
+
+        head = self.head
+        if not isinstance(head, GroupSum) or head.use_randperm:
+            return False
+        last = self.layers[-1]
+        features = last.output_size * last.output_dim_per_node
+        # groups at least 64 columns wide and no zero-padding warning to reproduce
+        return features % head.k == 0 and features // head.k >= 64
 
     def _chainable(self):
         width = None
@@ -49,7 +63,7 @@ class DWNStack(nn.Module):
                 x = self.encoder.encode(x)
             for layer in self.layers:
                 x = layer(x)
-            return x
+            return x if self.head is None else self.head(x)
         thresholds = None
         if self.encoder is not None:
             if self._fusable_encoder(x):
@@ -63,4 +77,7 @@ class DWNStack(nn.Module):
         plans = [layer.mapping_plan() for layer in self.layers]
         scalars = [layer.nodes[0].efd_scalars() for layer in self.layers]
         luts = [layer._banks["luts"].tensor() for layer in self.layers]
-        return ops.DWNStackFunction.apply(x, thresholds, plans, scalars, *luts)
+        if self.head is not None and self._fusable_head():
+            return ops.DWNStackFunction.apply(x, thresholds, plans, scalars, (self.head.k, self.head.tau), *luts)
+        y = ops.DWNStackFunction.apply(x, thresholds, plans, scalars, None, *luts)
+        return y if self.head is None else self.head(y)

@@ -168,8 +168,10 @@ class DWNStackFunction(torch.autograd.Function):
     first layer's input gradient, if asked for).  Same arithmetic as calling the layers one by one."""
 
     @staticmethod
-    def forward(ctx, x, source, plans, scalars, *luts):
-        """`source` says what the first layer reads:
+    def forward(ctx, x, source, plans, scalars, head, *luts):
+        """`head`: None, or (groups, tau) of a GroupSum that follows the last layer: the function then returns
+        the [B, groups] sums and neither the last layer's [B, N] output nor its gradient is ever written.
+        `source` says what the first layer reads:
         None                  x [B, I] itself;
         a tensor [F, nbits]   thermometer thresholds: x is raw data [B, F], its code is produced directly
                               as bit-planes and x gets no gradient (the code is a step function of it);
@@ -216,16 +218,25 @@ class DWNStackFunction(torch.autograd.Function):
             dims = (B, width, N, k, O)
             last = l == len(plans) - 1
             keep = _bytes(lib.dl_dwn_saved_bytes(*dims), x.device)
-            y = torch.empty((B, N * O), dtype=torch.float32, device=x.device) if last else None
             nxt = None if last else _bytes(lib.dl_dwn_planes_bytes(B, N * O), x.device)
-            nat.check(lib.dl_dwn_layer_fwd_planes(nat.ptr(planes), nat.ptr(plan.idx32), nat.ptr(lut), nat.ptr(y),
-                                                  nat.ptr(nxt), nat.ptr(keep), *dims, nat.stream()))
+            if last and head is not None:
+                groups, tau = head
+                y = torch.empty((B, groups), dtype=torch.float32, device=x.device)
+                ws = _bytes(lib.dl_dwn_groups_workspace_bytes(B, N, O, groups), x.device)
+                nat.check(lib.dl_dwn_layer_fwd_planes_groups(nat.ptr(planes), nat.ptr(plan.idx32), nat.ptr(lut), nat.ptr(y),
+                                                             nat.ptr(keep), nat.ptr(ws), ws.numel(), *dims, int(groups),
+                                                             float(tau), nat.stream()))
+            else:
+                y = torch.empty((B, N * O), dtype=torch.float32, device=x.device) if last else None
+                nat.check(lib.dl_dwn_layer_fwd_planes(nat.ptr(planes), nat.ptr(plan.idx32), nat.ptr(lut), nat.ptr(y),
+                                                      nat.ptr(nxt), nat.ptr(keep), *dims, nat.stream()))
             saved.append(keep)
             dims_all.append(dims)
             planes, width = nxt, N * O
         ctx.save_for_backward(*luts, *saved)
         ctx.plans, ctx.scalars, ctx.dims_all = plans, scalars, dims_all
         ctx.encoded = thresholds is not None
+        ctx.head = head
         return y
 
     @staticmethod
@@ -253,17 +264,24 @@ class DWNStackFunction(torch.autograd.Function):
                     gx = torch.empty((B, I), dtype=torch.float32, device=g.device)
             grads[l] = torch.empty_like(luts[l])
             ws = _bytes(lib.dl_dwn_bwd_workspace_bytes(*dims), g.device)
-            nat.check(lib.dl_dwn_layer_bwd_tiled(nat.ptr(saved[l]), nat.ptr(plan.inv_ptr), nat.ptr(plan.inv_pos),
-                                                 nat.ptr(luts[l]), nat.ptr(g), tiled, float(alpha), float(beta),
-                                                 nat.ptr(gx), gx_tiled, nat.ptr(grads[l]), nat.ptr(ws), ws.numel(), *dims,
-                                                 nat.stream()))
+            if l == n - 1 and ctx.head is not None:
+                groups, tau = ctx.head
+                nat.check(lib.dl_dwn_layer_bwd_groups(nat.ptr(saved[l]), nat.ptr(plan.inv_ptr), nat.ptr(plan.inv_pos),
+                                                      nat.ptr(luts[l]), nat.ptr(g), int(groups), float(tau), float(alpha),
+                                                      float(beta), nat.ptr(gx), gx_tiled, nat.ptr(grads[l]), nat.ptr(ws),
+                                                      ws.numel(), *dims, nat.stream()))
+            else:
+                nat.check(lib.dl_dwn_layer_bwd_tiled(nat.ptr(saved[l]), nat.ptr(plan.inv_ptr), nat.ptr(plan.inv_pos),
+                                                     nat.ptr(luts[l]), nat.ptr(g), tiled, float(alpha), float(beta),
+                                                     nat.ptr(gx), gx_tiled, nat.ptr(grads[l]), nat.ptr(ws), ws.numel(), *dims,
+                                                     nat.stream()))
             g, tiled = gx, gx_tiled
         if ctx.image is not None and g is not None:
             shape, geom = ctx.image
             gimg = torch.empty(shape, dtype=torch.float32, device=g.device)
             nat.check(lib.dl_fold(nat.ptr(g), 1, nat.ptr(gimg), *shape, *geom, nat.stream()))
             g = gimg
-        return (g, None, None, None, *grads)
+        return (g, None, None, None, None, *grads)
 
 
 def dwn_layer_eval(x, luts, plan):

@@ -108,6 +108,22 @@ int dl_dwn_layer_bwd_tiled(const void *saved, const int32_t *inv_ptr, const int3
                            const float *luts, const float *gy, int gy_tiled, float alpha, float beta,
                            float *gx, int gx_tiled, float *gluts, void *ws, size_t ws_bytes,
                            int B, int I, int N, int k, int O, void *stream);
+/* GroupSum head on the last layer of a chain (utils/modules.py:116-163 after random_layer.py:306-340).
+ * No counterpart in the reference, which writes the layer's [B, N*O] output, sums it per group and in
+ * the backward expands the [B, groups] gradient to [B, N*O] again.  Here the last layer hands out
+ *   logits[b][g] = (sum of its columns g*gs .. (g+1)*gs - 1) / tau,  gs = ceil(N*O / groups)
+ * (columns past N*O count as 0, as the zero-padding of GroupSum does) and its backward takes the
+ * gradient of the logits: column c gets glogits[b][c / gs] / tau.  Groups must be at least 64 columns
+ * wide (DL_ERR_UNSUPPORTED otherwise), k <= DL_MAX_FAST_K.  Sums run in a fixed order (reproducible).
+ *   workspace of the forward: dl_dwn_groups_workspace_bytes; of the backward: dl_dwn_bwd_workspace_bytes */
+size_t dl_dwn_groups_workspace_bytes(int B, int N, int O, int groups);
+int dl_dwn_layer_fwd_planes_groups(const void *planes_in, const int32_t *idx32, const float *luts, float *logits,
+                                   void *saved, void *ws, size_t ws_bytes, int B, int I, int N, int k, int O,
+                                   int groups, float tau, void *stream);
+int dl_dwn_layer_bwd_groups(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos, const float *luts,
+                            const float *glogits, int groups, float tau, float alpha, float beta,
+                            float *gx, int gx_tiled, float *gluts, void *ws, size_t ws_bytes,
+                            int B, int I, int N, int k, int O, void *stream);
 /* Eval forward (DWNNode.forward_eval, dwn_node.py:457-483): addr = floor(sum_j x_j 2^j)
  * with no thresholding of x (clamped to the table), y = (luts[n,d,addr] >= 0.5) as 0/1. */
 int dl_dwn_layer_eval(const float *x, const int32_t *idx32, const float *luts, float *y,

@@ -420,6 +420,87 @@ def test_dwn_stack_with_thermometer_encoder(case):
     assert torch.equal(stack(x), he)
 
 
+@pytest.mark.parametrize("case", [(130, 37, [60, 640], 6, 10, 1.0), (64, 100, [2000], 6, 10, 2.5), (700, 50, [300, 768], 4, 3, 0.5),
+                                  (65, 30, [90, 130], 5, 2, 1.0), (256, 64, [512], 6, 8, 1.0), (33, 40, [1000], 6, 7, 1.0)])
+def test_dwn_stack_with_group_sum_head(case):
+    """DWNStack(..., head=GroupSum): the last layer sums its columns per group itself.  Against the
+    layers one by one followed by GroupSum: logits to rtol 1e-5 (fp32 sums in another order), and
+    against the oracle's group_sum of the bit-exact layer output; table and input gradients to
+    rtol 1e-5; two runs give identical bits (fixed summation order).  The last case has groups that
+    do not divide the width and takes the unfused head."""
+    REGISTRY, NodeConfig, uniform_init, _ = _api()
+    from difflut_amd.layers import DWNStack
+    from difflut_amd.utils import GroupSum
+    import warnings
+    B, I, widths, k, groups, tau = case
+    torch.manual_seed(B + I + groups)
+    layers, width = [], I
+    for li, n in enumerate(widths):
+        layers.append(REGISTRY.get_layer("random")(width, n, REGISTRY.get_node("dwn"),
+                                                   NodeConfig(input_dim=k, output_dim=1, init_fn=uniform_init,
+                                                              init_kwargs={"a": -1.0, "b": 2.0}), seed=li + 21).cuda())
+        width = n
+    head = GroupSum(k=groups, tau=tau, use_randperm=False)
+    x = torch.rand(B, I, device="cuda")
+    glog = torch.randn(B, groups, device="cuda")
+    xa = x.clone().requires_grad_()
+    h = xa
+    for layer in layers:
+        h = layer(h)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        logits = head(h)
+    logits.backward(glog)
+    want_gl = [layer._banks["luts"].flat.grad.clone() for layer in layers]
+    want_gx = xa.grad.clone()
+    for layer in layers:
+        layer._banks["luts"].flat.grad = None
+    stack = DWNStack(layers, head=head).train()
+    assert stack._fusable_head() == (widths[-1] % groups == 0)
+    xb = x.clone().requires_grad_()
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        got = stack(xb)
+    assert got.shape == (B, groups)
+    torch.testing.assert_close(got.detach(), logits.detach(), rtol=1e-5, atol=1e-5)
+    want = orc.group_sum(h.detach().cpu().numpy(), groups, tau)
+    np.testing.assert_allclose(got.detach().cpu().numpy(), want, rtol=1e-5, atol=1e-5)
+    got.backward(glog)
+    for layer, want_g in zip(layers, want_gl):  # bins are sums of up to B values of size ~1/tau with cancellation
+        torch.testing.assert_close(layer._banks["luts"].flat.grad, want_g, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(xb.grad, want_gx, rtol=1e-5, atol=5e-6)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        again = stack(x)
+    assert torch.equal(again, got.detach())
+    # eval mode: members one by one, then the head
+    stack.eval()
+    he = x
+    for layer in layers:
+        layer.eval()
+        he = layer(he)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        assert torch.equal(stack(x), head(he))
+
+
+def test_group_head_entry_points_reject_bad_arguments():
+    """Error codes: -1 null pointer, -2 shape, -3 unsupported, -4 workspace too small."""
+    from difflut_amd import _native as nat
+    lib = nat.lib()
+    one = torch.zeros(4096, device="cuda")
+    p = one.data_ptr()
+    args = (64, 32, 128, 6, 1)
+    # groups narrower than 64 columns are not supported by the fused head
+    assert lib.dl_dwn_layer_fwd_planes_groups(p, p, p, p, p, p, 1 << 20, *args, 4, 1.0, nat.stream()) == -3
+    assert lib.dl_dwn_layer_fwd_planes_groups(p, p, p, p, p, p, 1 << 20, *args, 0, 1.0, nat.stream()) == -2
+    assert lib.dl_dwn_layer_fwd_planes_groups(p, p, p, p, p, p, 1 << 20, *args, 2, 0.0, nat.stream()) == -2
+    assert lib.dl_dwn_layer_fwd_planes_groups(p, p, p, p, p, p, 16, *args, 2, 1.0, nat.stream()) == -4
+    assert lib.dl_dwn_layer_fwd_planes_groups(p, p, p, None, p, p, 1 << 20, *args, 2, 1.0, nat.stream()) == -1
+    assert lib.dl_dwn_layer_bwd_groups(p, p, p, p, None, 2, 1.0, 0.1, 0.3, p, 0, p, p, 1 << 20, *args, nat.stream()) == -1
+    assert lib.dl_dwn_layer_bwd_groups(p, p, p, p, p, 2, -1.0, 0.1, 0.3, p, 0, p, p, 1 << 20, *args, nat.stream()) == -2
+
+
 def test_dwn_layer_step_replays_from_a_hip_graph():
     """The library never allocates or synchronises, and clears buffers with kernels, so a forward +
     backward can be captured once and replayed; every replay is checked against an eager run on
