@@ -700,7 +700,9 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
     // enough blocks to fill 256 CUs several times over, few enough that the per-block
     // histogram flush (one atomic per bin) stays small next to the streaming work
     const int col_tiles = dl_ceil_div(NO, DWN_HC);
-    int chunks = dl_ceil_div(1024, col_tiles);
+    // four blocks fit a CU (LDS): at most 1024 blocks, so that all of them are resident at once and
+    // no second, mostly empty round of blocks follows
+    int chunks = col_tiles >= 1024 ? 1 : 1024 / col_tiles;
     if (chunks > BT) chunks = BT;
     const int tpc = dl_ceil_div(BT, chunks);
     chunks = dl_ceil_div(BT, tpc);
