@@ -187,12 +187,12 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
     }
     if (GSUM) {
         // wavefront w adds columns w, w + 8, ... of the tile for its row (lane), one running sum per slot
-        const int g0 = c0 / gsize;
+        const int b1 = (c0 / gsize + 1) * gsize - c0;  // first column of the tile that belongs to slot 1
         float acc[DWN_GS_SLOTS];
 #pragma unroll
         for (int sl = 0; sl < DWN_GS_SLOTS; ++sl) acc[sl] = 0.0f;
         for (int cc = wave; cc < cend; cc += DWN_FW) {
-            const int sl = (c0 + cc) / gsize - g0;  // wave-uniform
+            const int sl = (cc >= b1 ? 1 : 0) + (cc >= b1 + gsize ? 1 : 0) + (cc >= b1 + 2 * gsize ? 1 : 0);  // wave-uniform
             const float v = tile[cc][lane];
 #pragma unroll
             for (int q = 0; q < DWN_GS_SLOTS; ++q) acc[q] += (q == sl) ? v : 0.0f;
@@ -358,6 +358,11 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
     float4 pre[4];
     unsigned apre[DWN_HC / 4];  // addresses of my 16 columns for the tile being fetched (lane = row)
     const int tc = threadIdx.x >> 4, tr = (threadIdx.x & 15) * 4;  // IN_T: my column in a pass of 16, my 4 rows
+    int grp[4] = {0, 0, 0, 0};  // GROUPS: the groups of my four columns
+    if (GROUPS) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) grp[i] = min(c0 + q * 4 + i, NO - 1) / gsize;
+    }
     auto fetch = [&](int t) {
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
@@ -369,11 +374,10 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
             } else if (GROUPS) {
                 if (b < B) {
                     const float *src = gy + (size_t)b * groups;
-                    const int c = c0 + q * 4;
-                    if (q * 4 + 0 < cend) pre[p].x = src[(c + 0) / gsize] * inv_tau;
-                    if (q * 4 + 1 < cend) pre[p].y = src[(c + 1) / gsize] * inv_tau;
-                    if (q * 4 + 2 < cend) pre[p].z = src[(c + 2) / gsize] * inv_tau;
-                    if (q * 4 + 3 < cend) pre[p].w = src[(c + 3) / gsize] * inv_tau;
+                    if (q * 4 + 0 < cend) pre[p].x = src[grp[0]] * inv_tau;
+                    if (q * 4 + 1 < cend) pre[p].y = src[grp[1]] * inv_tau;
+                    if (q * 4 + 2 < cend) pre[p].z = src[grp[2]] * inv_tau;
+                    if (q * 4 + 3 < cend) pre[p].w = src[grp[3]] * inv_tau;
                 }
             } else if (b < B) {
                 const float *src = gy + (size_t)b * NO + c0 + q * 4;
