@@ -41,6 +41,8 @@ WORKLOADS = {
     # secondary workloads of the same path, reported with their own metric names (see run_secondary)
     "prob_k4_b1024_i4096_n4096": (1024, 4096, 4096, 4, 1),
     "softmap_b512_i3136_m48000": (512, 3136, 8000, 6, 1),
+    # the whole layer of that configuration through the layer API: soft connectivity feeding 8000 DWN nodes
+    "learnable_layer_b512_i3136_n8000": (512, 3136, 8000, 6, 1),
     # the headline layer shape with the two other table-lookup node types
     "stable_k6_b4096_i16384_n8192": (4096, 16384, 8192, 6, 1),
     "hybrid_k6_b4096_i16384_n8192": (4096, 16384, 8192, 6, 1),
@@ -197,6 +199,50 @@ def run_conv(args):
     print(json.dumps(out_d))
 
 
+def run_learnable(args):
+    """LearnableLayer (soft connectivity over 3136 inputs -> 8000 DWN nodes with k=6): forward and backward with the
+    input, mapping-weight and table gradients, through the module API."""
+    from difflut_amd import REGISTRY
+    from difflut_amd.nodes.node_config import NodeConfig
+
+    dev = torch.device("cuda:0")
+    B, I, N, k, O = WORKLOADS[args.workload]
+    torch.manual_seed(0)
+    layer = REGISTRY.get_layer("learnable")(I, N, REGISTRY.get_node("dwn"), NodeConfig(input_dim=k, output_dim=O),
+                                            tau=1.0, tau_start=1.0, tau_min=1e-4, tau_decay_iters=1000,
+                                            use_cuda_soft=False).to(dev).train()
+    layer.mapping.precision = args.precision  # 0: fp32 matrix cores, 1: bf16 operands with fp32 accumulation
+    with torch.no_grad():
+        layer.mapping.W.normal_(0, 0.01)
+    x = torch.rand(B, I, device=dev, requires_grad=True)
+    gy = torch.randn(B, N * O, device=dev)
+    W = layer.mapping.W
+    banks = layer.bank_parameters()
+
+    def step():
+        x.grad = None
+        W.grad = None
+        for t in banks:
+            t.grad = None
+        layer(x).backward(gy)
+
+    ms = time_steps(step, args.steps, args.warmup)
+    M = N * k
+    flops = 3 * 2 * B * I * M
+    peak = 157.3 if args.precision == 0 else 2500.0
+    out = {"metric": "LUT-node evals/sec fwd+bwd (LearnableLayer soft connectivity 3136 -> 8000 DWN k=6 nodes, B=512)",
+           "value": B * N / (ms * 1e-3), "unit": "node-evals/s", "ms_per_step": ms,
+           "dtype": "f32" if args.precision == 0 else "bf16 operands, f32 accumulate (soft connectivity); f32 elsewhere",
+           "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "data": "synthetic",
+           "config": {"workload": args.workload, "batch": B, "inputs": I, "nodes": N, "k": k, "mapping_rows": M,
+                      "precision": args.precision},
+           "roofline_step": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
+                             "frac": flops / (ms * 1e-3) / 1e12 / peak, "algorithmic_flops_per_step": flops},
+           "kernel_ms": kernel_times(step, min(args.steps, 5))}
+    print(json.dumps(out))
+
+
 def maybe_graph(step, args):
     """With --graph: the step's launches captured once (after warm-up, on a side stream as torch requires) and
     replayed; the library never allocates, synchronises or uses memset nodes, so a step is capturable as it is."""
@@ -351,6 +397,8 @@ def main():
         return run_stack(args)
     if args.workload.startswith("conv"):
         return run_conv(args)
+    if args.workload.startswith("learnable"):
+        return run_learnable(args)
     if not args.workload.startswith("dwn"):
         return run_secondary(args)
     dev = torch.device("cuda:0")
