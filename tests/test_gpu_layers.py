@@ -421,7 +421,8 @@ def test_dwn_stack_with_thermometer_encoder(case):
 
 
 @pytest.mark.parametrize("case", [(130, 37, [60, 640], 6, 10, 1.0), (64, 100, [2000], 6, 10, 2.5), (700, 50, [300, 768], 4, 3, 0.5),
-                                  (65, 30, [90, 130], 5, 2, 1.0), (256, 64, [512], 6, 8, 1.0), (33, 40, [1000], 6, 7, 1.0)])
+                                  (65, 30, [90, 130], 5, 2, 1.0), (256, 64, [512], 6, 8, 1.0), (33, 40, [1000], 6, 7, 1.0),
+                                  (100, 48, [70, 192], 4, 3, 1.0, 2)])
 def test_dwn_stack_with_group_sum_head(case):
     """DWNStack(..., head=GroupSum): the last layer sums its columns per group itself.  Against the
     layers one by one followed by GroupSum: logits to rtol 1e-5 (fp32 sums in another order), and
@@ -432,14 +433,15 @@ def test_dwn_stack_with_group_sum_head(case):
     from difflut_amd.layers import DWNStack
     from difflut_amd.utils import GroupSum
     import warnings
-    B, I, widths, k, groups, tau = case
+    B, I, widths, k, groups, tau = case[:6]
+    O = case[6] if len(case) > 6 else 1  # outputs per node: the last case has two, groups run over node-major columns
     torch.manual_seed(B + I + groups)
     layers, width = [], I
     for li, n in enumerate(widths):
         layers.append(REGISTRY.get_layer("random")(width, n, REGISTRY.get_node("dwn"),
-                                                   NodeConfig(input_dim=k, output_dim=1, init_fn=uniform_init,
+                                                   NodeConfig(input_dim=k, output_dim=O, init_fn=uniform_init,
                                                               init_kwargs={"a": -1.0, "b": 2.0}), seed=li + 21).cuda())
-        width = n
+        width = n * O
     head = GroupSum(k=groups, tau=tau, use_randperm=False)
     x = torch.rand(B, I, device="cuda")
     glog = torch.randn(B, groups, device="cuda")
@@ -456,7 +458,7 @@ def test_dwn_stack_with_group_sum_head(case):
     for layer in layers:
         layer._banks["luts"].flat.grad = None
     stack = DWNStack(layers, head=head).train()
-    assert stack._fusable_head() == (widths[-1] % groups == 0)
+    assert stack._fusable_head() == (widths[-1] * O % groups == 0)
     xb = x.clone().requires_grad_()
     with warnings.catch_warnings():
         warnings.simplefilter("ignore")
