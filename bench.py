@@ -51,6 +51,8 @@ WORKLOADS = {
     "conv_b256_c4_28x28_o32_rf5_d2": (256, 4, 32, 6, 1),
     # whole training step of the deep stack through the layer API: (B, features, first layer width, k, O)
     "dwn_stack_b8192_train_step": (8192, 784, 16000, 6, 1),
+    # the same model in eval mode (inference): thermometer code and activations as bit-planes, GroupSum as a count
+    "dwn_stack_b8192_eval_forward": (8192, 784, 16000, 6, 1),
 }
 
 
@@ -121,6 +123,38 @@ def run_stack(args):
     from difflut_amd.layers import DWNStack
     # same layers; thermometer code and activations as bit-planes, tile-major gradients between layers
     stack = DWNStack(layers, encoder=enc, head=head).train()
+
+    if args.workload.endswith("eval_forward"):
+        stack.eval()
+        for layer in layers:
+            layer.eval()
+
+        def infer():
+            with torch.no_grad():
+                if args.layer_by_layer:
+                    h = enc.encode(x)
+                    for layer in layers:
+                        h = layer(h)
+                    return head(h)
+                return stack(x)
+
+        ms = time_steps(infer, args.steps, args.warmup)
+        evals = B * sum(widths)
+        ins = [F * 4] + widths[:-1]
+        nbytes = sum(4 * B * (i + n) for i, n in zip(ins, widths)) + sum(widths) * (1 << k) * 4
+        out = {"metric": "LUT-node evals/sec, inference (thermometer -> 4 DWN k=6 layers -> GroupSum)",
+               "value": evals / (ms * 1e-3), "unit": "node-evals/s", "ms_per_step": ms, "dtype": "f32 tables, 1-bit activations",
+               "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+               "vs_baseline": None, "data": "synthetic",
+               "config": {"workload": args.workload, "batch": B, "features": F, "layers": widths, "k": k,
+                          "execution": "layer by layer" if args.layer_by_layer else "chained (DWNStack)"},
+               "roofline_step": {"bound": "hbm", "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                 "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                 "algorithmic_bytes_per_step": nbytes,
+                                 "note": "bytes of the layer-by-layer fp32 formulation (x and y per layer, tables once)"},
+               "kernel_ms": kernel_times(infer, min(args.steps, 5))}
+        print(json.dumps(out))
+        return
 
     def step():
         opt.zero_grad(set_to_none=True)

@@ -106,7 +106,10 @@ __global__ __launch_bounds__(256) void dwn_pack_planes(const float *__restrict__
 // partial[(column tile * slots + slot)][row], slot = group - first group of the tile; dwn_group_finish
 // adds the tiles of a group in a fixed order.
 #define DWN_GS_SLOTS 4
-template <int K, bool O1, bool CHAIN = false, bool GSUM = false>
+// EVAL: the inference form (DWNNode.forward_eval on inputs that are exactly 0 or 1, where its address
+// floor(sum x_j 2^j) is the thresholded one): the output is (table entry >= 0.5) as 0/1, nothing is saved
+// for a backward.
+template <int K, bool O1, bool CHAIN = false, bool GSUM = false, bool EVAL = false>
 __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restrict__ planes, const int *__restrict__ idx32,
                                                                const float *__restrict__ luts, float *__restrict__ y,
                                                                uint8_t *__restrict__ addrT, u64 *__restrict__ planes_out,
@@ -167,14 +170,15 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
                 for (int j = K - 1; j >= 0; --j) addr = dwn_shift_in(addr, w[q][j]);
                 const float v = dl_lane_read(entry[q], (int)addr);
                 if (cc < cend) {
-                    tile[cc][lane] = v;
+                    tile[cc][lane] = EVAL ? (v >= 0.5f ? 1.0f : 0.0f) : v;
                     if (CHAIN && planes_out) {  // the next layer's view of this column: bit r = (y[64t+r][c] >= 0.5)
                         const u64 m = __ballot(v >= 0.5f);
                         if (lane == 0) plane_tile[cc] = m;
                     }
                     const int c = c0 + cc;
                     const int n = O1 ? c : c / O;
-                    if (O1 || c - n * O == 0) __builtin_amdgcn_raw_buffer_store_b8((uint8_t)addr, rs_addr, lane, n * 64, 0);
+                    if (!EVAL && (O1 || c - n * O == 0))
+                        __builtin_amdgcn_raw_buffer_store_b8((uint8_t)addr, rs_addr, lane, n * 64, 0);
                 }
             }
         }
@@ -618,9 +622,22 @@ extern "C" size_t dl_dwn_bwd_workspace_bytes(int B, int I, int N, int k, int O) 
 
 template <int K>
 static void dwn_launch_lookup(const u64 *planes, const int *idx32, const float *luts, float *y, uint8_t *addrT,
-                              u64 *planes_out, int B, int I, int N, int O, hipStream_t s, int gsize = 0, int slots = 0) {
+                              u64 *planes_out, int B, int I, int N, int O, hipStream_t s, int gsize = 0, int slots = 0,
+                              bool eval = false) {
     const int BT = dwn_bt(B);
     const int grid = dl_xcd_grid(dl_ceil_div((long long)N * O, DWN_TC), BT);
+    if (eval) {  // addrT is not written
+#define DWN_EVAL(O1_, CHAIN_, GSUM_)                                                                                     \
+    DL_TIMED("dwn_lookup_eval", s, (dwn_lookup_fwd<K, O1_, CHAIN_, GSUM_, true><<<grid, 64 * DWN_FW, 0, s>>>(            \
+                                       planes, idx32, luts, y, addrT, planes_out, B, I, N, O, BT, gsize > 0 ? gsize : 1, \
+                                       slots > 0 ? slots : 1)))
+        if (gsize > 0 && O == 1) DWN_EVAL(true, false, true);
+        else if (gsize > 0) DWN_EVAL(false, false, true);
+        else if (O == 1) DWN_EVAL(true, true, false);
+        else DWN_EVAL(false, true, false);
+#undef DWN_EVAL
+        return;
+    }
     if (gsize > 0) {  // y holds the per-tile group sums
         if (O == 1)
             DL_TIMED("dwn_lookup_fwd", s, (dwn_lookup_fwd<K, true, false, true><<<grid, 64 * DWN_FW, 0, s>>>(
@@ -896,6 +913,57 @@ extern "C" int dl_dwn_layer_fwd_planes_groups(const void *planes_in, const int32
         case 4: dwn_launch_lookup<4>(planes, idx32, luts, partial, addrT, nullptr, B, I, N, O, s, gsize, slots); break;
         case 5: dwn_launch_lookup<5>(planes, idx32, luts, partial, addrT, nullptr, B, I, N, O, s, gsize, slots); break;
         default: dwn_launch_lookup<6>(planes, idx32, luts, partial, addrT, nullptr, B, I, N, O, s, gsize, slots); break;
+    }
+    DL_TIMED("dwn_group_finish", s,
+             (dwn_group_finish<<<dl_ceil_div((long long)B * groups, 256), 256, 0, s>>>(partial, logits, B, dwn_bt(B) * 64, F,
+                                                                                     groups, gsize, slots, 1.0f / tau)));
+    return dl_launch_status();
+}
+
+// ---- inference on binary activations
+extern "C" int dl_dwn_layer_eval_planes(const void *planes_in, const int32_t *idx32, const float *luts, float *y,
+                                        void *planes_out, int B, int I, int N, int k, int O, void *stream) {
+    if (!planes_in || !idx32 || !luts || (!y && !planes_out)) return DL_ERR_NULL;
+    int rc = dwn_check(B, I, N, k, O);
+    if (rc) return rc;
+    if (!dwn_fast(N, k, O)) return DL_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+    const u64 *planes = (const u64 *)planes_in;
+    u64 *po = (u64 *)planes_out;
+    uint8_t *none = (uint8_t *)const_cast<float *>(luts);  // descriptor base of the unused address stores
+    switch (k) {
+        case 1: dwn_launch_lookup<1>(planes, idx32, luts, y, none, po, B, I, N, O, s, 0, 0, true); break;
+        case 2: dwn_launch_lookup<2>(planes, idx32, luts, y, none, po, B, I, N, O, s, 0, 0, true); break;
+        case 3: dwn_launch_lookup<3>(planes, idx32, luts, y, none, po, B, I, N, O, s, 0, 0, true); break;
+        case 4: dwn_launch_lookup<4>(planes, idx32, luts, y, none, po, B, I, N, O, s, 0, 0, true); break;
+        case 5: dwn_launch_lookup<5>(planes, idx32, luts, y, none, po, B, I, N, O, s, 0, 0, true); break;
+        default: dwn_launch_lookup<6>(planes, idx32, luts, y, none, po, B, I, N, O, s, 0, 0, true); break;
+    }
+    return dl_launch_status();
+}
+
+extern "C" int dl_dwn_layer_eval_planes_groups(const void *planes_in, const int32_t *idx32, const float *luts,
+                                               float *logits, void *ws, size_t ws_bytes, int B, int I, int N, int k, int O,
+                                               int groups, float tau, void *stream) {
+    if (!planes_in || !idx32 || !luts || !logits || !ws) return DL_ERR_NULL;
+    int rc = dwn_check(B, I, N, k, O);
+    if (rc) return rc;
+    if (groups <= 0 || !(tau > 0.0f)) return DL_ERR_SHAPE;
+    if (!dwn_fast(N, k, O)) return DL_ERR_UNSUPPORTED;
+    const int F = N * O, gsize = dwn_group_size(F, groups), slots = dwn_group_slots(gsize);
+    if (slots > DWN_GS_SLOTS) return DL_ERR_UNSUPPORTED;
+    if (ws_bytes < dl_dwn_groups_workspace_bytes(B, N, O, groups)) return DL_ERR_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    const u64 *planes = (const u64 *)planes_in;
+    float *partial = (float *)ws;
+    uint8_t *none = (uint8_t *)const_cast<float *>(luts);
+    switch (k) {
+        case 1: dwn_launch_lookup<1>(planes, idx32, luts, partial, none, nullptr, B, I, N, O, s, gsize, slots, true); break;
+        case 2: dwn_launch_lookup<2>(planes, idx32, luts, partial, none, nullptr, B, I, N, O, s, gsize, slots, true); break;
+        case 3: dwn_launch_lookup<3>(planes, idx32, luts, partial, none, nullptr, B, I, N, O, s, gsize, slots, true); break;
+        case 4: dwn_launch_lookup<4>(planes, idx32, luts, partial, none, nullptr, B, I, N, O, s, gsize, slots, true); break;
+        case 5: dwn_launch_lookup<5>(planes, idx32, luts, partial, none, nullptr, B, I, N, O, s, gsize, slots, true); break;
+        default: dwn_launch_lookup<6>(planes, idx32, luts, partial, none, nullptr, B, I, N, O, s, gsize, slots, true); break;
     }
     DL_TIMED("dwn_group_finish", s,
              (dwn_group_finish<<<dl_ceil_div((long long)B * groups, 256), 256, 0, s>>>(partial, logits, B, dwn_bt(B) * 64, F,

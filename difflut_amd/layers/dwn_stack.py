@@ -15,10 +15,11 @@ class DWNStack(nn.Module):
     """`DWNStack([layer1, layer2, ...])(x)` equals `layerN(... layer2(layer1(x)))`.
 
     Training-mode calls take the chained kernels when every member is a RandomLayer of DWN nodes
-    with at most 6 inputs and matching widths; anything else (and eval mode) runs the members
+    with at most 6 inputs and matching widths; so do eval-mode calls whose first input is known to
+    be binary (a fused thermometer encoder, or `binary_input=True`).  Anything else runs the members
     one after the other."""
 
-    def __init__(self, layers, encoder=None, head=None):
+    def __init__(self, layers, encoder=None, head=None, binary_input=False):
         """`encoder`: a fitted, flattening ThermometerEncoder whose code feeds the first layer; the stack
         then takes the raw features and equals `layerN(... layer1(encoder.encode(x)))`.  On the chained
         path the code is never written as a [batch, features * bits] fp32 tensor.
@@ -28,6 +29,9 @@ class DWNStack(nn.Module):
         self.layers = nn.ModuleList(layers)
         self.encoder = encoder
         self.head = head
+        # the caller's promise that x holds exact 0/1 values (an encoder's code does anyway): eval mode can then
+        # run chained as well, since the eval address floor(sum x_j 2^j) is the thresholded one
+        self.binary_input = binary_input
 
     def _fusable_head(self):
         from ..utils.modules import GroupSum
@@ -58,6 +62,16 @@ class DWNStack(nn.Module):
                 and torch.is_tensor(x) and x.shape[1] * enc.num_bits == self.layers[0].input_size)
 
     def forward(self, x):
+        if not self.training and self._chainable() and x.is_cuda and x.dim() == 2 and x.shape[0] > 0:
+            fused_encoder = self.encoder is not None and self._fusable_encoder(x)
+            if fused_encoder or (self.encoder is None and self.binary_input and x.shape[1] == self.layers[0].input_size):
+                thresholds = self.encoder.thresholds.to(x.device) if fused_encoder else None
+                plans = [layer.mapping_plan() for layer in self.layers]
+                luts = [layer._banks["luts"].tensor().detach() for layer in self.layers]
+                fused_head = self.head is not None and self._fusable_head()
+                with torch.no_grad():
+                    y = ops.dwn_stack_eval(x, thresholds, plans, luts, (self.head.k, self.head.tau) if fused_head else None)
+                    return y if self.head is None or fused_head else self.head(y)
         if not (self.training and self._chainable()):
             if self.encoder is not None:
                 x = self.encoder.encode(x)

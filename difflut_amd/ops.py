@@ -284,6 +284,53 @@ class DWNStackFunction(torch.autograd.Function):
         return (g, None, None, None, None, *grads)
 
 
+def dwn_stack_eval(x, thresholds, plans, luts, head=None):
+    """Inference through a chain of RandomLayer + DWN layers whose first input is binary: `thresholds` [F, nbits]
+    (x is raw data, its thermometer code feeds the first layer) or None (x [B, I] holds exact 0/1 values).
+    Activations stay bit-planes between the layers; returns the last layer's 0/1 output [B, N], or with
+    `head` = (groups, tau) its GroupSum [B, groups].  Equals calling the layers' eval forward one by one."""
+    nat.require_device(x, thresholds, *luts)
+    x = _f32(x)
+    lib = nat.lib()
+    B, width = x.shape
+    if thresholds is None:
+        planes = _bytes(lib.dl_dwn_planes_bytes(B, width), x.device)
+        nat.check(lib.dl_dwn_pack_planes(nat.ptr(x), nat.ptr(planes), B, width, nat.stream()))
+    else:
+        thr = _f32(thresholds)
+        if thr.dim() != 2 or thr.shape[0] != width:
+            raise RuntimeError(f"thresholds {tuple(thr.shape)} do not match {width} features")
+        nbits = thr.shape[1]
+        planes = _bytes(lib.dl_dwn_planes_bytes(B, width * nbits), x.device)
+        nat.check(lib.dl_thermometer_planes(nat.ptr(x), nat.ptr(thr), nat.ptr(planes), B, width, nbits, nat.stream()))
+        width *= nbits
+    y = None
+    for l, (plan, lut) in enumerate(zip(plans, luts)):
+        lut = _f32(lut)
+        N, O, L = lut.shape
+        k = plan.k
+        if k > FAST_K or (N, 1 << k, width) != (plan.N, L, plan.I):
+            raise RuntimeError(f"layer {l}: cannot chain (k={k}, tables {tuple(lut.shape)}, mapping [{plan.N},{k}] over "
+                               f"{plan.I} inputs, incoming width {width})")
+        dims = (B, width, N, k, O)
+        last = l == len(plans) - 1
+        if last and head is not None:
+            groups, tau = head
+            y = torch.empty((B, groups), dtype=torch.float32, device=x.device)
+            ws = _bytes(lib.dl_dwn_groups_workspace_bytes(B, N, O, groups), x.device)
+            nat.check(lib.dl_dwn_layer_eval_planes_groups(nat.ptr(planes), nat.ptr(plan.idx32), nat.ptr(lut), nat.ptr(y),
+                                                          nat.ptr(ws), ws.numel(), *dims, int(groups), float(tau),
+                                                          nat.stream()))
+        else:
+            y = torch.empty((B, N * O), dtype=torch.float32, device=x.device) if last else None
+            nxt = None if last else _bytes(lib.dl_dwn_planes_bytes(B, N * O), x.device)
+            nat.check(lib.dl_dwn_layer_eval_planes(nat.ptr(planes), nat.ptr(plan.idx32), nat.ptr(lut), nat.ptr(y),
+                                                   nat.ptr(nxt), *dims, nat.stream()))
+            planes = nxt
+        width = N * O
+    return y
+
+
 def dwn_layer_eval(x, luts, plan):
     nat.require_device(x, luts)
     x, luts = _f32(x), _f32(luts)

@@ -124,6 +124,19 @@ int dl_dwn_layer_bwd_groups(const void *saved, const int32_t *inv_ptr, const int
                             const float *glogits, int groups, float tau, float alpha, float beta,
                             float *gx, int gx_tiled, float *gluts, void *ws, size_t ws_bytes,
                             int B, int I, int N, int k, int O, void *stream);
+/* Inference on binary activations (DWNNode.forward_eval, dwn_node.py:457-483, for inputs that are exactly
+ * 0 or 1 - what a thermometer encoder or a preceding layer's eval output delivers; there its address
+ * floor(sum_j x_j 2^j) equals the thresholded one).  planes_in as dl_dwn_pack_planes /
+ * dl_thermometer_planes / a preceding call write them; y (nullable) = (table entry >= 0.5) as 0/1 fp32
+ * [B, N*O]; planes_out (nullable) = the same bits as planes for the next layer.  The *_groups form
+ * returns GroupSum of that output instead (utils/modules.py:116-163; workspace
+ * dl_dwn_groups_workspace_bytes, groups >= 64 columns wide).  No counterpart in the reference, which
+ * runs its layers on [B, N] fp32 tensors in eval mode too.  k <= DL_MAX_FAST_K. */
+int dl_dwn_layer_eval_planes(const void *planes_in, const int32_t *idx32, const float *luts, float *y,
+                             void *planes_out, int B, int I, int N, int k, int O, void *stream);
+int dl_dwn_layer_eval_planes_groups(const void *planes_in, const int32_t *idx32, const float *luts, float *logits,
+                                    void *ws, size_t ws_bytes, int B, int I, int N, int k, int O,
+                                    int groups, float tau, void *stream);
 /* Eval forward (DWNNode.forward_eval, dwn_node.py:457-483): addr = floor(sum_j x_j 2^j)
  * with no thresholding of x (clamped to the table), y = (luts[n,d,addr] >= 0.5) as 0/1. */
 int dl_dwn_layer_eval(const float *x, const int32_t *idx32, const float *luts, float *y,

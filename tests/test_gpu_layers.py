@@ -486,6 +486,57 @@ def test_dwn_stack_with_group_sum_head(case):
         assert torch.equal(stack(x), head(he))
 
 
+@pytest.mark.parametrize("case", [(130, 37, 4, [60, 640], 6, 10, 1), (64, 25, 4, [2000], 6, 10, 1), (700, 50, 1, [300, 768], 4, 3, 1),
+                                  (65, 30, 3, [90, 130], 5, None, 1), (100, 12, 4, [70, 192], 4, 3, 2), (33, 40, 2, [1000], 6, 7, 1)])
+def test_dwn_stack_eval_runs_chained_on_binary_input(case):
+    """Eval mode of DWNStack behind a thermometer encoder (or on 0/1 input with binary_input=True): bit-planes
+    between the layers, (table >= 0.5) outputs, GroupSum as a count.  Against the oracle's eval forward layer by
+    layer (bit-exact 0/1 outputs; the group sums are integers divided by tau) and against the members run
+    one by one."""
+    REGISTRY, NodeConfig, uniform_init, _ = _api()
+    from difflut_amd.layers import DWNStack
+    from difflut_amd.utils import GroupSum
+    import warnings
+    B, F, nbits, widths, k, groups, O = case
+    torch.manual_seed(B * 3 + F)
+    x = torch.rand(B, F, device="cuda")
+    enc = REGISTRY.build_encoder("thermometer", num_bits=nbits).fit(x)
+    layers, width = [], F * nbits
+    for li, n in enumerate(widths):
+        layers.append(REGISTRY.get_layer("random")(width, n, REGISTRY.get_node("dwn"),
+                                                   NodeConfig(input_dim=k, output_dim=O, init_fn=uniform_init,
+                                                              init_kwargs={"a": 0.0, "b": 1.0}), seed=li + 31).cuda())
+        width = n * O
+    head = GroupSum(k=groups, tau=1.5, use_randperm=False) if groups else None
+    # oracle: encode, then every layer's eval forward on the mapped bits
+    h = orc.thermometer_encode(x.cpu().numpy(), enc.thresholds.cpu().numpy()).reshape(B, -1).astype(np.float32)
+    for layer in layers:
+        idx = layer._mapping_indices.cpu().numpy().astype(np.int64)
+        luts = layer._banks["luts"].tensor().detach().cpu().numpy()
+        h = np.stack([orc.dwn_eval_forward(h[:, idx[n]], luts[n]) for n in range(idx.shape[0])], axis=1).reshape(B, -1)
+    want = h if head is None else orc.group_sum(h, groups, 1.5)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        stack = DWNStack(layers, encoder=enc, head=head).eval()
+        got = stack(x)
+        # the members one by one
+        he = enc.encode(x)
+        for layer in layers:
+            layer.eval()
+            he = layer(he)
+        loop = he if head is None else head(he)
+        # the same stack without the encoder, fed the code itself
+        code = enc.encode(x)
+        plain = DWNStack(layers, head=head, binary_input=True).eval()
+        got_code = plain(code)
+    assert not got.requires_grad
+    if head is None:
+        assert np.array_equal(got.cpu().numpy(), want)
+    else:
+        np.testing.assert_allclose(got.cpu().numpy(), want, rtol=1e-6, atol=0)
+    assert torch.equal(got, loop) and torch.equal(got_code, got)
+
+
 def test_group_head_entry_points_reject_bad_arguments():
     """Error codes: -1 null pointer, -2 shape, -3 unsupported, -4 workspace too small."""
     from difflut_amd import _native as nat
