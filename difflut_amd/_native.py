@@ -33,6 +33,8 @@ SIGNATURES = {
     "dl_dwn_pack_planes": (_I, [_P, _P, _I, _I, _P]),
     "dl_dwn_layer_fwd_planes": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "dl_dwn_layer_bwd_tiled": (_I, [_P, _P, _P, _P, _P, _I, _F, _F, _P, _I, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
+    "dl_dwn_eval_workspace_bytes": (_Z, [_I] * 5),
+    "dl_dwn_layer_eval_ws": (_I, [_P, _P, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
     "dl_dwn_layer_eval_planes": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "dl_dwn_layer_eval_planes_groups": (_I, [_P, _P, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _I, _F, _P]),
     "dl_dwn_groups_workspace_bytes": (_Z, [_I] * 4),

@@ -8,3 +8,6 @@ int dwn_generic_forward(const float *x, const int *idx32, const float *luts, flo
 int dwn_generic_backward(const float *x, const int *idx32, const int *inv_ptr, const int *inv_pos, const float *luts,
                          const float *gy, float alpha, float beta, const float *scale, float *gx, float *gluts, int B, int I,
                          int N, int k, int O, hipStream_t s);
+// Eval forward for any input values; returns at once when *skip_if_set (device, nullable) is non-zero.
+int dwn_generic_eval(const float *x, const int *idx32, const float *luts, float *y, int B, int I, int N, int k, int O,
+                     const int *skip_if_set, hipStream_t s);

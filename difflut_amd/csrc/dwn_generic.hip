@@ -69,9 +69,12 @@ __global__ __launch_bounds__(256) void dwn_generic_bwd_luts(const float *__restr
 }
 
 // Eval: address = floor(sum_j x_j 2^j), no thresholding of x; table value binarised at 0.5.
+// `skip_if_set` (nullable): a device flag; when it reads non-zero another kernel produces y and this one returns.
 __global__ __launch_bounds__(256) void dwn_eval_fwd(const float *__restrict__ x, const int *__restrict__ idx32,
                                                      const float *__restrict__ luts, float *__restrict__ y,
-                                                     int B, int I, int N, int K, int O) {
+                                                     int B, int I, int N, int K, int O,
+                                                     const int *__restrict__ skip_if_set) {
+    if (skip_if_set && *skip_if_set != 0) return;
     const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
     const long long NO = (long long)N * O;
     if (gid >= (long long)B * NO) return;
@@ -115,6 +118,14 @@ extern "C" int dl_dwn_layer_eval(const float *x, const int32_t *idx32, const flo
     if (!x || !idx32 || !luts || !y) return DL_ERR_NULL;
     if (B <= 0 || I <= 0 || N <= 0 || k <= 0 || O <= 0) return DL_ERR_SHAPE;
     if (k > DL_MAX_K) return DL_ERR_UNSUPPORTED;
-    dwn_eval_fwd<<<dl_ceil_div((long long)B * N * O, 256), 256, 0, (hipStream_t)stream>>>(x, idx32, luts, y, B, I, N, k, O);
+    dwn_eval_fwd<<<dl_ceil_div((long long)B * N * O, 256), 256, 0, (hipStream_t)stream>>>(x, idx32, luts, y, B, I, N, k, O,
+                                                                                          nullptr);
+    return dl_launch_status();
+}
+
+int dwn_generic_eval(const float *x, const int *idx32, const float *luts, float *y, int B, int I, int N, int k, int O,
+                     const int *skip_if_set, hipStream_t s) {
+    DL_TIMED("dwn_eval_generic", s, (dwn_eval_fwd<<<dl_ceil_div((long long)B * N * O, 256), 256, 0, s>>>(
+                                        x, idx32, luts, y, B, I, N, k, O, skip_if_set)));
     return dl_launch_status();
 }

@@ -45,10 +45,12 @@ static void dl_fill_zero(float *p, long long n, hipStream_t s) {
 // ---------------------------------------------------------------------------------
 // pack_planes: grid (ceil(I / (256*VEC)), B/64 rounded up), 256 threads, thread = VEC inputs.
 // Every load of a wavefront is one contiguous 64*VEC*4-byte piece of a row of x.
-template <int VEC>
+// CHECK: also clears *all_binary (preset to 1 by the caller) when some value is neither 0 nor 1.
+template <int VEC, bool CHECK = false>
 __global__ __launch_bounds__(256) void dwn_pack_planes(const float *__restrict__ x, u64 *__restrict__ planes,
-                                                        int B, int I) {
+                                                        int B, int I, int *__restrict__ all_binary = nullptr) {
     const int t = blockIdx.y;
+    bool odd = false;  // saw a value other than 0 and 1
     const int i0 = (blockIdx.x * 256 + threadIdx.x) * VEC;
     if (i0 >= I) return;
     const int rows = min(64, B - t * 64);
@@ -69,8 +71,13 @@ __global__ __launch_bounds__(256) void dwn_pack_planes(const float *__restrict__
                     acc[1] |= (q.y >= 0.5f ? 1u : 0u) << r;
                     acc[2] |= (q.z >= 0.5f ? 1u : 0u) << r;
                     acc[3] |= (q.w >= 0.5f ? 1u : 0u) << r;
+                    if (CHECK)
+                        odd = odd || !((q.x == 0.0f || q.x == 1.0f) && (q.y == 0.0f || q.y == 1.0f) &&
+                                       (q.z == 0.0f || q.z == 1.0f) && (q.w == 0.0f || q.w == 1.0f));
                 } else {
-                    acc[0] |= (src[0] >= 0.5f ? 1u : 0u) << r;
+                    const float v0 = src[0];
+                    acc[0] |= (v0 >= 0.5f ? 1u : 0u) << r;
+                    if (CHECK) odd = odd || !(v0 == 0.0f || v0 == 1.0f);
                 }
             }
         }
@@ -78,7 +85,9 @@ __global__ __launch_bounds__(256) void dwn_pack_planes(const float *__restrict__
         for (int r = 0; r < rows; ++r) {
 #pragma unroll
             for (int v = 0; v < VEC; ++v) {
-                const unsigned bit = base[(size_t)r * I + v] >= 0.5f ? 1u : 0u;
+                const float val = base[(size_t)r * I + v];
+                const unsigned bit = val >= 0.5f ? 1u : 0u;
+                if (CHECK) odd = odd || !(val == 0.0f || val == 1.0f);
                 if (r < 32) lo[v] |= bit << r; else hi[v] |= bit << (r - 32);
             }
         }
@@ -86,6 +95,10 @@ __global__ __launch_bounds__(256) void dwn_pack_planes(const float *__restrict__
     u64 *out = planes + (size_t)t * I + i0;
 #pragma unroll
     for (int v = 0; v < VEC; ++v) out[v] = ((u64)hi[v] << 32) | lo[v];
+    if (CHECK && odd) *all_binary = 0;  // every writer stores the same value
+}
+__global__ void dwn_set_flag(int *flag, int value) {
+    if (threadIdx.x == 0) *flag = value;
 }
 
 // ---------------------------------------------------------------------------------
@@ -114,7 +127,8 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
                                                                const float *__restrict__ luts, float *__restrict__ y,
                                                                uint8_t *__restrict__ addrT, u64 *__restrict__ planes_out,
                                                                int B, int I, int N, int O, int BT, int gsize = 1,
-                                                               int slots = 1) {
+                                                               int slots = 1, const int *__restrict__ run_if_set = nullptr) {
+    if (EVAL && run_if_set && *run_if_set == 0) return;  // the inputs were not all 0/1: the generic kernel answers
     __shared__ float tile[DWN_TC][65];  // [column][row]
     __shared__ u64 plane_tile[CHAIN ? DWN_TC : 1];  // thresholded outputs of the tile's columns, one bit per row
     __shared__ float gpart[GSUM ? DWN_FW : 1][GSUM ? DWN_GS_SLOTS : 1][64];  // [wavefront][slot][row]
@@ -623,14 +637,14 @@ extern "C" size_t dl_dwn_bwd_workspace_bytes(int B, int I, int N, int k, int O) 
 template <int K>
 static void dwn_launch_lookup(const u64 *planes, const int *idx32, const float *luts, float *y, uint8_t *addrT,
                               u64 *planes_out, int B, int I, int N, int O, hipStream_t s, int gsize = 0, int slots = 0,
-                              bool eval = false) {
+                              bool eval = false, const int *run_if_set = nullptr) {
     const int BT = dwn_bt(B);
     const int grid = dl_xcd_grid(dl_ceil_div((long long)N * O, DWN_TC), BT);
     if (eval) {  // addrT is not written
 #define DWN_EVAL(O1_, CHAIN_, GSUM_)                                                                                     \
     DL_TIMED("dwn_lookup_eval", s, (dwn_lookup_fwd<K, O1_, CHAIN_, GSUM_, true><<<grid, 64 * DWN_FW, 0, s>>>(            \
                                        planes, idx32, luts, y, addrT, planes_out, B, I, N, O, BT, gsize > 0 ? gsize : 1, \
-                                       slots > 0 ? slots : 1)))
+                                       slots > 0 ? slots : 1, run_if_set)))
         if (gsize > 0 && O == 1) DWN_EVAL(true, false, true);
         else if (gsize > 0) DWN_EVAL(false, false, true);
         else if (O == 1) DWN_EVAL(true, true, false);
@@ -940,6 +954,43 @@ extern "C" int dl_dwn_layer_eval_planes(const void *planes_in, const int32_t *id
         default: dwn_launch_lookup<6>(planes, idx32, luts, y, none, po, B, I, N, O, s, 0, 0, true); break;
     }
     return dl_launch_status();
+}
+
+// Eval forward of one layer on [B, I] fp32 input, exact for any values: the input is packed into bit-planes while
+// being checked; if every value is 0 or 1 the bit-plane kernel answers, otherwise the generic one does (both are
+// launched, one of them returns at once - no host synchronisation).
+extern "C" size_t dl_dwn_eval_workspace_bytes(int B, int I, int N, int k, int O) {
+    return dwn_fast(N, k, O) && B > 0 && I > 0 ? dwn_planes_bytes(B, I) + 256 : 256;
+}
+extern "C" int dl_dwn_layer_eval_ws(const float *x, const int32_t *idx32, const float *luts, float *y, void *ws,
+                                    size_t ws_bytes, int B, int I, int N, int k, int O, void *stream) {
+    if (!x || !idx32 || !luts || !y) return DL_ERR_NULL;
+    int rc = dwn_check(B, I, N, k, O);
+    if (rc) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    if (!dwn_fast(N, k, O)) return dwn_generic_eval(x, idx32, luts, y, B, I, N, k, O, nullptr, s);
+    if (!ws) return DL_ERR_NULL;
+    if (ws_bytes < dl_dwn_eval_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
+    u64 *planes = (u64 *)ws;
+    int *flag = (int *)((char *)ws + dwn_planes_bytes(B, I));
+    const int BT = dwn_bt(B);
+    dwn_set_flag<<<1, 64, 0, s>>>(flag, 1);
+    if (I % 4 == 0 && ((uintptr_t)x & 15) == 0)
+        DL_TIMED("dwn_pack_planes", s,
+                 (dwn_pack_planes<4, true><<<dim3(dl_ceil_div(I, 1024), BT), 256, 0, s>>>(x, planes, B, I, flag)));
+    else
+        DL_TIMED("dwn_pack_planes", s,
+                 (dwn_pack_planes<1, true><<<dim3(dl_ceil_div(I, 256), BT), 256, 0, s>>>(x, planes, B, I, flag)));
+    uint8_t *none = (uint8_t *)const_cast<float *>(luts);
+    switch (k) {
+        case 1: dwn_launch_lookup<1>(planes, idx32, luts, y, none, nullptr, B, I, N, O, s, 0, 0, true, flag); break;
+        case 2: dwn_launch_lookup<2>(planes, idx32, luts, y, none, nullptr, B, I, N, O, s, 0, 0, true, flag); break;
+        case 3: dwn_launch_lookup<3>(planes, idx32, luts, y, none, nullptr, B, I, N, O, s, 0, 0, true, flag); break;
+        case 4: dwn_launch_lookup<4>(planes, idx32, luts, y, none, nullptr, B, I, N, O, s, 0, 0, true, flag); break;
+        case 5: dwn_launch_lookup<5>(planes, idx32, luts, y, none, nullptr, B, I, N, O, s, 0, 0, true, flag); break;
+        default: dwn_launch_lookup<6>(planes, idx32, luts, y, none, nullptr, B, I, N, O, s, 0, 0, true, flag); break;
+    }
+    return dwn_generic_eval(x, idx32, luts, y, B, I, N, k, O, flag, s);
 }
 
 extern "C" int dl_dwn_layer_eval_planes_groups(const void *planes_in, const int32_t *idx32, const float *luts,

@@ -337,8 +337,11 @@ def dwn_layer_eval(x, luts, plan):
     B, I = x.shape
     N, O, _ = luts.shape
     y = torch.empty((B, N * O), dtype=torch.float32, device=x.device)
-    nat.check(nat.lib().dl_dwn_layer_eval(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(luts), nat.ptr(y), B, I, N, plan.k, O,
-                                          nat.stream()))
+    lib = nat.lib()
+    dims = (B, I, N, plan.k, O)
+    ws = _bytes(lib.dl_dwn_eval_workspace_bytes(*dims), x.device)
+    nat.check(lib.dl_dwn_layer_eval_ws(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(luts), nat.ptr(y), nat.ptr(ws), ws.numel(),
+                                       *dims, nat.stream()))
     return y
 
 

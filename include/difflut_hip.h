@@ -124,6 +124,12 @@ int dl_dwn_layer_bwd_groups(const void *saved, const int32_t *inv_ptr, const int
                             const float *glogits, int groups, float tau, float alpha, float beta,
                             float *gx, int gx_tiled, float *gluts, void *ws, size_t ws_bytes,
                             int B, int I, int N, int k, int O, void *stream);
+/* The eval forward below with a workspace (dl_dwn_eval_workspace_bytes): the same result for any input, and
+ * the bit-plane kernels' speed when every input value is exactly 0 or 1 (checked on the device while packing;
+ * no host synchronisation - both kernels are launched and one returns at once). */
+size_t dl_dwn_eval_workspace_bytes(int B, int I, int N, int k, int O);
+int dl_dwn_layer_eval_ws(const float *x, const int32_t *idx32, const float *luts, float *y, void *ws,
+                         size_t ws_bytes, int B, int I, int N, int k, int O, void *stream);
 /* Inference on binary activations (DWNNode.forward_eval, dwn_node.py:457-483, for inputs that are exactly
  * 0 or 1 - what a thermometer encoder or a preceding layer's eval output delivers; there its address
  * floor(sum_j x_j 2^j) equals the thresholded one).  planes_in as dl_dwn_pack_planes /

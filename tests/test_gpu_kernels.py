@@ -138,6 +138,31 @@ def test_dwn_eval_forward(shape):
         assert np.array_equal(y[:, n], orc.dwn_eval_forward(m[:, n], luts[n]))
 
 
+@pytest.mark.parametrize("shape", [(130, 40, 150, 6, 1), (64, 36, 70, 4, 2), (257, 33, 129, 5, 1)])
+def test_dwn_eval_forward_any_input_values(shape):
+    """The eval entry point with a workspace answers through the bit-plane kernels when every input is 0 or 1 and
+    through the literal float address otherwise; both against the oracle, including inputs where the two
+    addresses differ (0.7 counts as 0.7 * 2^j, not as a set bit) and a single odd value in a binary batch."""
+    ops = _ops()
+    B, I, N, k, O = shape
+    xb, idx, luts, _ = make_case(11, *shape, lo=0.0, hi=1.0, binary=True)
+    rng = np.random.default_rng(5)
+    xf = rng.random((B, I)).astype(np.float32) * 1.2          # arbitrary values, some above 1
+    xo = xb.copy()
+    xo[B // 2, idx[N // 2, 0]] = 0.25                          # one value that is neither 0 nor 1
+    plan = ops.MappingPlan(dev(idx, torch.int32), I)
+    for x in (xb, xf, xo, xb):                                 # the flag is reset on every call
+        y = ops.dwn_layer_eval(dev(x), dev(luts), plan).cpu().numpy().reshape(B, N, O)
+        m = orc.gather_forward(x, idx)
+        L = 1 << k
+        for n in range(N):
+            addr = (m[:, n] * (2.0 ** np.arange(k)).astype(np.float32)).sum(-1, dtype=np.float32).astype(np.int64)
+            want = (luts[n][:, np.clip(addr, 0, L - 1)].T >= np.float32(0.5)).astype(np.float32)  # clamped like the kernel
+            assert np.array_equal(y[:, n], want)
+            if x is not xf:
+                assert np.array_equal(want, orc.dwn_eval_forward(m[:, n], luts[n]))
+
+
 @pytest.mark.parametrize("tag", ["k6o2", "k4o1", "k2o3"])
 def test_dwn_node_against_reference_vectors(golden, tag):
     """Same inputs the reference's own CPU path was run on (tests/golden)."""
