@@ -49,6 +49,8 @@ SIGNATURES = {
     "dl_prob_bwd_workspace_bytes": (_Z, [_I] * 5),
     "dl_prob_layer_fwd": (_I, [_P, _P, _P, _F, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
     "dl_prob_layer_bwd": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
+    "dl_prob_eval_workspace_bytes": (_Z, [_I] * 5),
+    "dl_prob_layer_eval_ws": (_I, [_P, _P, _P, _F, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
     "dl_prob_layer_eval": (_I, [_P, _P, _P, _F, _P, _I, _I, _I, _I, _I, _P]),
     "dl_soft_map_saved_bytes": (_Z, [_I] * 4),
     "dl_soft_map_workspace_bytes": (_Z, [_I] * 4),

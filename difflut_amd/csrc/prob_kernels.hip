@@ -651,6 +651,37 @@ extern "C" int dl_hybrid_layer_bwd(const float *x, const int32_t *idx32, const i
     return dl_launch_status();
 }
 
+// Eval forward with a workspace: the binarised sigmoid table of every node is the table of a DWN layer, so the
+// DWN eval path (bit-planes when every input is 0 or 1, the literal float address otherwise) answers.
+extern "C" size_t dl_dwn_eval_workspace_bytes(int B, int I, int N, int k, int O);
+extern "C" int dl_dwn_layer_eval_ws(const float *x, const int32_t *idx32, const float *luts, float *y, void *ws,
+                                    size_t ws_bytes, int B, int I, int N, int k, int O, void *stream);
+static inline size_t prob_eval_table_bytes(int N, int k, int O) { return dl_align256((size_t)N * O * ((size_t)1 << k) * 4); }
+extern "C" size_t dl_prob_eval_workspace_bytes(int B, int I, int N, int k, int O) {
+    if (B <= 0 || I <= 0 || N <= 0 || k <= 0 || O <= 0 || k > DL_MAX_FAST_K) return 256;
+    return prob_eval_table_bytes(N, k, O) + dl_dwn_eval_workspace_bytes(B, I, N, k, O);
+}
+extern "C" int dl_prob_layer_eval_ws(const float *x, const int32_t *idx32, const float *raw_w, float temperature, float *y,
+                                     void *ws, size_t ws_bytes, int B, int I, int N, int k, int O, void *stream) {
+    if (!x || !idx32 || !raw_w || !y) return DL_ERR_NULL;
+    int rc = prob_check(B, I, N, k, O);
+    if (rc) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    if (k > DL_MAX_FAST_K) {
+        DL_TIMED("prob_eval_kernel", s, (prob_eval_kernel<<<dl_ceil_div((long long)B * N * O, 256), 256, 0, s>>>(
+                                            x, idx32, raw_w, prob_inv_t(temperature), y, B, I, N, k, O)));
+        return dl_launch_status();
+    }
+    if (!ws) return DL_ERR_NULL;
+    if (ws_bytes < dl_prob_eval_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
+    float *sig = (float *)ws;
+    const int L = 1 << k;
+    DL_TIMED("prob_sig_table", s, (prob_sig_table<<<dl_ceil_div((long long)N * L * O, 256), 256, 0, s>>>(
+                                      raw_w, prob_inv_t(temperature), sig, N, L, O)));
+    const size_t tb = prob_eval_table_bytes(N, k, O);
+    return dl_dwn_layer_eval_ws(x, idx32, sig, y, (char *)ws + tb, ws_bytes - tb, B, I, N, k, O, stream);
+}
+
 extern "C" int dl_prob_layer_eval(const float *x, const int32_t *idx32, const float *raw_w, float temperature, float *y,
                                   int B, int I, int N, int k, int O, void *stream) {
     if (!x || !idx32 || !raw_w || !y) return DL_ERR_NULL;

@@ -494,8 +494,11 @@ def prob_layer_eval(x, raw, plan, temperature):
     B, I = x.shape
     N, _, O = raw.shape
     y = torch.empty((B, N * O), dtype=torch.float32, device=x.device)
-    nat.check(nat.lib().dl_prob_layer_eval(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(raw), float(temperature),
-                                           nat.ptr(y), B, I, N, plan.k, O, nat.stream()))
+    lib = nat.lib()
+    dims = (B, I, N, plan.k, O)
+    ws = _bytes(lib.dl_prob_eval_workspace_bytes(*dims), x.device)
+    nat.check(lib.dl_prob_layer_eval_ws(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(raw), float(temperature), nat.ptr(y),
+                                        nat.ptr(ws), ws.numel(), *dims, nat.stream()))
     return y
 
 

@@ -220,6 +220,12 @@ int dl_prob_layer_bwd(const float *x, const void *saved, const int32_t *idx32,
 /* Eval forward (probabilistic_node.py:302-328): y = (sigmoid(raw_w[n,addr,d]/T) >= 0.5). */
 int dl_prob_layer_eval(const float *x, const int32_t *idx32, const float *raw_w, float temperature,
                        float *y, int B, int I, int N, int k, int O, void *stream);
+/* The same with a workspace (dl_prob_eval_workspace_bytes): the binarised sigmoid tables are looked up through
+ * the DWN eval path, i.e. through bit-planes when every input value is exactly 0 or 1 (decided on the device,
+ * same result for any input). */
+size_t dl_prob_eval_workspace_bytes(int B, int I, int N, int k, int O);
+int dl_prob_layer_eval_ws(const float *x, const int32_t *idx32, const float *raw_w, float temperature, float *y,
+                          void *ws, size_t ws_bytes, int B, int I, int N, int k, int O, void *stream);
 
 /* ------------------------------------------------------------------------
  * LearnableLayer soft connectivity (training) and hard selection (eval).

@@ -163,6 +163,38 @@ def test_dwn_eval_forward_any_input_values(shape):
                 assert np.array_equal(want, orc.dwn_eval_forward(m[:, n], luts[n]))
 
 
+@pytest.mark.parametrize("shape", [(130, 40, 150, 4, 1), (64, 36, 70, 6, 2), (200, 33, 90, 3, 1)])
+def test_prob_eval_forward_any_input_values(shape):
+    """Probabilistic eval through the workspace entry point (binarised sigmoid table looked up by the DWN eval
+    path) against the oracle, for 0/1 inputs (bit-plane kernels), arbitrary inputs and a single odd value
+    (generic kernel), and against the entry point without a workspace."""
+    from difflut_amd import _native as nat
+    ops = _ops()
+    B, I, N, k, O = shape
+    rng = np.random.default_rng(21)
+    idx = orc.random_mapping(I, N, k, seed=4).numpy().astype(np.int64)
+    raw = rng.standard_normal((N, 1 << k, O)).astype(np.float32)
+    raw[0, 0, 0] = 0.0                                         # sigmoid(0) = 0.5 counts as 1
+    xb = rng.integers(0, 2, (B, I)).astype(np.float32)
+    xf = rng.random((B, I)).astype(np.float32)
+    xo = xb.copy()
+    xo[3, idx[1, 0]] = 0.5
+    plan = ops.MappingPlan(dev(idx, torch.int32), I)
+    lib = nat.lib()
+    rawd = dev(raw)
+    for x in (xb, xf, xo):
+        xd = dev(x)
+        y = ops.prob_layer_eval(xd, rawd, plan, 0.7)
+        plain = torch.empty_like(y)
+        nat.check(lib.dl_prob_layer_eval(xd.data_ptr(), plan.idx32.data_ptr(), rawd.data_ptr(), 0.7, plain.data_ptr(),
+                                         B, I, N, k, O, nat.stream()))
+        assert torch.equal(y, plain)
+        m = orc.gather_forward(x, idx)
+        got = y.cpu().numpy().reshape(B, N, O)
+        for n in range(N):
+            assert np.array_equal(got[:, n], orc.prob_eval_forward(m[:, n], raw[n], 0.7))
+
+
 @pytest.mark.parametrize("tag", ["k6o2", "k4o1", "k2o3"])
 def test_dwn_node_against_reference_vectors(golden, tag):
     """Same inputs the reference's own CPU path was run on (tests/golden)."""
