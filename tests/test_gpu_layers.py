@@ -420,6 +420,61 @@ def test_dwn_stack_with_thermometer_encoder(case):
     assert torch.equal(stack(x), he)
 
 
+def test_full_size_deep_stack_b8192():
+    """The deep-stack configuration at its full size (8192 x 784 -> thermometer 4 bits -> 16000/8000/4000/2000
+    DWN k=6 nodes -> GroupSum 10 -> cross-entropy): the chained run against the layers one by one (logits and
+    loss to rtol 1e-5, every table gradient to rtol 1e-5 with a floor of a few ulps of its scale), two chained
+    runs bit-identical in the logits, conservation of each table's gradient mass, and eval mode chained ==
+    eval mode layer by layer, bit for bit."""
+    REGISTRY, NodeConfig, _, _ = _api()
+    from difflut_amd.layers import DWNStack
+    from difflut_amd.utils import GroupSum
+    B, F, k = 8192, 784, 6
+    widths = [16000, 8000, 4000, 2000]
+    torch.manual_seed(0)
+    x = torch.rand(B, F, device="cuda")
+    labels = torch.randint(0, 10, (B,), device="cuda")
+    enc = REGISTRY.build_encoder("thermometer", num_bits=4).fit(x)
+    layers, width = [], F * 4
+    for n in widths:
+        layers.append(REGISTRY.get_layer("random")(width, n, REGISTRY.get_node("dwn"),
+                                                   NodeConfig(input_dim=k, output_dim=1), seed=42).cuda())
+        width = n
+    head = GroupSum(k=10, tau=1.0, use_randperm=False)
+    h = enc.encode(x)
+    for layer in layers:
+        h = layer(h)
+    logits = head(h)
+    loss = torch.nn.functional.cross_entropy(logits, labels)
+    loss.backward()
+    want_gl = [layer._banks["luts"].flat.grad.clone() for layer in layers]
+    for layer in layers:
+        layer._banks["luts"].flat.grad = None
+    stack = DWNStack(layers, encoder=enc, head=head).train()
+    got = stack(x)
+    torch.testing.assert_close(got.detach(), logits.detach(), rtol=1e-5, atol=1e-4)
+    loss2 = torch.nn.functional.cross_entropy(got, labels)
+    torch.testing.assert_close(loss2.detach(), loss.detach(), rtol=1e-5, atol=0)
+    loss2.backward()
+    for layer, want in zip(layers, want_gl):
+        g = layer._banks["luts"].flat.grad
+        torch.testing.assert_close(g, want, rtol=1e-5, atol=float(want.abs().max()) * 4e-6)
+    assert torch.equal(stack(x).detach(), got.detach())
+    # the last layer's table gradient: every node's bins add up to the sum of its output gradient over the batch
+    p = torch.softmax(got.detach().double(), dim=1)
+    p[torch.arange(B), labels] -= 1.0
+    per_group = (p / B).sum(0)                                  # d loss / d logit, summed over the batch
+    mass = layers[-1]._banks["luts"].flat.grad.double().view(widths[-1], -1).sum(1)
+    torch.testing.assert_close(mass, per_group.repeat_interleave(widths[-1] // 10), rtol=1e-4, atol=1e-7)
+    # inference
+    stack.eval()
+    he = enc.encode(x)
+    for layer in layers:
+        layer.eval()
+        he = layer(he)
+    assert torch.equal(stack(x), head(he))
+
+
 @pytest.mark.parametrize("case", [(130, 37, [60, 640], 6, 10, 1.0), (64, 100, [2000], 6, 10, 2.5), (700, 50, [300, 768], 4, 3, 0.5),
                                   (65, 30, [90, 130], 5, 2, 1.0), (256, 64, [512], 6, 8, 1.0), (33, 40, [1000], 6, 7, 1.0),
                                   (100, 48, [70, 192], 4, 3, 1.0, 2)])
