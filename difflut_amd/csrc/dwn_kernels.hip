@@ -462,6 +462,69 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
     for (int e = threadIdx.x; e < cend * L; e += 256) atomicAdd(&gluts[(size_t)c0 * L + e], hist[e / L][e % L]);
 }
 
+// hist_tiled: the histogram alone, for gy that arrives tile-major ([B/64][N*O][64]).  Nothing has to be
+// transposed then: lane = (column, quarter), a quad covers one column, and lane `hr` of the quad loads the
+// 16-byte pieces 4m + hr (m = 0..3) of the column's 256 bytes, i.e. rows 16m + 4hr + e, together with the four
+// address bytes of the same rows (one 32-bit load per m).  Step (m, e) then adds four rows per column with the
+// quad merge of transpose_hist; no LDS tile, no block barrier inside the tile loop.
+__global__ __launch_bounds__(256) void dwn_bwd_hist_tiled(const float *__restrict__ gy, const uint8_t *__restrict__ addrT,
+                                                           float *__restrict__ gluts, int NO, int O, int L, int BT,
+                                                           int tiles_per_chunk) {
+    __shared__ float hist[DWN_HC][65];  // [column][bin]
+    const int c0 = blockIdx.x * DWN_HC;
+    const int lane = threadIdx.x & 63;
+    const int wave = dl_uniform(threadIdx.x >> 6);
+    const int cend = min(DWN_HC, NO - c0);
+    for (int e = threadIdx.x; e < DWN_HC * 65; e += 256) (&hist[0][0])[e] = 0.0f;
+    __syncthreads();
+    const int t_begin = blockIdx.y * tiles_per_chunk;
+    const int t_end = min(BT, t_begin + tiles_per_chunk);
+    const int hc = wave * (DWN_HC / 4) + (lane >> 2), hr = lane & 3;
+    const int N = NO / O;
+    if (hc < cend && t_begin < t_end) {  // whole quads share hc
+        const int c = c0 + hc;
+        const float *gcol = gy + (size_t)c * 64 + hr * 4;
+        const uint8_t *acol = addrT + (size_t)(c / O) * 64 + hr * 4;
+        float4 g[4], gn[4];
+        unsigned aw[4], awn[4];
+        auto fetch = [&](int t, float4 (&gg)[4], unsigned (&aa)[4]) {
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                gg[m] = *reinterpret_cast<const float4 *>(gcol + (size_t)t * NO * 64 + m * 16);
+                aa[m] = *reinterpret_cast<const unsigned *>(acol + (size_t)t * N * 64 + m * 16);
+            }
+        };
+        fetch(t_begin, g, aw);
+        for (int t = t_begin; t < t_end; ++t) {
+            if (t + 1 < t_end) fetch(t + 1, gn, awn);
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                const float vs[4] = {g[m].x, g[m].y, g[m].z, g[m].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float v = vs[e];
+                    const unsigned a = (aw[m] >> (8 * e)) & 0xffu;
+                    float sum = v;
+                    bool leader = true;
+                    const unsigned a1 = (unsigned)dwn_quad_xor<1>((int)a), a2 = (unsigned)dwn_quad_xor<2>((int)a),
+                                   a3 = (unsigned)dwn_quad_xor<3>((int)a);
+                    const float v1 = __int_as_float(dwn_quad_xor<1>(__float_as_int(v))),
+                                v2 = __int_as_float(dwn_quad_xor<2>(__float_as_int(v))),
+                                v3 = __int_as_float(dwn_quad_xor<3>(__float_as_int(v)));
+                    if (a1 == a) { sum += v1; leader = leader && (hr ^ 1) > hr; }
+                    if (a2 == a) { sum += v2; leader = leader && (hr ^ 2) > hr; }
+                    if (a3 == a) { sum += v3; leader = leader && (hr ^ 3) > hr; }
+                    if (leader) hist[hc][a] += sum;
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < 4; ++m) { g[m] = gn[m]; aw[m] = awn[m]; }
+        }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < cend * L; e += 256) atomicAdd(&gluts[(size_t)c0 * L + e], hist[e / L][e % L]);
+}
+
 // ---------------------------------------------------------------------------------
 // bwd_gx: one block per (64-input slab, 64-row batch tile), 256 threads, lane = batch row.  A wavefront
 // owns 16 consecutive inputs, i.e. one contiguous run of CSR entries.  The run is read 64 entries
@@ -760,8 +823,8 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
                                                   gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc, head->groups,
                                                   head->gsize, head->inv_tau)));
     else if (gy_tiled)
-        DL_TIMED("dwn_bwd_hist_tiled", s, (dwn_bwd_transpose_hist<false, true><<<hgrid, 256, 0, s>>>(
-                                              gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc)));
+        DL_TIMED("dwn_bwd_hist_tiled", s,
+                 (dwn_bwd_hist_tiled<<<hgrid, 256, 0, s>>>(gy, addrT, gluts, (int)NO, O, L, BT, tpc)));
     else if (gx)
         DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<true><<<hgrid, 256, 0, s>>>(
                                                   gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc)));
