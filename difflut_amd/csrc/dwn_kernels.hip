@@ -349,16 +349,11 @@ __device__ __forceinline__ int dwn_quad_xor(int v) {
     constexpr int ctrl = X == 1 ? 0xB1 : (X == 2 ? 0x4E : 0x1B);  // quad_perm [1,0,3,2] / [2,3,0,1] / [3,2,1,0]
     return __builtin_amdgcn_update_dpp(0, v, ctrl, 0xf, 0xf, true);
 }
-// IN_T: gy arrives tile-major already ([B/64][N*O][64], e.g. the input gradient a following layer
-// wrote in that form); only the histogram is left to do.
-// GROUPS: gy is the gradient of a GroupSum head, [B][groups]: column c takes gy[b][c / gsize] * inv_tau,
-// so the [B, N*O] gradient of the layer's output is never written.
-template <bool WRITE_T, bool IN_T = false, bool GROUPS = false>
+template <bool WRITE_T>
 __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__restrict__ gy, const uint8_t *__restrict__ addrT,
                                                                float *__restrict__ gyT, float *__restrict__ gluts,
                                                                int B, int NO, int O, int L, int BP, int BT,
-                                                               int tiles_per_chunk, int groups = 0, int gsize = 1,
-                                                               float inv_tau = 1.0f) {
+                                                               int tiles_per_chunk) {
     __shared__ float tile[64][DWN_HC + 1];       // [row][column]
     __shared__ float hist[DWN_HC][65];           // [column][bin]
     __shared__ uint8_t atile[DWN_HC][64 + 4];    // [column][row] addresses
@@ -375,29 +370,12 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
     const int wc0 = wave * (DWN_HC / 4);  // my wavefront's first column
     float4 pre[4];
     unsigned apre[DWN_HC / 4];  // addresses of my 16 columns for the tile being fetched (lane = row)
-    const int tc = threadIdx.x >> 4, tr = (threadIdx.x & 15) * 4;  // IN_T: my column in a pass of 16, my 4 rows
-    int grp[4] = {0, 0, 0, 0};  // GROUPS: the groups of my four columns
-    if (GROUPS) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) grp[i] = min(c0 + q * 4 + i, NO - 1) / gsize;
-    }
     auto fetch = [&](int t) {
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
             const int b = t * 64 + rr + 16 * p;
             pre[p] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (IN_T) {  // 16 threads x 16 B = the 256 contiguous bytes of one column
-                if (tc + 16 * p < cend)
-                    pre[p] = *reinterpret_cast<const float4 *>(gy + ((size_t)t * NO + c0 + tc + 16 * p) * 64 + tr);
-            } else if (GROUPS) {
-                if (b < B) {
-                    const float *src = gy + (size_t)b * groups;
-                    if (q * 4 + 0 < cend) pre[p].x = src[grp[0]] * inv_tau;
-                    if (q * 4 + 1 < cend) pre[p].y = src[grp[1]] * inv_tau;
-                    if (q * 4 + 2 < cend) pre[p].z = src[grp[2]] * inv_tau;
-                    if (q * 4 + 3 < cend) pre[p].w = src[grp[3]] * inv_tau;
-                }
-            } else if (b < B) {
+            if (b < B) {
                 const float *src = gy + (size_t)b * NO + c0 + q * 4;
                 if (vec4) {
                     pre[p] = *reinterpret_cast<const float4 *>(src);
@@ -421,13 +399,8 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
         __syncthreads();  // previous tile fully consumed (and hist cleared on the first pass)
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
-            if (IN_T) {
-                tile[tr][tc + 16 * p] = pre[p].x; tile[tr + 1][tc + 16 * p] = pre[p].y;
-                tile[tr + 2][tc + 16 * p] = pre[p].z; tile[tr + 3][tc + 16 * p] = pre[p].w;
-            } else {
-                float *dst = &tile[rr + 16 * p][q * 4];
-                dst[0] = pre[p].x; dst[1] = pre[p].y; dst[2] = pre[p].z; dst[3] = pre[p].w;
-            }
+            float *dst = &tile[rr + 16 * p][q * 4];
+            dst[0] = pre[p].x; dst[1] = pre[p].y; dst[2] = pre[p].z; dst[3] = pre[p].w;
         }
 #pragma unroll
         for (int u = 0; u < DWN_HC / 4; ++u) atile[wc0 + u][lane] = (uint8_t)apre[u];
@@ -467,9 +440,13 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
 // 16-byte pieces 4m + hr (m = 0..3) of the column's 256 bytes, i.e. rows 16m + 4hr + e, together with the four
 // address bytes of the same rows (one 32-bit load per m).  Step (m, e) then adds four rows per column with the
 // quad merge of transpose_hist; no LDS tile, no block barrier inside the tile loop.
+// GROUPS: gy is the [B][groups] gradient of a GroupSum head instead (column c takes gy[b][c / gsize] * inv_tau);
+// the tile-major gradient is then written to gyT (when non-null) for the gather that follows.
+template <bool GROUPS = false>
 __global__ __launch_bounds__(256) void dwn_bwd_hist_tiled(const float *__restrict__ gy, const uint8_t *__restrict__ addrT,
                                                            float *__restrict__ gluts, int NO, int O, int L, int BT,
-                                                           int tiles_per_chunk) {
+                                                           int tiles_per_chunk, float *__restrict__ gyT = nullptr, int B = 0,
+                                                           int groups = 0, int gsize = 1, float inv_tau = 1.0f) {
     __shared__ float hist[DWN_HC][65];  // [column][bin]
     const int c0 = blockIdx.x * DWN_HC;
     const int lane = threadIdx.x & 63;
@@ -487,10 +464,21 @@ __global__ __launch_bounds__(256) void dwn_bwd_hist_tiled(const float *__restric
         const uint8_t *acol = addrT + (size_t)(c / O) * 64 + hr * 4;
         float4 g[4], gn[4];
         unsigned aw[4], awn[4];
+        const int grp = GROUPS ? c / gsize : 0;
         auto fetch = [&](int t, float4 (&gg)[4], unsigned (&aa)[4]) {
 #pragma unroll
             for (int m = 0; m < 4; ++m) {
-                gg[m] = *reinterpret_cast<const float4 *>(gcol + (size_t)t * NO * 64 + m * 16);
+                if (GROUPS) {
+                    const int b = t * 64 + m * 16 + hr * 4;  // my four rows of this piece
+                    const float *src = gy + (size_t)b * groups + grp;
+                    gg[m].x = b + 0 < B ? src[0] * inv_tau : 0.0f;
+                    gg[m].y = b + 1 < B ? src[groups] * inv_tau : 0.0f;
+                    gg[m].z = b + 2 < B ? src[2 * groups] * inv_tau : 0.0f;
+                    gg[m].w = b + 3 < B ? src[3 * groups] * inv_tau : 0.0f;
+                    if (gyT) *reinterpret_cast<float4 *>(gyT + ((size_t)t * NO + c) * 64 + hr * 4 + m * 16) = gg[m];
+                } else {
+                    gg[m] = *reinterpret_cast<const float4 *>(gcol + (size_t)t * NO * 64 + m * 16);
+                }
                 aa[m] = *reinterpret_cast<const unsigned *>(acol + (size_t)t * N * 64 + m * 16);
             }
         };
@@ -814,17 +802,13 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
                  (dwn_efd_table<<<dl_ceil_div(NO, 4), 256, 0, s>>>(luts, D, gluts, (int)NO, k, alpha, beta, sform ? 1 : 0)));
     else
         dl_fill_zero(gluts, NO * L, s);
-    if (head && gx)
-        DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<true, false, true><<<hgrid, 256, 0, s>>>(
-                                                  gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc, head->groups,
-                                                  head->gsize, head->inv_tau)));
-    else if (head)
-        DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<false, false, true><<<hgrid, 256, 0, s>>>(
-                                                  gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc, head->groups,
-                                                  head->gsize, head->inv_tau)));
+    if (head)
+        DL_TIMED("dwn_bwd_hist_groups", s, (dwn_bwd_hist_tiled<true><<<hgrid, 256, 0, s>>>(
+                                               gy, addrT, gluts, (int)NO, O, L, BT, tpc, gx ? gyT : nullptr, B, head->groups,
+                                               head->gsize, head->inv_tau)));
     else if (gy_tiled)
         DL_TIMED("dwn_bwd_hist_tiled", s,
-                 (dwn_bwd_hist_tiled<<<hgrid, 256, 0, s>>>(gy, addrT, gluts, (int)NO, O, L, BT, tpc)));
+                 (dwn_bwd_hist_tiled<false><<<hgrid, 256, 0, s>>>(gy, addrT, gluts, (int)NO, O, L, BT, tpc)));
     else if (gx)
         DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<true><<<hgrid, 256, 0, s>>>(
                                                   gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc)));
