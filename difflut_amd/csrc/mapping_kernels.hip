@@ -60,9 +60,10 @@ __global__ __launch_bounds__(256) void thermometer_kernel(const float *__restric
 
 // Thermometer bits as bit-planes for a following DWN layer: word (t, f*nbits + j) holds, in bit r,
 // (x[64t + r][f] > thr[f][j]).  Block = (64 features, batch tile t): the x tile is read row-wise
-// (coalesced) into LDS, then each wavefront takes 16 features with lane = row, one ballot per
-// threshold.  A lane keeps the words whose index is congruent to it and the wavefront stores 64
-// consecutive words at a time.  Rows past B read as "not greater".
+// (coalesced) into LDS; then every thread builds whole output words, one (feature, threshold) pair at a
+// time, by walking the 64 rows of its feature in LDS (lanes of one feature read the same word: a
+// broadcast; different features sit in different banks).  Consecutive threads hold consecutive words, so
+// the stores are contiguous.  Rows past B read as "not greater".
 __global__ __launch_bounds__(256) void thermometer_planes_kernel(const float *__restrict__ x, const float *__restrict__ thr,
                                                                   unsigned long long *__restrict__ planes, int B, int F,
                                                                   int nbits) {
@@ -74,27 +75,19 @@ __global__ __launch_bounds__(256) void thermometer_planes_kernel(const float *__
         tile[c][r] = (b < B && f0 + c < F) ? x[(size_t)b * F + f0 + c] : -INFINITY;
     }
     __syncthreads();
-    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int fbeg = f0 + w * 16, fend = min(F, fbeg + 16);
-    if (fbeg >= fend) return;
-    const int words = (fend - fbeg) * nbits;
-    unsigned long long *out = planes + (size_t)t * F * nbits + (size_t)fbeg * nbits;
-    const float *th = thr + (size_t)fbeg * nbits;
-    float mythr = 0.0f;  // one threshold per lane for the current run of 64 words, handed round below
-    unsigned long long mine = 0;
-    int q = 0;
-    for (int ff = 0; ff < fend - fbeg; ++ff) {
-        const float v = tile[w * 16 + ff][lane];
-        for (int j = 0; j < nbits; ++j, ++q) {
-            const int slot = q & 63;
-            if (slot == 0) mythr = q + lane < words ? th[q + lane] : 0.0f;
-            const float t_q = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mythr), slot));
-            const unsigned long long mask = __ballot(v > t_q);  // strict compare, as the encoder
-            if (slot == lane) mine = mask;
-            if (slot == 63 || q == words - 1) {
-                if (lane <= slot) out[q - slot + lane] = mine;
-            }
+    const int words = min(64, F - f0) * nbits;
+    const float *th = thr + (size_t)f0 * nbits;
+    unsigned long long *out = planes + ((size_t)t * F + f0) * nbits;
+    for (int w = threadIdx.x; w < words; w += 256) {
+        const float *row = tile[w / nbits];
+        const float limit = th[w];
+        unsigned lo = 0u, hi = 0u;
+#pragma unroll
+        for (int r = 0; r < 32; ++r) {
+            lo |= (row[r] > limit ? 1u : 0u) << r;  // strict compare, as the encoder
+            hi |= (row[r + 32] > limit ? 1u : 0u) << r;
         }
+        out[w] = ((unsigned long long)hi << 32) | lo;
     }
 }
 
