@@ -520,32 +520,33 @@ __global__ __launch_bounds__(256) void dwn_bwd_hist_tiled(const float *__restric
 // per step with wave-uniform addressing: the 8 x 3 vector loads of a step are requested together,
 // then evaluated.  The entries of one input are consecutive, so its sum is
 // kept in a register and written to the LDS tile once, in CSR order (reproducible sums).
-#define DWN_IS 64
-#define DWN_WI (DWN_IS / 4)  // inputs per wavefront
+#define DWN_WI 16        // inputs per wavefront (slab of 64 inputs per block)
+#define DWN_WI_SMALL 4   // for layers with long CSR lists per input: slabs of 16 inputs
 #define DWN_EG 8
-template <int K, bool O1, bool SFORM>
+template <int K, bool O1, bool SFORM, int WI = DWN_WI>
 __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT, const uint8_t *__restrict__ addrT,
                                                    const float *__restrict__ D, const int *__restrict__ inv_ptr,
                                                    const int *__restrict__ inv_pos, float *__restrict__ gx,
                                                    int B, int I, int N, int O, int BT, int out_tiled) {
-    __shared__ float tile[DWN_IS][65];  // [input][row]
+    constexpr int IS = 4 * WI;  // inputs per block
+    __shared__ float tile[IS][65];  // [input][row]
     constexpr int Lh = 1 << (K - 1);
     int slab, t;
-    if (!dl_xcd_map((I + DWN_IS - 1) / DWN_IS, BT, slab, t)) return;
-    const int i0 = slab * DWN_IS;
+    if (!dl_xcd_map((I + IS - 1) / IS, BT, slab, t)) return;
+    const int i0 = slab * IS;
     const int NO = N * O;
     const int lane = threadIdx.x & 63;
     const int wave = dl_uniform(threadIdx.x >> 6);
-    const int iend = min(DWN_IS, I - i0);
+    const int iend = min(IS, I - i0);
     const uint8_t *addr_t = addrT + (size_t)t * N * 64 + lane;
     const float *gy_t = gyT + (size_t)t * NO * 64 + lane;
-    const int wbeg = wave * DWN_WI;
-    // CSR pointers of my inputs: lane l (0..DWN_WI) holds inv_ptr[first + l], clamped at I
-    const int myptr = inv_ptr[min(i0 + wbeg + min(lane, DWN_WI), I)];
+    const int wbeg = wave * WI;
+    // CSR pointers of my inputs: lane l (0..WI) holds inv_ptr[first + l], clamped at I
+    const int myptr = inv_ptr[min(i0 + wbeg + min(lane, WI), I)];
 #pragma unroll
-    for (int r = 0; r < DWN_WI; ++r) tile[wbeg + r][lane] = 0.0f;  // inputs nobody reads keep 0
+    for (int r = 0; r < WI; ++r) tile[wbeg + r][lane] = 0.0f;  // inputs nobody reads keep 0
     const int ebeg = __builtin_amdgcn_readlane(myptr, 0);
-    const int eend = __builtin_amdgcn_readlane(myptr, DWN_WI);
+    const int eend = __builtin_amdgcn_readlane(myptr, WI);
     struct Group {
         int rj[DWN_EG], ri[DWN_EG];
         bool live[DWN_EG];
@@ -560,7 +561,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT,
         const int p = valid ? inv_pos[e] : 0;
         int ii = 0;  // local input of entry e = number of my inputs that end at or before e
 #pragma unroll
-        for (int l = 1; l <= DWN_WI; ++l) ii += (__builtin_amdgcn_readlane(myptr, l) <= e) ? 1 : 0;
+        for (int l = 1; l <= WI; ++l) ii += (__builtin_amdgcn_readlane(myptr, l) <= e) ? 1 : 0;
         const int n = p / K, j = p - n * K;
         const int rec = valid ? ((n << 8) | (j << 5) | ii) : -1;
         const int cnt = min(64, eend - base);
@@ -635,14 +636,14 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT,
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int r = 0; r < DWN_WI; ++r)
+        for (int r = 0; r < WI; ++r)
             if (wbeg + r < iend)  // streamed past the L2, which holds the rows the gather re-reads
                 __builtin_nontemporal_store(tile[wbeg + r][lane], &gx[((size_t)t * I + i0 + wbeg + r) * 64 + lane]);
         return;
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < 64 * DWN_IS; e += 256) {
-        const int r = e / DWN_IS, ii = e % DWN_IS;
+    for (int e = threadIdx.x; e < 64 * IS; e += 256) {
+        const int r = e / IS, ii = e % IS;
         const int b = t * 64 + r;
         if (b < B && ii < iend) __builtin_nontemporal_store(tile[ii][r], &gx[(size_t)b * I + i0 + ii]);
     }
@@ -755,7 +756,23 @@ template <int K>
 static void dwn_launch_gx(const float *gyT, const uint8_t *addrT, const float *D, const int *inv_ptr, const int *inv_pos,
                           float *gx, int B, int I, int N, int O, bool sform, int out_tiled, hipStream_t s) {
     const int BT = dwn_bt(B);
-    const int grid = dl_xcd_grid(dl_ceil_div(I, DWN_IS), BT);
+    // Long CSR lists per input (average N*k/I: ~70 on the first level of a convolutional layer, 15 under a learnable
+    // mapping) want fewer inputs per wavefront: more, shorter and evenly filled blocks.  Measured at B = 4096, k = 6:
+    // lists of 3 - 16 inputs per wavefront is best (169 vs 221 us); 7.7 - 4 inputs (67 vs 73 us); 15 - 4 (134 vs
+    // 179 us); 31 - 4 (368 vs 442 us); 69 with tile-major output - 1 (249 vs 265 vs 375 us).
+    if (O == 1 && sform && out_tiled && (long long)N * K >= 32LL * I) {
+        const int grid_s = dl_xcd_grid(dl_ceil_div(I, 4), BT);
+        DL_TIMED("dwn_bwd_gx", s, (dwn_bwd_gx<K, true, true, 1><<<grid_s, 256, 0, s>>>(gyT, addrT, D, inv_ptr, inv_pos, gx, B,
+                                                                                     I, N, O, BT, out_tiled)));
+        return;
+    }
+    if (O == 1 && sform && (long long)N * K >= 6LL * I) {
+        const int grid_s = dl_xcd_grid(dl_ceil_div(I, 4 * DWN_WI_SMALL), BT);
+        DL_TIMED("dwn_bwd_gx", s, (dwn_bwd_gx<K, true, true, DWN_WI_SMALL><<<grid_s, 256, 0, s>>>(
+                                      gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, BT, out_tiled)));
+        return;
+    }
+    const int grid = dl_xcd_grid(dl_ceil_div(I, 4 * DWN_WI), BT);
 #define DWN_GX(O1_, S_) \
     DL_TIMED("dwn_bwd_gx", s, (dwn_bwd_gx<K, O1_, S_><<<grid, 256, 0, s>>>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, BT, out_tiled)))
     if (O == 1 && sform) DWN_GX(true, true);
