@@ -555,6 +555,47 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT,
     };
     float acc = 0.0f;  // running sum of the input `cur`
     int cur = -1;
+    // Uniform fan-in: a table of f full permutations (RandomLayer with N*k = f*I) uses every input exactly f times.
+    // For f = 3 - the reference's usual ratio - a wavefront whose 16 inputs all have three entries replays its 48
+    // entries fully unrolled: which input an entry belongs to and where a sum ends are then known at compile time,
+    // so there is no bookkeeping per entry.  Same order of additions as the general loop below.
+    constexpr int FAN = 3;
+    bool uniform3 = false;
+    if (WI == 16 && O1 && SFORM) {
+        const int len = __shfl_down(myptr, 1) - myptr;  // lanes 0..15: entries of my input
+        uniform3 = __ballot(lane >= WI || len == FAN) == ~0ull;
+    }
+    if (WI == 16 && O1 && SFORM && uniform3) {
+        const int p = lane < WI * FAN ? inv_pos[ebeg + lane] : 0;
+        const int n = p / K;
+        const int rec = (n << 3) | (p - n * K);
+#pragma unroll
+        for (int s0 = 0; s0 < WI * FAN; s0 += DWN_EG) {
+            int rj[DWN_EG];
+            unsigned a[DWN_EG];
+            float g[DWN_EG], coef[DWN_EG];
+#pragma unroll
+            for (int q = 0; q < DWN_EG; ++q) {
+                const int r = __builtin_amdgcn_readlane(rec, s0 + q);
+                const int rn = r >> 3;
+                rj[q] = r & 7;
+                a[q] = addr_t[(size_t)rn * 64];
+                g[q] = gy_t[(size_t)rn * 64];
+                coef[q] = D[(size_t)rn * (2 * Lh) + (lane & (2 * Lh - 1))];
+            }
+#pragma unroll
+            for (int q = 0; q < DWN_EG; ++q) {
+                const float hi = dl_lane_read(coef[q], (int)(a[q] | (1u << rj[q])));
+                const float lo = dl_lane_read(coef[q], (int)(a[q] & ~(1u << rj[q])));
+                const float term = g[q] * (hi - lo);
+                constexpr int dummy = 0;
+                (void)dummy;
+                const int s = s0 + q;  // compile-time after unrolling
+                acc = (s % FAN == 0) ? 0.0f + term : acc + term;
+                if (s % FAN == FAN - 1) tile[wbeg + s / FAN][lane] = acc;
+            }
+        }
+    } else
     for (int base = ebeg; base < eend; base += 64) {
         const int e = base + lane;
         const bool valid = e < eend;
