@@ -105,14 +105,26 @@ __global__ __launch_bounds__(256) void group_sum_fwd_kernel(const float *__restr
     if (lane == 0) y[w] = acc * inv_tau;
 }
 
+// thread = four consecutive features of one row
 __global__ __launch_bounds__(256) void group_sum_bwd_kernel(const float *__restrict__ gy, float *__restrict__ gx,
                                                              long long total, int F, int groups, int gsize,
                                                              float inv_tau) {
-    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (gid >= total) return;
-    const long long b = gid / F;
-    const int f = (int)(gid % F);
-    gx[gid] = gy[b * groups + f / gsize] * inv_tau;
+    const long long e = ((long long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (e >= total) return;
+    if ((F & 3) == 0 && (((uintptr_t)gx) & 15) == 0) {
+        const long long b = e / F;
+        const int f = (int)(e - b * F);
+        const float *src = gy + b * groups;
+        typedef float f4 __attribute__((ext_vector_type(4)));
+        const f4 v = {src[(f + 0) / gsize] * inv_tau, src[(f + 1) / gsize] * inv_tau, src[(f + 2) / gsize] * inv_tau,
+                      src[(f + 3) / gsize] * inv_tau};
+        __builtin_nontemporal_store(v, reinterpret_cast<f4 *>(gx + e));
+        return;
+    }
+    for (long long i = e; i < min(total, e + 4); ++i) {
+        const long long b = i / F;
+        gx[i] = gy[b * groups + (int)(i - b * F) / gsize] * inv_tau;
+    }
 }
 
 // ---------------------------------------------------------------------------------
@@ -179,8 +191,9 @@ extern "C" int dl_group_sum_fwd(const float *x, float *y, int B, int F, int grou
     if (!x || !y) return DL_ERR_NULL;
     if (B <= 0 || F <= 0 || groups <= 0 || !(tau > 0.0f)) return DL_ERR_SHAPE;
     const int gsize = (F + groups - 1) / groups;  // features zero-padded up to groups * gsize
-    group_sum_fwd_kernel<<<dl_ceil_div((long long)B * groups, 4), 256, 0, (hipStream_t)stream>>>(x, y, B, F, groups,
-                                                                                                gsize, 1.0f / tau);
+    DL_TIMED("group_sum_fwd", (hipStream_t)stream,
+             (group_sum_fwd_kernel<<<dl_ceil_div((long long)B * groups, 4), 256, 0, (hipStream_t)stream>>>(
+                 x, y, B, F, groups, gsize, 1.0f / tau)));
     return dl_launch_status();
 }
 
@@ -189,8 +202,9 @@ extern "C" int dl_group_sum_bwd(const float *gy, float *gx, int B, int F, int gr
     if (B <= 0 || F <= 0 || groups <= 0 || !(tau > 0.0f)) return DL_ERR_SHAPE;
     const int gsize = (F + groups - 1) / groups;
     const long long total = (long long)B * F;
-    group_sum_bwd_kernel<<<dl_ceil_div(total, 256), 256, 0, (hipStream_t)stream>>>(gy, gx, total, F, groups, gsize,
-                                                                                  1.0f / tau);
+    DL_TIMED("group_sum_bwd", (hipStream_t)stream,
+             (group_sum_bwd_kernel<<<dl_ceil_div(total, 1024), 256, 0, (hipStream_t)stream>>>(gy, gx, total, F, groups, gsize,
+                                                                                           1.0f / tau)));
     return dl_launch_status();
 }
 
