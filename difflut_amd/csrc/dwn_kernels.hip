@@ -21,6 +21,7 @@
 //                           gx[b,i] = sum gyT[c][b] * D[c][j][a'(b)]  - a gather in fixed order
 // k > 6 goes to the one-thread-per-element kernels of dwn_generic.hip.
 #include "dl_common.h"
+#include <type_traits>
 #include "dwn_generic.h"
 
 typedef unsigned long long u64;
@@ -155,14 +156,18 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
         const int c = min(c0 + wbeg + min(s / K, DWN_WC - 1), NO - 1);
         myidx[v] = idx32[(O1 ? c : c / O) * K + s % K] * 8;  // byte offset of the input's plane word
     }
-    if (wbeg < cend) {
+    // FULL: all 128 columns of the tile exist (every tile but possibly the last): no clamps, no per-column checks,
+    // so the column offsets fold into the instructions
+    u64 my_plane = 0;  // CHAIN: lane l keeps the thresholded bits of my wavefront's column l
+    auto columns = [&](auto full_tag) {
+        constexpr bool FULL = decltype(full_tag)::value;
 #pragma unroll
         for (int g = 0; g < DWN_WC; g += DWN_CG) {
             u64 w[DWN_CG][K];
             float entry[DWN_CG];
 #pragma unroll
             for (int q = 0; q < DWN_CG; ++q) {
-                const int c = min(c0 + wbeg + g + q, NO - 1);
+                const int c = FULL ? c0 + wbeg + g + q : min(c0 + wbeg + g + q, NO - 1);
                 // table row of column c, one entry per lane; the row offset travels in an SGPR
                 entry[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_luts, lane4s, c * (L * 4), 0));
 #pragma unroll
@@ -183,11 +188,11 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
 #pragma unroll
                 for (int j = K - 1; j >= 0; --j) addr = dwn_shift_in(addr, w[q][j]);
                 const float v = dl_lane_read(entry[q], (int)addr);
-                if (cc < cend) {
+                if (FULL || cc < cend) {
                     tile[cc][lane] = EVAL ? (v >= 0.5f ? 1.0f : 0.0f) : v;
                     if (CHAIN && planes_out) {  // the next layer's view of this column: bit r = (y[64t+r][c] >= 0.5)
                         const u64 m = __ballot(v >= 0.5f);
-                        if (lane == 0) plane_tile[cc] = m;
+                        if (lane == g + q) my_plane = m;  // a select, the column number is a constant here
                     }
                     const int c = c0 + cc;
                     const int n = O1 ? c : c / O;
@@ -196,7 +201,13 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
                 }
             }
         }
+    };
+    if (CHAIN && c0 + DWN_TC <= NO) {  // (the variant that writes y gains nothing from a second copy of the loop)
+        columns(std::true_type{});
+    } else if (wbeg < cend) {
+        columns(std::false_type{});
     }
+    if (CHAIN && planes_out && lane < DWN_WC && wbeg + lane < cend) plane_tile[wbeg + lane] = my_plane;
     __syncthreads();
     if (CHAIN && planes_out && (int)threadIdx.x < cend) {
         const int rows = min(64, B - t * 64);  // rows past B read as 0, like the planes packed from x
