@@ -705,8 +705,10 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT,
 // Host side
 static inline int dwn_bt(int B) { return (B + 63) / 64; }
 static inline size_t dwn_planes_bytes(int B, int I) { return dl_align256((size_t)dwn_bt(B) * I * sizeof(u64)); }
+// room for either coefficient form: k * 2^(k-1) floats per column (D form) or 2^k (S form, the larger one at k = 1)
 static inline size_t dwn_table_bytes(int N, int k, int O) {
-    return dl_align256((size_t)N * O * k * ((size_t)1 << (k - 1)) * sizeof(float));
+    const size_t d_form = (size_t)k << (k - 1), s_form = (size_t)1 << k;
+    return dl_align256((size_t)N * O * (d_form > s_form ? d_form : s_form) * sizeof(float));
 }
 static inline size_t dwn_gyT_bytes(int B, int N, int O) {
     return dl_align256((size_t)N * O * dwn_bt(B) * 64 * sizeof(float));

@@ -40,6 +40,7 @@ DWN_SHAPES = [  # (B, I, N, k, O)
     (64, 128, 256, 6, 1),
     (130, 300, 77, 5, 3),
     (1, 7, 5, 1, 1),
+    (322, 52, 80, 1, 1),   # k = 1: the S-form table (2 floats per node) is larger than the D form (1 float)
     (65, 9, 300, 2, 1),
     (200, 1030, 515, 6, 2),
     (9, 30, 11, 7, 2),     # k > 6: generic kernels
