@@ -88,6 +88,44 @@ def test_dwn_backward_few_inputs_many_rows(shape):
     np.testing.assert_allclose(lt.grad.cpu().numpy(), wl, rtol=1e-5, atol=2e-4)  # ~B/2^k terms per bin
 
 
+@pytest.mark.parametrize("shape", [(700, 20, 200, 6, 1), (130, 50, 64, 5, 1), (260, 9, 40, 6, 1), (65, 100, 50, 6, 1)])
+def test_dwn_backward_tile_major_output_all_list_lengths(shape):
+    """The tile-major form of the input gradient (what a chained layer or the fold of a convolutional layer
+    reads) through the C entry point, for average CSR list lengths of 60, 6.4, 27 and 3: the gather runs with
+    1, 4, 4 and 16 inputs per wavefront.  Every tile against the row-major result of the same call sequence
+    and against the oracle."""
+    from difflut_amd import _native as nat
+    B, I, N, k, O = shape
+    ops = _ops()
+    lib = nat.lib()
+    x, idx, luts, gy = make_case(sum(shape) % 997, *shape)
+    plan = ops.MappingPlan(dev(idx, torch.int32), I)
+    alpha, beta = 0.5 * 0.75 ** (k - 1), 1.0 / 3.0
+    dims = (B, I, N, k, O)
+    xd, ld, gd = dev(x), dev(luts), dev(gy.reshape(B, N * O))
+    y = torch.empty(B, N * O, device=DEV)
+    saved = torch.empty(lib.dl_dwn_saved_bytes(*dims), dtype=torch.uint8, device=DEV)
+    wf = torch.empty(lib.dl_dwn_fwd_workspace_bytes(*dims), dtype=torch.uint8, device=DEV)
+    wb = torch.empty(lib.dl_dwn_bwd_workspace_bytes(*dims), dtype=torch.uint8, device=DEV)
+    nat.check(lib.dl_dwn_layer_fwd(xd.data_ptr(), plan.idx32.data_ptr(), ld.data_ptr(), y.data_ptr(), saved.data_ptr(),
+                                   wf.data_ptr(), wf.numel(), *dims, nat.stream()))
+    BT = (B + 63) // 64
+    results = []
+    for tiled in (0, 1):
+        gx = torch.zeros(BT * I * 64 if tiled else B * I, device=DEV)
+        gl = torch.empty_like(ld)
+        nat.check(lib.dl_dwn_layer_bwd_tiled(saved.data_ptr(), plan.inv_ptr.data_ptr(), plan.inv_pos.data_ptr(), ld.data_ptr(),
+                                             gd.data_ptr(), 0, alpha, beta, gx.data_ptr(), tiled, gl.data_ptr(), wb.data_ptr(),
+                                             wb.numel(), *dims, nat.stream()))
+        results.append((gx, gl))
+    row_major = results[0][0].view(B, I)
+    tile_major = results[1][0].view(BT, I, 64).permute(0, 2, 1).reshape(BT * 64, I)[:B]
+    assert torch.equal(tile_major, row_major)  # same sums in the same order, another layout
+    wx, wl = orc.dwn_layer_backward(x, idx, luts, gy, np.float32(alpha), np.float32(beta))
+    np.testing.assert_allclose(row_major.cpu().numpy(), wx, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(results[1][1].cpu().numpy(), wl, rtol=1e-5, atol=2e-4)
+
+
 def test_dwn_threshold_is_inclusive_and_exact_at_half():
     ops = _ops()
     x = np.array([[0.5, 0.49999997, 0.50000006, 0.0, 1.0, -3.0]], dtype=np.float32)
