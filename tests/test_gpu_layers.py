@@ -420,6 +420,34 @@ def test_dwn_stack_with_thermometer_encoder(case):
     assert torch.equal(stack(x), he)
 
 
+def test_more_than_2_31_output_elements():
+    """A layer whose output has more than 2^31 elements (131109 rows x 16400 nodes; about 30 GB of device memory in
+    all): sampled rows of the forward and of the input gradient against the oracle, and the mass of every node's
+    table gradient against the column sums of the upstream gradient.  Guards the 64-bit offsets."""
+    from difflut_amd import ops
+    B, I, N, k, O = 131072 + 37, 512, 16400, 6, 1
+    assert B * N > 2 ** 31
+    torch.manual_seed(0)
+    x = torch.rand(B, I, device="cuda")
+    idx = orc.random_mapping(I, N, k, seed=3)
+    plan = ops.MappingPlan(idx.cuda(), I)
+    luts = (torch.rand(N, O, 64, device="cuda") * 2 - 1).requires_grad_()
+    xt = x.clone().requires_grad_()
+    y = ops.DWNLayerFunction.apply(xt, luts, plan, 0.1, 1.0 / 3.0)
+    rows = torch.tensor([0, 1, 63, 64, 65535, 65536, 131071, 131072, B - 1])
+    idx_np, luts_np = idx.numpy().astype(np.int64), luts.detach().cpu().numpy()
+    want = orc.dwn_layer_forward(x[rows].cpu().numpy(), idx_np, luts_np).reshape(len(rows), -1)
+    assert np.array_equal(y[rows].detach().cpu().numpy(), want)
+    gy = torch.randn(B, N, device="cuda")
+    y.backward(gy)
+    mass = luts.grad.double().sum(-1).view(-1)
+    col = gy.double().sum(0)
+    torch.testing.assert_close(mass, col, rtol=1e-4, atol=1e-4 * float(col.abs().max()))
+    gxs, _ = orc.dwn_layer_backward(x[rows].cpu().numpy(), idx_np, luts_np, gy[rows].cpu().numpy().reshape(len(rows), N, 1),
+                                    np.float32(0.1), np.float32(1.0 / 3.0))
+    np.testing.assert_allclose(xt.grad[rows].cpu().numpy(), gxs, rtol=1e-5, atol=2e-5)  # ~190 terms per input
+
+
 def test_full_size_deep_stack_b8192():
     """The deep-stack configuration at its full size (8192 x 784 -> thermometer 4 bits -> 16000/8000/4000/2000
     DWN k=6 nodes -> GroupSum 10 -> cross-entropy): the chained run against the layers one by one (logits and
