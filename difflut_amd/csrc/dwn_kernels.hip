@@ -365,7 +365,7 @@ template <bool WRITE_T>
 __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__restrict__ gy, const uint8_t *__restrict__ addrT,
                                                                float *__restrict__ gyT, float *__restrict__ gluts,
                                                                int B, int NO, int O, int L, int BP, int BT,
-                                                               int tiles_per_chunk) {
+                                                               int tiles_per_chunk, const float *__restrict__ scale = nullptr) {
     __shared__ float tile[64][DWN_HC + 1];       // [row][column]
     __shared__ float hist[DWN_HC][65];           // [column][bin]
     __shared__ uint8_t atile[DWN_HC][64 + 4];    // [column][row] addresses
@@ -444,7 +444,9 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
         }
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < cend * L; e += 256) atomicAdd(&gluts[(size_t)c0 * L + e], hist[e / L][e % L]);
+    // scale (nullable): the stabilised node multiplies a node's table gradient by its gradient_scale
+    for (int e = threadIdx.x; e < cend * L; e += 256)
+        atomicAdd(&gluts[(size_t)c0 * L + e], hist[e / L][e % L] * (scale ? scale[(c0 + e / L) / O] : 1.0f));
 }
 
 // hist_tiled: the histogram alone, for gy that arrives tile-major ([B/64][N*O][64]).  Nothing has to be
@@ -883,10 +885,10 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
                  (dwn_bwd_hist_tiled<false><<<hgrid, 256, 0, s>>>(gy, addrT, gluts, (int)NO, O, L, BT, tpc)));
     else if (gx)
         DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<true><<<hgrid, 256, 0, s>>>(
-                                                  gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc)));
+                                                  gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc, scale)));
     else
         DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<false><<<hgrid, 256, 0, s>>>(
-                                                  gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc)));
+                                                  gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc, scale)));
     if (gx) {
         const float *src = gy_tiled ? gy : gyT;
         switch (k) {
@@ -898,7 +900,7 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
             default: dwn_launch_gx<6>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, s); break;
         }
     }
-    if (scale)
+    if (scale && (gy_tiled || head))  // the row-major histogram applies the scale when it flushes
         DL_TIMED("dwn_scale_tables", s,
                  (dwn_scale_tables<<<dl_ceil_div(NO * L, 256), 256, 0, s>>>(gluts, scale, NO * L, L, O)));
     return dl_launch_status();
