@@ -20,14 +20,33 @@ def sources():
     return sorted(glob.glob(os.path.join(CSRC, "*.hip")))
 
 
-def build(verbose=False):
-    """Always recompiles; returns the path of the shared library."""
+def build(verbose=False, jobs=None):
+    """Always recompiles (the sources in parallel, one hipcc per file), then links; returns the path of the library."""
+    from concurrent.futures import ThreadPoolExecutor
+
     os.makedirs(LIB_DIR, exist_ok=True)
+    obj_dir = os.path.join(LIB_DIR, "_obj")
+    os.makedirs(obj_dir, exist_ok=True)
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + HIPCC_FLAGS + ["-o", LIB_PATH] + sources()
+    compile_flags = [f for f in HIPCC_FLAGS if f != "-shared"] + ["-c"]
+
+    def compile_one(src):
+        obj = os.path.join(obj_dir, os.path.basename(src) + ".o")
+        cmd = [hipcc] + compile_flags + ["-o", obj, src]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError("hipcc failed on " + src + ":\n" + res.stdout + res.stderr)
+        if verbose:
+            print(" ".join(cmd))
+        return obj
+
+    srcs = sources()
+    with ThreadPoolExecutor(max_workers=jobs or min(8, len(srcs))) as pool:
+        objs = list(pool.map(compile_one, srcs))
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + res.stdout + res.stderr)
+        raise RuntimeError("hipcc (link) failed:\n" + res.stdout + res.stderr)
     if verbose:
         print(" ".join(cmd))
     return LIB_PATH
