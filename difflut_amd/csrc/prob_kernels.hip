@@ -40,9 +40,24 @@ __global__ __launch_bounds__(256) void prob_sig_table(const float *__restrict__ 
     sig[e] = dl_sigmoid(raw[((size_t)n * L + a) * O + d] * inv_t);
 }
 
-// grid (ceil(C / 64), B/64 rounded up), 256 threads
-__global__ __launch_bounds__(256) void prob_to_tiles(const float *__restrict__ src, float *__restrict__ dst, int B, int C) {
+// grid (ceil(C / 64), B/64 rounded up), 256 threads.  With `sig` set the launch carries extra rows of blocks
+// (blockIdx.y >= tiles) that build the sigmoid table in the same launch: the two jobs are independent and each is
+// too short to fill the machine on its own.
+__global__ __launch_bounds__(256) void prob_to_tiles(const float *__restrict__ src, float *__restrict__ dst, int B, int C,
+                                                      int tiles = 1 << 30, const float *__restrict__ raw = nullptr,
+                                                      float inv_t = 1.0f, float *__restrict__ sig = nullptr, int N = 0,
+                                                      int L = 1, int O = 1) {
     __shared__ float tile[64][65];  // [column][row]
+    if ((int)blockIdx.y >= tiles) {
+        const long long e = ((long long)(blockIdx.y - tiles) * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
+        if (e < (long long)N * L * O) {
+            const int a = (int)(e % L);
+            const long long c = e / L;
+            const int n = (int)(c / O), d = (int)(c % O);
+            sig[e] = dl_sigmoid(raw[((size_t)n * L + a) * O + d] * inv_t);
+        }
+        return;
+    }
     const int t = blockIdx.y, c0 = blockIdx.x * 64;
     if ((C & 3) == 0 && c0 + 64 <= C && (((uintptr_t)src) & 15) == 0) {
 #pragma unroll
@@ -533,8 +548,12 @@ extern "C" int dl_prob_layer_fwd(const float *x, const int32_t *idx32, const flo
     const int BT = prob_bt(B), L = 1 << k;
     float *sig = (float *)saved;
     float *xT = (float *)((char *)saved + prob_sig_bytes(N, k, O));
-    DL_TIMED("prob_sig_table", s, (prob_sig_table<<<dl_ceil_div((long long)N * L * O, 256), 256, 0, s>>>(raw_w, inv_t, sig, N, L, O)));
-    DL_TIMED("prob_to_tiles_x", s, (prob_to_tiles<<<dim3(dl_ceil_div(I, 64), BT), 256, 0, s>>>(x, xT, B, I)));
+    {   // x re-tiled and the sigmoid table built in one launch
+        const int gx_ = dl_ceil_div(I, 64);
+        const int extra = dl_ceil_div(dl_ceil_div((long long)N * L * O, 256), gx_);
+        DL_TIMED("prob_to_tiles_x+sig_table", s, (prob_to_tiles<<<dim3(gx_, BT + extra), 256, 0, s>>>(
+                                                     x, xT, B, I, BT, raw_w, inv_t, sig, N, L, O)));
+    }
     const int grid = dl_xcd_grid(dl_ceil_div((long long)N * O, PROB_TC), BT);
 #define CALL(KK) DL_TIMED("prob_fwd_t", s, (prob_fwd_t<KK><<<grid, 64 * PROB_FW, 0, s>>>(xT, idx32, sig, y, B, I, N, O, BT)))
     PROB_DISPATCH(k, CALL)
