@@ -277,10 +277,21 @@ __global__ __launch_bounds__(256) void prob_bwd_t(const float *__restrict__ xT, 
 
 // graw[n,a,d] = sigmoid'(w/T)/T * sum over chunks of gpart[chunk][c][a];
 // sig == null (hybrid node): the plain sum, kept in the table's own layout [c][a]
-__global__ __launch_bounds__(256) void prob_reduce_weights(const float *__restrict__ gpart, const float *__restrict__ sig,
-                                                            float inv_t, float *__restrict__ graw, int N, int L, int O,
-                                                            int chunks) {
-    const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+struct ProbReduce {  // the table-gradient reduction, also carried as extra blocks of the gather launch
+    const float *gpart, *sig;
+    float inv_t;
+    float *graw;
+    int N, L, O, chunks;
+};
+__device__ __forceinline__ void prob_reduce_element(const ProbReduce &R, long long e);
+__global__ __launch_bounds__(256) void prob_reduce_weights(ProbReduce R) {
+    prob_reduce_element(R, (long long)blockIdx.x * 256 + threadIdx.x);
+}
+__device__ __forceinline__ void prob_reduce_element(const ProbReduce &R, long long e) {
+    const float *gpart = R.gpart, *sig = R.sig;
+    const float inv_t = R.inv_t;
+    float *graw = R.graw;
+    const int N = R.N, L = R.L, O = R.O, chunks = R.chunks;
     const long long total = (long long)N * L * O;
     if (e >= total) return;
     float acc = 0.0f;
@@ -305,8 +316,12 @@ __global__ __launch_bounds__(256) void prob_reduce_weights(const float *__restri
 template <bool FAST>
 __global__ __launch_bounds__(256) void prob_gather_t(const float *__restrict__ gmT, const int *__restrict__ inv_ptr,
                                                       const int *__restrict__ inv_pos, float *__restrict__ gx, int B,
-                                                      int I, int N, int K, int O, int BT) {
+                                                      int I, int N, int K, int O, int BT, int gather_blocks, ProbReduce R) {
     __shared__ float tile[PROB_IS][65];  // [input][row]
+    if ((int)blockIdx.x >= gather_blocks) {  // the blocks appended for the independent table-gradient reduction
+        prob_reduce_element(R, (long long)(blockIdx.x - gather_blocks) * 256 + threadIdx.x);
+        return;
+    }
     int slab, t;
     if (!dl_xcd_map((I + PROB_IS - 1) / PROB_IS, BT, slab, t)) return;
     const int i0 = slab * PROB_IS;
@@ -408,6 +423,24 @@ __global__ __launch_bounds__(256) void prob_gather_t(const float *__restrict__ g
             if (b < B && ii < iend) gx[(size_t)b * I + i0 + ii] = tile[ii][r];
         }
     }
+}
+
+// the gather and the reduction of the table-gradient partials do not depend on each other: one launch, the
+// reduction as extra blocks behind the gather's
+static void prob_launch_gather_and_reduce(const float *gmT, const int *inv_ptr, const int *inv_pos, float *gx, int B, int I,
+                                          int N, int k, int O, int BT, const ProbReduce &R, long long WT, hipStream_t s) {
+    const int rblocks = dl_ceil_div(WT, 256);
+    if (!gx) {
+        DL_TIMED("prob_reduce_weights", s, (prob_reduce_weights<<<rblocks, 256, 0, s>>>(R)));
+        return;
+    }
+    const int gblocks = dl_xcd_grid(dl_ceil_div(I, PROB_IS), BT);
+    if (O == 1)
+        DL_TIMED("prob_gather_t+reduce", s, (prob_gather_t<true><<<gblocks + rblocks, 256, 0, s>>>(gmT, inv_ptr, inv_pos, gx, B, I,
+                                                                                               N, k, O, BT, gblocks, R)));
+    else
+        DL_TIMED("prob_gather_t+reduce", s, (prob_gather_t<false><<<gblocks + rblocks, 256, 0, s>>>(gmT, inv_ptr, inv_pos, gx, B, I,
+                                                                                                N, k, O, BT, gblocks, R)));
 }
 
 // ---------------------------------------------------------------------------------
@@ -604,16 +637,8 @@ extern "C" int dl_prob_layer_bwd(const float *x, const void *saved, const int32_
                                                                                   BT, tpc, gx != nullptr)))
     PROB_DISPATCH(k, CALL)
 #undef CALL
-    DL_TIMED("prob_reduce_weights", s,
-             (prob_reduce_weights<<<dl_ceil_div(WT, 256), 256, 0, s>>>(gpart, sig, inv_t, graw, N, L, O, chunks)));
-    if (gx && O == 1)
-        DL_TIMED("prob_gather_t", s,
-                 (prob_gather_t<true><<<dl_xcd_grid(dl_ceil_div(I, PROB_IS), BT), 256, 0, s>>>(gmT, inv_ptr, inv_pos, gx, B, I,
-                                                                                             N, k, O, BT)));
-    else if (gx)
-        DL_TIMED("prob_gather_t", s,
-                 (prob_gather_t<false><<<dl_xcd_grid(dl_ceil_div(I, PROB_IS), BT), 256, 0, s>>>(gmT, inv_ptr, inv_pos, gx, B, I,
-                                                                                              N, k, O, BT)));
+    const ProbReduce R = {gpart, sig, inv_t, graw, N, L, O, chunks};
+    prob_launch_gather_and_reduce(gmT, inv_ptr, inv_pos, gx, B, I, N, k, O, BT, R, WT, s);
     return dl_launch_status();
 }
 
@@ -657,16 +682,8 @@ extern "C" int dl_hybrid_layer_bwd(const float *x, const int32_t *idx32, const i
                                                                                  BT, tpc, gx != nullptr)))
     PROB_DISPATCH(k, CALL)
 #undef CALL
-    DL_TIMED("prob_reduce_weights", s,
-             (prob_reduce_weights<<<dl_ceil_div(WT, 256), 256, 0, s>>>(gpart, nullptr, 1.0f, gluts, N, L, O, chunks)));
-    if (gx && O == 1)
-        DL_TIMED("prob_gather_t", s,
-                 (prob_gather_t<true><<<dl_xcd_grid(dl_ceil_div(I, PROB_IS), BT), 256, 0, s>>>(gmT, inv_ptr, inv_pos, gx, B, I,
-                                                                                             N, k, O, BT)));
-    else if (gx)
-        DL_TIMED("prob_gather_t", s,
-                 (prob_gather_t<false><<<dl_xcd_grid(dl_ceil_div(I, PROB_IS), BT), 256, 0, s>>>(gmT, inv_ptr, inv_pos, gx, B, I,
-                                                                                              N, k, O, BT)));
+    const ProbReduce R = {gpart, nullptr, 1.0f, gluts, N, L, O, chunks};
+    prob_launch_gather_and_reduce(gmT, inv_ptr, inv_pos, gx, B, I, N, k, O, BT, R, WT, s);
     return dl_launch_status();
 }
 
