@@ -680,6 +680,55 @@ def test_dwn_layer_step_replays_from_a_hip_graph():
         torch.testing.assert_close(gls, wgl, rtol=1e-5, atol=1e-6)  # float atomics: order may differ
 
 
+def test_inference_stack_replays_from_a_hip_graph():
+    """Chained inference (thermometer planes -> eval lookups -> GroupSum count) and a single layer's eval forward
+    (device-side check of its input, both kernels launched) captured once and replayed on new inputs, with
+    eager runs and synchronisations in between; every replay equals the eager result."""
+    REGISTRY, NodeConfig, uniform_init, _ = _api()
+    from difflut_amd.layers import DWNStack
+    from difflut_amd.utils import GroupSum
+    torch.manual_seed(11)
+    B, F = 200, 30
+    xs = [torch.rand(B, F, device="cuda") for _ in range(4)]
+    enc = REGISTRY.build_encoder("thermometer", num_bits=3).fit(xs[0])
+    layers, width = [], F * 3
+    for li, n in enumerate([150, 128]):
+        layers.append(REGISTRY.get_layer("random")(width, n, REGISTRY.get_node("dwn"),
+                                                   NodeConfig(input_dim=6, output_dim=1, init_fn=uniform_init,
+                                                              init_kwargs={"a": 0.0, "b": 1.0}), seed=li + 41).cuda())
+        width = n
+    stack = DWNStack(layers, encoder=enc, head=GroupSum(k=2, tau=1.0, use_randperm=False)).eval()
+    single = layers[0].eval()
+    static_x = xs[0].clone()
+    static_bits = enc.encode(xs[0]).clone()
+    static_bits[0, 0] = 0.5                      # not binary: the generic kernel must answer for this input
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side), torch.no_grad():
+        for _ in range(2):
+            stack(static_x)
+            single(static_bits)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph), torch.no_grad():
+        out_stack = stack(static_x)
+        out_single = single(static_bits)
+    for i, x in enumerate(xs):
+        bits = enc.encode(x)
+        if i % 2 == 0:
+            bits[0, 0] = 0.5
+        static_x.copy_(x)
+        static_bits.copy_(bits)
+        graph.replay()
+        torch.cuda.synchronize()
+        with torch.no_grad():
+            want_stack = stack(x)
+            want_single = single(bits)
+        torch.cuda.synchronize()
+        assert torch.equal(out_stack, want_stack), f"replay {i}: stack"
+        assert torch.equal(out_single, want_single), f"replay {i}: single layer ({'mixed' if i % 2 == 0 else 'binary'} input)"
+
+
 def test_legacy_extension_names_and_signatures(golden):
     """tests/test_layers/test_fused_kernels.py:159-179 imports efd_cuda / efd_fused_cuda by bare name;
     the shims answer with the reference's signatures."""
