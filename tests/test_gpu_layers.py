@@ -680,6 +680,53 @@ def test_dwn_layer_step_replays_from_a_hip_graph():
         torch.testing.assert_close(gls, wgl, rtol=1e-5, atol=1e-6)  # float atomics: order may differ
 
 
+def test_training_stack_step_replays_from_a_hip_graph():
+    """Forward + backward of a chained stack (thermometer planes in, GroupSum head out) captured once and replayed on
+    new inputs and upstream gradients; logits bit-equal to eager, table gradients to rtol 1e-5 (atomic adds)."""
+    REGISTRY, NodeConfig, uniform_init, _ = _api()
+    from difflut_amd.layers import DWNStack
+    from difflut_amd.utils import GroupSum
+    torch.manual_seed(13)
+    B, F = 300, 40
+    xs = [torch.rand(B, F, device="cuda") for _ in range(3)]
+    gs = [torch.randn(B, 4, device="cuda") for _ in range(3)]
+    enc = REGISTRY.build_encoder("thermometer", num_bits=2).fit(xs[0])
+    layers, width = [], F * 2
+    for li, n in enumerate([120, 240, 256]):
+        layers.append(REGISTRY.get_layer("random")(width, n, REGISTRY.get_node("dwn"),
+                                                   NodeConfig(input_dim=6, output_dim=1, init_fn=uniform_init,
+                                                              init_kwargs={"a": -1.0, "b": 2.0}), seed=li + 51).cuda())
+        width = n
+    stack = DWNStack(layers, encoder=enc, head=GroupSum(k=4, tau=2.0, use_randperm=False)).train()
+    banks = [layer._banks["luts"].flat for layer in layers]
+    static_x, static_g = xs[0].clone(), gs[0].clone()
+
+    def step(x, g):
+        out = stack(x)
+        grads = torch.autograd.grad(out, banks, g)
+        return out.detach(), grads
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step(static_x, static_g)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_c, grads_c = step(static_x, static_g)
+    for i, (x, g) in enumerate(zip(xs, gs)):
+        static_x.copy_(x)
+        static_g.copy_(g)
+        graph.replay()
+        torch.cuda.synchronize()
+        want_out, want_grads = step(x, g)
+        torch.cuda.synchronize()
+        assert torch.equal(out_c, want_out), f"replay {i}"
+        for got, want in zip(grads_c, want_grads):
+            torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-5)
+
+
 def test_inference_stack_replays_from_a_hip_graph():
     """Chained inference (thermometer planes -> eval lookups -> GroupSum count) and a single layer's eval forward
     (device-side check of its input, both kernels launched) captured once and replayed on new inputs, with
