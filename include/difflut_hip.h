@@ -15,7 +15,9 @@
  *
  * Shapes: B batch rows, I layer inputs, N nodes, k inputs per node, L = 2^k
  * table entries, O outputs per node, M = N*k selections of a learnable layer.
- * All float tensors are fp32, row-major, contiguous.
+ * All float tensors are fp32, row-major, contiguous.  Workspaces, `saved` buffers, bit-planes and tile-major
+ * tensors must be 16-byte aligned (what hipMalloc and torch's allocator return is enough); fp32 tensors
+ * take vectorised paths when they are 16-byte aligned and their row length is a multiple of 4.
  */
 #ifndef DIFFLUT_HIP_H
 #define DIFFLUT_HIP_H
