@@ -65,6 +65,8 @@ SIGNATURES = {
     "dl_unfold": (_I, [_P, _P, _P] + [_I] * 10 + [_P]),
     "dl_fold": (_I, [_P, _I, _P] + [_I] * 10 + [_P]),
     "dl_group_sum_fwd": (_I, [_P, _P, _I, _I, _I, _F, _P]),
+    "dl_cross_entropy_workspace_bytes": (_Z, [_I]),
+    "dl_cross_entropy": (_I, [_P, _P, _P, _P, _P, _Z, _I, _I, _P]),
     "dl_group_sum_bwd": (_I, [_P, _P, _I, _I, _I, _F, _P]),
     "dl_profile_enable": (_I, [_I]),
     "dl_profile_read": (_I, [ctypes.c_char_p, _Z, ctypes.POINTER(_F), _I]),

@@ -128,6 +128,40 @@ __global__ __launch_bounds__(256) void group_sum_bwd_kernel(const float *__restr
 }
 
 // ---------------------------------------------------------------------------------
+// Cross-entropy with mean reduction over the batch on [B, C] logits (the loss that follows GroupSum in the
+// training configurations): one thread per row computes the row's loss (logsumexp - logit[label]) and the
+// gradient of the MEAN loss, (softmax - onehot) / B; a single block then adds the B row losses in a fixed order.
+__global__ __launch_bounds__(256) void cross_entropy_rows(const float *__restrict__ logits, const long long *__restrict__ labels,
+                                                           float *__restrict__ row_loss, float *__restrict__ glogits, int B,
+                                                           int C) {
+    const int b = blockIdx.x * 256 + threadIdx.x;
+    if (b >= B) return;
+    const float *z = logits + (size_t)b * C;
+    float m = -INFINITY;
+    for (int c = 0; c < C; ++c) m = fmaxf(m, z[c]);
+    float sum = 0.0f;
+    for (int c = 0; c < C; ++c) sum += expf(z[c] - m);
+    const long long label = labels[b];
+    const bool ok = label >= 0 && label < C;
+    row_loss[b] = ok ? (logf(sum) + m) - z[label] : 0.0f;  // rows with a label outside [0, C) are left out
+    const float inv = 1.0f / sum, invB = 1.0f / (float)B;
+    float *g = glogits + (size_t)b * C;
+    for (int c = 0; c < C; ++c) g[c] = ok ? (expf(z[c] - m) * inv - (c == label ? 1.0f : 0.0f)) * invB : 0.0f;
+}
+__global__ __launch_bounds__(256) void cross_entropy_mean(const float *__restrict__ row_loss, float *__restrict__ loss, int B) {
+    __shared__ float part[256];
+    float acc = 0.0f;
+    for (int b = threadIdx.x; b < B; b += 256) acc += row_loss[b];
+    part[threadIdx.x] = acc;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) part[threadIdx.x] += part[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *loss = part[0] / (float)B;
+}
+
+// ---------------------------------------------------------------------------------
 extern "C" int dl_gather_fwd(const float *x, const void *idx, int idx_bits, float *m, int B, int I, int N, int k,
                              void *stream) {
     if (!x || !idx || !m) return DL_ERR_NULL;
@@ -184,6 +218,19 @@ extern "C" int dl_thermometer_planes(const float *x, const float *thr, void *pla
     DL_TIMED("thermometer_planes", s,
              (thermometer_planes_kernel<<<dim3(dl_ceil_div(F, 64), dl_ceil_div(B, 64)), 256, 0, s>>>(
                  x, thr, (unsigned long long *)planes, B, F, nbits)));
+    return dl_launch_status();
+}
+
+extern "C" size_t dl_cross_entropy_workspace_bytes(int B) { return B > 0 ? dl_align256((size_t)B * sizeof(float)) : 256; }
+extern "C" int dl_cross_entropy(const float *logits, const long long *labels, float *loss, float *glogits, void *ws,
+                                size_t ws_bytes, int B, int C, void *stream) {
+    if (!logits || !labels || !loss || !glogits || !ws) return DL_ERR_NULL;
+    if (B <= 0 || C <= 0) return DL_ERR_SHAPE;
+    if (ws_bytes < dl_cross_entropy_workspace_bytes(B)) return DL_ERR_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    DL_TIMED("cross_entropy_rows", s,
+             (cross_entropy_rows<<<dl_ceil_div(B, 256), 256, 0, s>>>(logits, labels, (float *)ws, glogits, B, C)));
+    DL_TIMED("cross_entropy_mean", s, (cross_entropy_mean<<<1, 256, 0, s>>>((const float *)ws, loss, B)));
     return dl_launch_status();
 }
 

@@ -585,6 +585,33 @@ def thermometer_encode(x, thresholds):
     return bits
 
 
+class CrossEntropyFunction(torch.autograd.Function):
+    """Mean cross-entropy of [B, C] logits against int64 class labels: loss and its gradient from one pass
+    (what torch.nn.functional.cross_entropy and its backward compute for the logits GroupSum returns)."""
+
+    @staticmethod
+    def forward(ctx, logits, labels):
+        nat.require_device(logits, labels)
+        logits = _f32(logits)
+        if logits.dim() != 2 or labels.shape != (logits.shape[0],):
+            raise RuntimeError(f"expected logits [B, C] and labels [B], got {tuple(logits.shape)} and {tuple(labels.shape)}")
+        labels = labels.to(torch.int64).contiguous()
+        B, C = logits.shape
+        lib = nat.lib()
+        loss = torch.empty((), dtype=torch.float32, device=logits.device)
+        glogits = torch.empty_like(logits)
+        ws = _bytes(lib.dl_cross_entropy_workspace_bytes(B), logits.device)
+        nat.check(lib.dl_cross_entropy(nat.ptr(logits), nat.ptr(labels), nat.ptr(loss), nat.ptr(glogits), nat.ptr(ws),
+                                       ws.numel(), B, C, nat.stream()))
+        ctx.save_for_backward(glogits)
+        return loss
+
+    @staticmethod
+    def backward(ctx, gloss):
+        (glogits,) = ctx.saved_tensors
+        return glogits * gloss, None
+
+
 class GroupSumFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, groups, tau):

@@ -276,6 +276,15 @@ int dl_thermometer_encode(const float *x, const float *thr, float *bits, int B, 
 int dl_thermometer_planes(const float *x, const float *thr, void *planes, int B, int F, int nbits,
                           void *stream);
 int dl_group_sum_fwd(const float *x, float *y, int B, int F, int groups, float tau, void *stream);
+/* Cross-entropy with mean reduction on the [B, C] logits that GroupSum returns (the loss of the training
+ * configurations; torch.nn.CrossEntropyLoss in the reference's examples and tests, e.g.
+ * tests/test_layers/test_convolutional_learning.py): *loss = mean_b(logsumexp(logits[b]) - logits[b][labels[b]]),
+ * glogits = d loss / d logits = (softmax - onehot) / B, both from one pass over the logits; the B row losses
+ * are added in a fixed order.  labels are int64 class indices; rows whose label is outside [0, C) add nothing.
+ * Workspace: dl_cross_entropy_workspace_bytes(B). */
+size_t dl_cross_entropy_workspace_bytes(int B);
+int dl_cross_entropy(const float *logits, const long long *labels, float *loss, float *glogits, void *ws,
+                     size_t ws_bytes, int B, int C, void *stream);
 int dl_group_sum_bwd(const float *gy, float *gx, int B, int F, int groups, float tau, void *stream);
 
 /* ------------------------------------------------------------------------

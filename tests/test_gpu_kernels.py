@@ -410,6 +410,34 @@ def test_thermometer_and_group_sum(golden):
     np.testing.assert_allclose(y.cpu().numpy(), orc.group_sum(x, 4, 1.0), rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("shape", [(8192, 10), (1, 3), (257, 1), (1000, 64), (33, 300)])
+def test_cross_entropy_against_torch(shape):
+    """Fused mean cross-entropy and its gradient against torch's own (float64 on the CPU): loss to rtol 1e-6,
+    gradient to rtol 1e-5 with a floor of 1e-9 (entries are (softmax - onehot) / B); large logits do not overflow;
+    a row with a label outside the classes adds nothing."""
+    from difflut_amd.utils import cross_entropy
+    B, C = shape
+    rng = np.random.default_rng(B + C)
+    z = (rng.standard_normal((B, C)) * 4).astype(np.float32)
+    z[0, 0] = 90.0                                        # exp(90) overflows fp32 without the max shift
+    y = rng.integers(0, C, (B,))
+    zt = dev(z).requires_grad_()
+    loss = cross_entropy(zt, torch.as_tensor(y, device=DEV))
+    (loss * 3.0).backward()
+    zr = torch.tensor(z, dtype=torch.float64, requires_grad=True)
+    want = torch.nn.functional.cross_entropy(zr, torch.as_tensor(y))
+    (want * 3.0).backward()
+    np.testing.assert_allclose(loss.item(), want.item(), rtol=1e-6)
+    np.testing.assert_allclose(zt.grad.cpu().numpy(), zr.grad.numpy(), rtol=1e-5, atol=1e-9)
+    if B > 1:
+        y2 = y.copy()
+        y2[1] = C + 5
+        l2 = cross_entropy(dev(z), torch.as_tensor(y2, device=DEV))
+        keep = np.ones(B, bool); keep[1] = False
+        ref = torch.nn.functional.cross_entropy(torch.tensor(z[keep], dtype=torch.float64), torch.as_tensor(y[keep]), reduction="sum") / B
+        np.testing.assert_allclose(l2.item(), ref.item(), rtol=1e-6)
+
+
 # ------------------------------------------------------------------------------ error paths
 def test_argument_errors_are_reported_not_launched():
     from difflut_amd import _native as nat
