@@ -962,6 +962,116 @@ extern "C" int dl_table_sigmoid_bwd(const float *gluts, const float *luts, float
 }
 
 // ---------------------------------------------------------------------------------
+// Bit-sliced inference for a layer between two bit-plane tensors.  Lanes are NODES here: a lane keeps its column's
+// truth table as 2^k bits (table entry >= 0.5), fetches the k plane words of its inputs for a batch tile (64 rows in
+// one 64-bit word each) and evaluates the table on all 64 rows at once as a multiplexer tree of bitwise operations:
+// level j halves the table with the word of input j,  v[i] = v[2i] ^ ((v[2i] ^ v[2i+1]) & x_j).  About 6 vector
+// instructions per (node, tile) instead of 13 vector + 26 scalar in the lookup kernel, and the result of a lane is
+// already the plane word of its column.  A block takes 256 columns and walks `tiles_per_block` tiles with the same
+// indices and tables in registers.
+// SAVE: the training forward of a chained hidden layer - the same planes out, plus the address of every
+// (node, row) for the backward ([tile][node][64] bytes): the k plane words are turned into 16 words of four
+// address bytes each (a nibble of rows times 0x204081 puts its four bits at the bottom of four bytes).
+template <int K, bool SAVE = false>
+__global__ __launch_bounds__(256) void dwn_eval_bitsliced(const u64 *__restrict__ planes, const int *__restrict__ idx32,
+                                                           const float *__restrict__ luts, u64 *__restrict__ planes_out,
+                                                           int B, int I, int N, int O, int BT, int tiles_per_block,
+                                                           uint8_t *__restrict__ addrT = nullptr) {
+    constexpr int L = 1 << K;
+    const int NO = N * O;
+    const int lane = threadIdx.x & 63;
+    const int wave = dl_uniform(threadIdx.x >> 6);
+    const int wc0 = (blockIdx.x * 4 + wave) * 64;  // my wavefront's first column
+    if (wc0 >= NO) return;
+    const int c = min(wc0 + lane, NO - 1);
+    // truth tables of the wavefront's 64 columns: row u of the tables is read with lane = entry and voted on
+    unsigned t_lo = 0u, t_hi = 0u;
+    for (int u = 0; u < 64; ++u) {
+        const int cu = min(wc0 + u, NO - 1);
+        const float v = lane < L ? luts[(size_t)cu * L + lane] : 0.0f;
+        const u64 bits = __ballot(v >= 0.5f);
+        if (lane == u) { t_lo = (unsigned)bits; t_hi = (unsigned)(bits >> 32); }
+    }
+    int off[K];  // word offsets of my inputs inside a tile's planes
+#pragma unroll
+    for (int j = 0; j < K; ++j) off[j] = idx32[(size_t)(c / O) * K + j];
+    const int t_begin = blockIdx.y * tiles_per_block;
+    const int t_end = min(BT, t_begin + tiles_per_block);
+    u64 w[K], wn[K];
+    auto fetch = [&](int t, u64 (&dst)[K]) {
+#pragma unroll
+        for (int j = 0; j < K; ++j) dst[j] = planes[(size_t)t * I + off[j]];
+    };
+    if (t_begin < t_end) fetch(t_begin, w);
+    for (int t = t_begin; t < t_end; ++t) {
+        if (t + 1 < t_end) fetch(t + 1, wn);
+        unsigned vlo[L / 2 > 0 ? L / 2 : 1], vhi[L / 2 > 0 ? L / 2 : 1];
+        const unsigned x0lo = (unsigned)w[0], x0hi = (unsigned)(w[0] >> 32);
+#pragma unroll
+        for (int i = 0; i < L / 2; ++i) {  // level of input 0: the leaves are table bits, spread to 0 / ~0
+            const unsigned src0 = (2 * i < 32) ? t_lo : t_hi, src1 = (2 * i + 1 < 32) ? t_lo : t_hi;
+            const unsigned m0 = (unsigned)__builtin_amdgcn_sbfe((int)src0, (2 * i) & 31, 1);
+            const unsigned m1 = (unsigned)__builtin_amdgcn_sbfe((int)src1, (2 * i + 1) & 31, 1);
+            const unsigned d = m0 ^ m1;
+            vlo[i] = m0 ^ (d & x0lo);
+            vhi[i] = m0 ^ (d & x0hi);
+        }
+#pragma unroll
+        for (int j = 1; j < K; ++j) {
+            const unsigned xlo = (unsigned)w[j], xhi = (unsigned)(w[j] >> 32);
+#pragma unroll
+            for (int i = 0; i < (L >> (j + 1)); ++i) {
+                vlo[i] = vlo[2 * i] ^ ((vlo[2 * i] ^ vlo[2 * i + 1]) & xlo);
+                vhi[i] = vhi[2 * i] ^ ((vhi[2 * i] ^ vhi[2 * i + 1]) & xhi);
+            }
+        }
+        const int rows = min(64, B - t * 64);  // rows past B stay 0, like the planes packed from x
+        const u64 valid = rows == 64 ? ~0ull : ((1ull << rows) - 1ull);
+        if (wc0 + lane < NO) planes_out[(size_t)t * NO + wc0 + lane] = (((u64)vhi[0] << 32) | vlo[0]) & valid;
+        if (SAVE && wc0 + lane < NO && c % O == 0) {
+            typedef unsigned u4v __attribute__((ext_vector_type(4)));
+            u4v *dst = reinterpret_cast<u4v *>(addrT + ((size_t)t * N + c / O) * 64);
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                unsigned word[4];
+#pragma unroll
+                for (int qq = 0; qq < 4; ++qq) {
+                    const int q = q4 * 4 + qq;  // rows 4q .. 4q + 3
+                    unsigned acc = 0u;
+#pragma unroll
+                    for (int j = 0; j < K; ++j) {
+                        const unsigned half = q < 8 ? (unsigned)w[j] : (unsigned)(w[j] >> 32);
+                        const unsigned nib = (half >> (4 * (q & 7))) & 0xFu;
+                        acc |= ((nib * 0x204081u) & 0x01010101u) << j;
+                    }
+                    word[qq] = acc;
+                }
+                const u4v v = {word[0], word[1], word[2], word[3]};
+                dst[q4] = v;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < K; ++j) w[j] = wn[j];
+    }
+}
+
+template <int K>
+static void dwn_launch_eval_bitsliced(const u64 *planes, const int *idx32, const float *luts, u64 *planes_out, int B, int I,
+                                      int N, int O, hipStream_t s, uint8_t *addrT = nullptr) {
+    const int BT = dwn_bt(B);
+    const int col_blocks = dl_ceil_div((long long)N * O, 256);
+    int chunks = col_blocks >= 2048 ? 1 : 2048 / col_blocks;  // about 2048 blocks, each long enough to repay its tables
+    if (chunks > BT) chunks = BT;
+    const int tpb = dl_ceil_div(BT, chunks);
+    if (addrT)
+        DL_TIMED("dwn_fwd_bitsliced", s, (dwn_eval_bitsliced<K, true><<<dim3(col_blocks, dl_ceil_div(BT, tpb)), 256, 0, s>>>(
+                                             planes, idx32, luts, planes_out, B, I, N, O, BT, tpb, addrT)));
+    else
+        DL_TIMED("dwn_eval_bitsliced", s, (dwn_eval_bitsliced<K><<<dim3(col_blocks, dl_ceil_div(BT, tpb)), 256, 0, s>>>(
+                                              planes, idx32, luts, planes_out, B, I, N, O, BT, tpb)));
+}
+
+// ---------------------------------------------------------------------------------
 // Chained layers: activations between two DWN layers never take their [B, N] fp32 form.
 extern "C" size_t dl_dwn_planes_bytes(int B, int C) { return (B > 0 && C > 0) ? dwn_planes_bytes(B, C) : 256; }
 extern "C" size_t dl_dwn_tiled_bytes(int B, int C) {
@@ -990,6 +1100,17 @@ extern "C" int dl_dwn_layer_fwd_planes(const void *planes_in, const int32_t *idx
     const u64 *planes = (const u64 *)planes_in;
     uint8_t *addrT = (uint8_t *)saved;
     u64 *po = (u64 *)planes_out;
+    if (!y) {  // a hidden layer of a chain: only planes and saved addresses leave it - the bit-sliced form
+        switch (k) {
+            case 1: dwn_launch_eval_bitsliced<1>(planes, idx32, luts, po, B, I, N, O, s, addrT); break;
+            case 2: dwn_launch_eval_bitsliced<2>(planes, idx32, luts, po, B, I, N, O, s, addrT); break;
+            case 3: dwn_launch_eval_bitsliced<3>(planes, idx32, luts, po, B, I, N, O, s, addrT); break;
+            case 4: dwn_launch_eval_bitsliced<4>(planes, idx32, luts, po, B, I, N, O, s, addrT); break;
+            case 5: dwn_launch_eval_bitsliced<5>(planes, idx32, luts, po, B, I, N, O, s, addrT); break;
+            default: dwn_launch_eval_bitsliced<6>(planes, idx32, luts, po, B, I, N, O, s, addrT); break;
+        }
+        return dl_launch_status();
+    }
     switch (k) {
         case 1: dwn_launch_lookup<1>(planes, idx32, luts, y, addrT, po, B, I, N, O, s); break;
         case 2: dwn_launch_lookup<2>(planes, idx32, luts, y, addrT, po, B, I, N, O, s); break;
@@ -1056,86 +1177,6 @@ extern "C" int dl_dwn_layer_fwd_planes_groups(const void *planes_in, const int32
 }
 
 // ---- inference on binary activations
-// ---------------------------------------------------------------------------------
-// Bit-sliced inference for a layer between two bit-plane tensors.  Lanes are NODES here: a lane keeps its column's
-// truth table as 2^k bits (table entry >= 0.5), fetches the k plane words of its inputs for a batch tile (64 rows in
-// one 64-bit word each) and evaluates the table on all 64 rows at once as a multiplexer tree of bitwise operations:
-// level j halves the table with the word of input j,  v[i] = v[2i] ^ ((v[2i] ^ v[2i+1]) & x_j).  About 6 vector
-// instructions per (node, tile) instead of 13 vector + 26 scalar in the lookup kernel, and the result of a lane is
-// already the plane word of its column.  A block takes 256 columns and walks `tiles_per_block` tiles with the same
-// indices and tables in registers.
-template <int K>
-__global__ __launch_bounds__(256) void dwn_eval_bitsliced(const u64 *__restrict__ planes, const int *__restrict__ idx32,
-                                                           const float *__restrict__ luts, u64 *__restrict__ planes_out,
-                                                           int B, int I, int N, int O, int BT, int tiles_per_block) {
-    constexpr int L = 1 << K;
-    const int NO = N * O;
-    const int lane = threadIdx.x & 63;
-    const int wave = dl_uniform(threadIdx.x >> 6);
-    const int wc0 = (blockIdx.x * 4 + wave) * 64;  // my wavefront's first column
-    if (wc0 >= NO) return;
-    const int c = min(wc0 + lane, NO - 1);
-    // truth tables of the wavefront's 64 columns: row u of the tables is read with lane = entry and voted on
-    unsigned t_lo = 0u, t_hi = 0u;
-    for (int u = 0; u < 64; ++u) {
-        const int cu = min(wc0 + u, NO - 1);
-        const float v = lane < L ? luts[(size_t)cu * L + lane] : 0.0f;
-        const u64 bits = __ballot(v >= 0.5f);
-        if (lane == u) { t_lo = (unsigned)bits; t_hi = (unsigned)(bits >> 32); }
-    }
-    int off[K];  // word offsets of my inputs inside a tile's planes
-#pragma unroll
-    for (int j = 0; j < K; ++j) off[j] = idx32[(size_t)(c / O) * K + j];
-    const int t_begin = blockIdx.y * tiles_per_block;
-    const int t_end = min(BT, t_begin + tiles_per_block);
-    u64 w[K], wn[K];
-    auto fetch = [&](int t, u64 (&dst)[K]) {
-#pragma unroll
-        for (int j = 0; j < K; ++j) dst[j] = planes[(size_t)t * I + off[j]];
-    };
-    if (t_begin < t_end) fetch(t_begin, w);
-    for (int t = t_begin; t < t_end; ++t) {
-        if (t + 1 < t_end) fetch(t + 1, wn);
-        unsigned vlo[L / 2 > 0 ? L / 2 : 1], vhi[L / 2 > 0 ? L / 2 : 1];
-        const unsigned x0lo = (unsigned)w[0], x0hi = (unsigned)(w[0] >> 32);
-#pragma unroll
-        for (int i = 0; i < L / 2; ++i) {  // level of input 0: the leaves are table bits, spread to 0 / ~0
-            const unsigned src0 = (2 * i < 32) ? t_lo : t_hi, src1 = (2 * i + 1 < 32) ? t_lo : t_hi;
-            const unsigned m0 = (unsigned)__builtin_amdgcn_sbfe((int)src0, (2 * i) & 31, 1);
-            const unsigned m1 = (unsigned)__builtin_amdgcn_sbfe((int)src1, (2 * i + 1) & 31, 1);
-            const unsigned d = m0 ^ m1;
-            vlo[i] = m0 ^ (d & x0lo);
-            vhi[i] = m0 ^ (d & x0hi);
-        }
-#pragma unroll
-        for (int j = 1; j < K; ++j) {
-            const unsigned xlo = (unsigned)w[j], xhi = (unsigned)(w[j] >> 32);
-#pragma unroll
-            for (int i = 0; i < (L >> (j + 1)); ++i) {
-                vlo[i] = vlo[2 * i] ^ ((vlo[2 * i] ^ vlo[2 * i + 1]) & xlo);
-                vhi[i] = vhi[2 * i] ^ ((vhi[2 * i] ^ vhi[2 * i + 1]) & xhi);
-            }
-        }
-        const int rows = min(64, B - t * 64);  // rows past B stay 0, like the planes packed from x
-        const u64 valid = rows == 64 ? ~0ull : ((1ull << rows) - 1ull);
-        if (wc0 + lane < NO) planes_out[(size_t)t * NO + wc0 + lane] = (((u64)vhi[0] << 32) | vlo[0]) & valid;
-#pragma unroll
-        for (int j = 0; j < K; ++j) w[j] = wn[j];
-    }
-}
-
-template <int K>
-static void dwn_launch_eval_bitsliced(const u64 *planes, const int *idx32, const float *luts, u64 *planes_out, int B, int I,
-                                      int N, int O, hipStream_t s) {
-    const int BT = dwn_bt(B);
-    const int col_blocks = dl_ceil_div((long long)N * O, 256);
-    int chunks = col_blocks >= 2048 ? 1 : 2048 / col_blocks;  // about 2048 blocks, each long enough to repay its tables
-    if (chunks > BT) chunks = BT;
-    const int tpb = dl_ceil_div(BT, chunks);
-    DL_TIMED("dwn_eval_bitsliced", s, (dwn_eval_bitsliced<K><<<dim3(col_blocks, dl_ceil_div(BT, tpb)), 256, 0, s>>>(
-                                          planes, idx32, luts, planes_out, B, I, N, O, BT, tpb)));
-}
-
 extern "C" int dl_dwn_layer_eval_planes(const void *planes_in, const int32_t *idx32, const float *luts, float *y,
                                         void *planes_out, int B, int I, int N, int k, int O, void *stream) {
     if (!planes_in || !idx32 || !luts || (!y && !planes_out)) return DL_ERR_NULL;
