@@ -320,7 +320,9 @@ def test_full_size_soft_mapping_b512_i3136_m48000(precision):
 
 
 @pytest.mark.parametrize("shape", [((70, 50), [40, 33, 20], 6), ((130, 64), [128, 64], 4), ((64, 30), [25], 3),
-                                   ((200, 96), [300, 150, 75, 10], 6)])
+                                   ((200, 96), [300, 150, 75, 10], 6),
+                                   # wide hidden layer, ragged batch: the bit-sliced forward walks several tiles per block
+                                   ((4100, 96), [16000, 300], 6)])
 @pytest.mark.parametrize("input_grad", [True, False])
 def test_dwn_stack_equals_layer_by_layer(shape, input_grad):
     """Chained execution (bit-planes forward, tile-major gradients backward) against the same layers
@@ -353,8 +355,10 @@ def test_dwn_stack_equals_layer_by_layer(shape, input_grad):
     y = stack(xb)
     assert torch.equal(y.detach(), want_y)
     y.backward(gy)
+    # a bin of the table gradient sums about B / 2^k values of size ~1 and its blocks flush with atomics in any order:
+    # the floor is a few fp32 ulps of that sum
     for layer, want in zip(layers, want_gl):
-        torch.testing.assert_close(layer._banks["luts"].flat.grad, want, rtol=1e-5, atol=1e-6)
+        torch.testing.assert_close(layer._banks["luts"].flat.grad, want, rtol=1e-5, atol=max(1e-6, 2.5e-9 * B))
     if input_grad:
         torch.testing.assert_close(xb.grad, want_gx, rtol=1e-5, atol=2e-6)
     # eval mode and non-chainable members fall back to the members' own forward
