@@ -184,6 +184,63 @@ def test_smallest_training_configuration_end_to_end(golden):
                                rtol=1e-5, atol=1e-7)
 
 
+def test_first_benchmark_configuration_full_size_against_oracle():
+    """The reference's CPU-runnable configuration at its full size: U[0,1] inputs [256, 784] -> thermometer with 4
+    thresholds -> 3136 bits -> RandomLayer(seed 42, k = 6) -> 2000 DWN nodes, tables U[-1,1] -> GroupSum into 10
+    classes -> cross-entropy on random labels, one forward + backward.  Module by module and as one DWNStack
+    (thermometer and GroupSum folded into the layer's kernels) against the oracle: bits, mapping table, layer output
+    and logits bit-exact / to 1e-6, table gradients to rtol 1e-5."""
+    REGISTRY, NodeConfig, uniform_init, _ = _api()
+    from difflut_amd.layers import DWNStack
+    from difflut_amd.utils import GroupSum
+    torch.manual_seed(0)
+    B, F, NB, N, k, G = 256, 784, 4, 2000, 6, 10
+    x = torch.rand(B, F)
+    labels = torch.randint(0, G, (B,))
+    thr = orc.thermometer_fit(x.numpy(), NB)
+    bits = orc.thermometer_encode(x.numpy(), thr).reshape(B, F * NB).astype(np.float32)
+    layer = REGISTRY.get_layer("random")(F * NB, N, REGISTRY.get_node("dwn"),
+                                         NodeConfig(input_dim=k, output_dim=1, init_fn=uniform_init,
+                                                    init_kwargs={"a": -1.0, "b": 1.0}), seed=42).cuda()
+    idx = layer._mapping_indices.cpu().numpy().astype(np.int64)
+    assert np.array_equal(idx, orc.random_mapping(F * NB, N, k, seed=42).numpy().astype(np.int64))
+    luts = stacked(layer, "luts")
+    alpha, beta = float(layer.nodes[0].alpha), float(layer.nodes[0].beta)
+    # oracle: forward, logits, loss and the gradient that reaches the tables
+    want_y = c_oracle.dwn_layer_forward(bits, idx, luts).reshape(B, N)
+    want_logits = orc.group_sum(want_y, G, 1.0)
+    lt = torch.tensor(want_logits, dtype=torch.float64, requires_grad=True)
+    want_loss = torch.nn.functional.cross_entropy(lt, labels)
+    want_loss.backward()
+    g_y = np.repeat(lt.grad.numpy(), N // G, axis=1).astype(np.float32).reshape(B, N, 1)
+    _, want_gl = c_oracle.dwn_layer_backward(bits, idx, luts, g_y, alpha, beta)
+    # module by module
+    xd = x.cuda()
+    enc = REGISTRY.build_encoder("thermometer", num_bits=NB).fit(xd)
+    got_bits = enc.encode(xd)
+    assert np.array_equal(got_bits.cpu().numpy().reshape(B, -1), bits)
+    y = layer(got_bits)
+    assert np.array_equal(y.detach().cpu().numpy(), want_y)
+    head = GroupSum(k=G, tau=1.0, use_randperm=False)
+    logits = head(y)
+    np.testing.assert_allclose(logits.detach().cpu().numpy(), want_logits, rtol=1e-6, atol=1e-5)  # sums of 200 values
+    loss = torch.nn.functional.cross_entropy(logits, labels.cuda())
+    assert loss.item() == pytest.approx(want_loss.item(), rel=1e-6)
+    loss.backward()
+    got_gl = torch.stack([n.luts.grad for n in layer.nodes]).cpu().numpy()
+    np.testing.assert_allclose(got_gl, want_gl, rtol=1e-5, atol=1e-8)  # a bin holds ~4 terms of size ~1e-3
+    # the same step as one chained call
+    layer._banks["luts"].flat.grad = None
+    for n in layer.nodes:
+        n.luts.grad = None
+    stack = DWNStack([layer], encoder=enc, head=head).train()
+    logits2 = stack(xd)
+    np.testing.assert_allclose(logits2.detach().cpu().numpy(), want_logits, rtol=1e-6, atol=1e-5)
+    torch.nn.functional.cross_entropy(logits2, labels.cuda()).backward()
+    np.testing.assert_allclose(layer._banks["luts"].flat.grad.cpu().numpy().reshape(want_gl.shape), want_gl,
+                               rtol=1e-5, atol=1e-8)
+
+
 def test_adam_steps_change_tables_in_place():
     REGISTRY, NodeConfig, uniform_init, _ = _api()
     layer = REGISTRY.get_layer("random")(64, 40, REGISTRY.get_node("dwn"), NodeConfig(input_dim=6, output_dim=1),
