@@ -70,7 +70,8 @@ __global__ __launch_bounds__(256) void dwn_pack_planes(const float *__restrict__
         for (int r = 0; r < DWN_PACK_ROWS; ++r) {
             const float *src = base + (size_t)r * I;
             if constexpr (VEC == 4) {
-                const float4 q = *reinterpret_cast<const float4 *>(src);
+                typedef float f4v __attribute__((ext_vector_type(4)));
+                const f4v q = __builtin_nontemporal_load(reinterpret_cast<const f4v *>(src));  // x is read once
                 acc[0] |= (q.x >= 0.5f ? 1u : 0u) << r;
                 acc[1] |= (q.y >= 0.5f ? 1u : 0u) << r;
                 acc[2] |= (q.z >= 0.5f ? 1u : 0u) << r;
@@ -79,7 +80,7 @@ __global__ __launch_bounds__(256) void dwn_pack_planes(const float *__restrict__
                     odd = odd || !((q.x == 0.0f || q.x == 1.0f) && (q.y == 0.0f || q.y == 1.0f) &&
                                    (q.z == 0.0f || q.z == 1.0f) && (q.w == 0.0f || q.w == 1.0f));
             } else {
-                const float v0 = src[0];
+                const float v0 = __builtin_nontemporal_load(src);
                 acc[0] |= (v0 >= 0.5f ? 1u : 0u) << r;
                 if (CHECK) odd = odd || !(v0 == 0.0f || v0 == 1.0f);
             }
@@ -390,7 +391,9 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
             if (b < B) {
                 const float *src = gy + (size_t)b * NO + c0 + q * 4;
                 if (vec4) {
-                    pre[p] = *reinterpret_cast<const float4 *>(src);
+                    typedef float f4v __attribute__((ext_vector_type(4)));
+                    const f4v g4 = __builtin_nontemporal_load(reinterpret_cast<const f4v *>(src));  // gy is read once
+                    pre[p] = make_float4(g4.x, g4.y, g4.z, g4.w);
                 } else {
                     if (q * 4 + 0 < cend) pre[p].x = src[0];
                     if (q * 4 + 1 < cend) pre[p].y = src[1];
