@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # (FETCH_SIZE scaled by 2.0 after calibration against a plain copy, plus WRITE_SIZE; the runs and
 # the calibration are written up under profiles/).  Measured, not computed: None where no run exists.
 MEASURED_TRAFFIC = {
-    ("dwn_k6_b4096_i16384_n8192", "dwn_bwd_gx"): 906390118,  # (304.2 * 2 + 256.0) MiB
+    ("dwn_k6_b4096_i16384_n8192", "dwn_bwd_gx"): 901565644,  # (301.9 * 2 + 256.0) MiB
 }
 
 WORKLOADS = {
