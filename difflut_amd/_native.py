@@ -26,6 +26,7 @@ SIGNATURES = {
     "dl_dwn_fwd_workspace_bytes": (_Z, [_I] * 5),
     "dl_dwn_bwd_workspace_bytes": (_Z, [_I] * 5),
     "dl_dwn_layer_fwd": (_I, [_P, _P, _P, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
+    "dl_dwn_layer_fwd_static": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "dl_dwn_layer_bwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _F, _F, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
     "dl_dwn_layer_eval": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "dl_dwn_planes_bytes": (_Z, [_I] * 2),

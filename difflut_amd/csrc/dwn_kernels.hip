@@ -21,6 +21,7 @@
 //                           gx[b,i] = sum gyT[c][b] * D[c][j][a'(b)]  - a gather in fixed order
 // k > 6 goes to the one-thread-per-element kernels of dwn_generic.hip.
 #include "dl_common.h"
+#include <mutex>
 #include <type_traits>
 #include "dwn_generic.h"
 
@@ -785,16 +786,9 @@ static void dwn_launch_lookup(const u64 *planes, const int *idx32, const float *
 #undef DWN_LOOKUP
 }
 
-extern "C" int dl_dwn_layer_fwd(const float *x, const int32_t *idx32, const float *luts, float *y, void *saved,
-                                void *ws, size_t ws_bytes, int B, int I, int N, int k, int O, void *stream) {
-    if (!x || !idx32 || !luts || !y) return DL_ERR_NULL;
-    int rc = dwn_check(B, I, N, k, O);
-    if (rc) return rc;
-    hipStream_t s = (hipStream_t)stream;
-    if (!dwn_fast(N, k, O)) return dwn_generic_forward(x, idx32, luts, y, B, I, N, k, O, s);
-    if (!saved || !ws) return DL_ERR_NULL;
-    if (ws_bytes < dl_dwn_fwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
-    u64 *planes = (u64 *)ws;
+// forward of the k <= 6 path: x -> bit-planes (scratch) -> y and the saved addresses
+static int dwn_forward_fast(const float *x, const int32_t *idx32, const float *luts, float *y, void *saved, u64 *planes,
+                            int B, int I, int N, int k, int O, hipStream_t s) {
     const int BT = dwn_bt(B);
     if (I % 4 == 0 && ((uintptr_t)x & 15) == 0)
         DL_TIMED("dwn_pack_planes", s, (dwn_pack_planes<4><<<dim3(dl_ceil_div(I, 1024), 4 * BT), 256, 0, s>>>(x, planes, B, I)));
@@ -810,6 +804,60 @@ extern "C" int dl_dwn_layer_fwd(const float *x, const int32_t *idx32, const floa
         default: dwn_launch_lookup<6>(planes, idx32, luts, y, addrT, nullptr, B, I, N, O, s); break;
     }
     return dl_launch_status();
+}
+
+extern "C" int dl_dwn_layer_fwd(const float *x, const int32_t *idx32, const float *luts, float *y, void *saved,
+                                void *ws, size_t ws_bytes, int B, int I, int N, int k, int O, void *stream) {
+    if (!x || !idx32 || !luts || !y) return DL_ERR_NULL;
+    int rc = dwn_check(B, I, N, k, O);
+    if (rc) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    if (!dwn_fast(N, k, O)) return dwn_generic_forward(x, idx32, luts, y, B, I, N, k, O, s);
+    if (!saved || !ws) return DL_ERR_NULL;
+    if (ws_bytes < dl_dwn_fwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
+    return dwn_forward_fast(x, idx32, luts, y, saved, (u64 *)ws, B, I, N, k, O, s);
+}
+
+// ---- the same forward for callers that cannot allocate a workspace.  The bit-planes go to a device array that
+// belongs to the library: every GPU the library runs on holds its own copy of it (DL_DWN_STATIC_SCRATCH_BYTES, until
+// the process ends) at its own address, looked up once per device.  `scratch` itself is only the host-side handle
+// of the symbol - kernels are always given the looked-up device address.
+static __device__ __align__(256) unsigned char scratch[DL_DWN_STATIC_SCRATCH_BYTES];
+#define DWN_MAX_DEVICES 64
+static void *g_scratch_ptr[DWN_MAX_DEVICES];  // device address of `scratch` on each device, null until looked up
+static std::mutex g_scratch_mutex;
+
+static int dwn_scratch_address(void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= DWN_MAX_DEVICES) return DL_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));  // the current device's copy
+        if (e != hipSuccess) return (int)e;
+        if (!p) return DL_ERR_NULL;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return DL_OK;
+}
+
+extern "C" int dl_dwn_layer_fwd_static(const float *x, const int32_t *idx32, const float *luts, float *y, void *saved,
+                                       int B, int I, int N, int k, int O, void *stream) {
+    if (!x || !idx32 || !luts || !y) return DL_ERR_NULL;
+    int rc = dwn_check(B, I, N, k, O);
+    if (rc) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    if (!dwn_fast(N, k, O)) return dwn_generic_forward(x, idx32, luts, y, B, I, N, k, O, s);  // uses no scratch
+    if (!saved) return DL_ERR_NULL;
+    if (dwn_planes_bytes(B, I) > (size_t)DL_DWN_STATIC_SCRATCH_BYTES) return DL_ERR_SCRATCH;
+    void *planes = nullptr;
+    rc = dwn_scratch_address(&planes);
+    if (rc) return rc;
+    // every plane word of the ceil(B/64) tiles is rewritten by the pack kernel, so nothing has to be cleared
+    return dwn_forward_fast(x, idx32, luts, y, saved, (u64 *)planes, B, I, N, k, O, s);
 }
 
 template <int K>

@@ -316,6 +316,7 @@ extern "C" const char *dl_error_string(int code) {
         case DL_ERR_UNSUPPORTED: return "k, O or an option is outside what the kernels cover";
         case DL_ERR_WORKSPACE: return "workspace is smaller than the matching *_workspace_bytes()";
         case DL_ERR_INDEX: return "an index is outside [0, I)";
+        case DL_ERR_SCRATCH: return "the call needs more scratch than the library's static device array holds";
         default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
     }
 }

@@ -35,6 +35,7 @@ extern "C" {
 #define DL_ERR_UNSUPPORTED (-3) /* k, O or an option outside what the kernels cover */
 #define DL_ERR_WORKSPACE (-4)   /* workspace smaller than the matching *_workspace_bytes() */
 #define DL_ERR_INDEX (-5)       /* an index table entry is outside [0, I) (host-checked entry points only) */
+#define DL_ERR_SCRATCH (-6)     /* dl_dwn_layer_fwd_static: the call needs more than DL_DWN_STATIC_SCRATCH_BYTES */
 
 #define DL_MAX_FAST_K 6  /* tables of up to 64 entries sit one-per-lane in a wavefront */
 #define DL_MAX_K 16      /* generic kernels */
@@ -80,6 +81,18 @@ size_t dl_dwn_bwd_workspace_bytes(int B, int I, int N, int k, int O);
 int dl_dwn_layer_fwd(const float *x, const int32_t *idx32, const float *luts, float *y,
                      void *saved, void *ws, size_t ws_bytes,
                      int B, int I, int N, int k, int O, void *stream);
+/* dl_dwn_layer_fwd for callers that cannot allocate device memory at all - code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc - and so cannot bring a workspace either.  It has no
+ * counterpart in the reference.  Same arguments minus `ws`, same kernels, same results: the bit-planes that
+ * dl_dwn_layer_fwd puts into `ws` go to a device array owned by the library instead
+ * (DL_DWN_STATIC_SCRATCH_BYTES on every GPU the library runs on, held until the process ends).  The call
+ * allocates and frees nothing.  Limit: ceil(B/64) * I * 8 <= DL_DWN_STATIC_SCRATCH_BYTES when
+ * k <= DL_MAX_FAST_K (e.g. B = 4096 with I = 16384), otherwise DL_ERR_SCRATCH; larger k uses no scratch.
+ * All calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams, two threads)
+ * race on it and must be serialised by the caller.  Nothing in it has to survive between calls. */
+#define DL_DWN_STATIC_SCRATCH_BYTES (8u << 20)
+int dl_dwn_layer_fwd_static(const float *x, const int32_t *idx32, const float *luts, float *y,
+                            void *saved, int B, int I, int N, int k, int O, void *stream);
 /* Extended-finite-difference backward (dwn_node.py:167-229):
  *   gx[b,i]     = sum_{(n,j): idx=i} alpha * sum_d gy[b,n,d] *
  *                 sum_kappa s(kappa_j) luts[n,d,kappa] beta^popc((addr ^ kappa) & ~(1<<j))
