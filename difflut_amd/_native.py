@@ -28,6 +28,7 @@ SIGNATURES = {
     "dl_dwn_layer_fwd": (_I, [_P, _P, _P, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
     "dl_dwn_layer_fwd_static": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "dl_dwn_layer_bwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _F, _F, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
+    "dl_dwn_layer_bwd_nodes": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
     "dl_dwn_layer_eval": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "dl_dwn_planes_bytes": (_Z, [_I] * 2),
     "dl_dwn_tiled_bytes": (_Z, [_I] * 2),

@@ -28,7 +28,8 @@ __global__ __launch_bounds__(256) void dwn_generic_bwd_gx(const float *__restric
                                                            const int *__restrict__ inv_ptr, const int *__restrict__ inv_pos,
                                                            const float *__restrict__ luts, const float *__restrict__ gy,
                                                            float alpha, float beta, const float *__restrict__ scale,
-                                                           float *__restrict__ gx, int B, int I, int N, int K, int O) {
+                                                           float *__restrict__ gx, int B, int I, int N, int K, int O,
+                                                           const float *__restrict__ alpha_n, const float *__restrict__ beta_n) {
     const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
     if (gid >= (long long)B * I) return;
     const int b = (int)(gid / I), i = (int)(gid % I);
@@ -42,6 +43,9 @@ __global__ __launch_bounds__(256) void dwn_generic_bwd_gx(const float *__restric
         const int n = p / K, j = p - n * K;
         const unsigned a = dwn_addr_generic(x + (size_t)b * I, idx32 + (size_t)n * K, K);
         const unsigned keep = ~(1u << j);
+        if (beta_n)  // the node's own beta
+            for (int h = 1; h <= K; ++h) bp[h] = bp[h - 1] * (double)beta_n[n];
+        const double al = scale ? (double)scale[n] : (alpha_n ? (double)alpha_n[n] : (double)alpha);
         for (int d = 0; d < O; ++d) {
             const float *lut = luts + (((size_t)n * O + d) << K);
             double s = 0.0;
@@ -49,7 +53,7 @@ __global__ __launch_bounds__(256) void dwn_generic_bwd_gx(const float *__restric
                 const double w = bp[__popc((a ^ (unsigned)kap) & keep)];
                 s += (((unsigned)kap >> j) & 1u) ? (double)lut[kap] * w : -(double)lut[kap] * w;
             }
-            acc += gy[((size_t)b * N + n) * O + d] * (float)((scale ? (double)scale[n] : (double)alpha) * s);
+            acc += gy[((size_t)b * N + n) * O + d] * (float)(al * s);
         }
     }
     gx[gid] = acc;
@@ -103,13 +107,13 @@ int dwn_generic_forward(const float *x, const int *idx32, const float *luts, flo
 
 int dwn_generic_backward(const float *x, const int *idx32, const int *inv_ptr, const int *inv_pos, const float *luts,
                          const float *gy, float alpha, float beta, const float *scale, float *gx, float *gluts, int B, int I,
-                         int N, int k, int O, hipStream_t s) {
+                         int N, int k, int O, hipStream_t s, const float *alpha_n, const float *beta_n) {
     const long long NO = (long long)N * O;
     dwn_generic_zero<<<dl_ceil_div(NO << k, 256), 256, 0, s>>>(gluts, NO << k);
     dwn_generic_bwd_luts<<<dl_ceil_div((long long)B * NO, 256), 256, 0, s>>>(x, idx32, gy, scale, gluts, B, I, N, k, O);
     if (gx)
         dwn_generic_bwd_gx<<<dl_ceil_div((long long)B * I, 256), 256, 0, s>>>(x, idx32, inv_ptr, inv_pos, luts, gy, alpha,
-                                                                            beta, scale, gx, B, I, N, k, O);
+                                                                            beta, scale, gx, B, I, N, k, O, alpha_n, beta_n);
     return dl_launch_status();
 }
 

@@ -261,12 +261,16 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
 //           D[c][j][a'] = S[c][a | bit j] - S[c][a & ~bit j].  Cheaper to build, a third of the
 //           memory, shared by the k slots of a node - but it amplifies rounding by
 //           (1+|beta|)^k / (1-beta), so it is only used for |beta| <= 1/2 (the default is 1/3).
+// alpha_n / beta_n (nullable): the nodes' own alpha and beta [N] instead of one value for the layer.
 __global__ __launch_bounds__(256) void dwn_efd_table(const float *__restrict__ luts, float *__restrict__ D,
                                                       float *__restrict__ gluts, int NO, int K, float alpha, float beta,
-                                                      int sform) {
+                                                      int sform, const float *__restrict__ alpha_n = nullptr,
+                                                      const float *__restrict__ beta_n = nullptr, int O = 1) {
     const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int a = threadIdx.x & 63;
     if (c >= NO) return;
+    if (alpha_n) alpha = alpha_n[c / O];
+    if (beta_n) beta = beta_n[c / O];
     const int L = 1 << K, Lh = L >> 1;
     const bool live = a < L;
     const double v0 = live ? (double)luts[(size_t)c * L + a] : 0.0;
@@ -901,7 +905,8 @@ struct DwnGroupHead {
 static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos, const float *luts,
                              const float *gy, int gy_tiled, float alpha, float beta, const float *scale, float *gx,
                              int gx_tiled, float *gluts, void *ws, int B, int I, int N, int k, int O, hipStream_t s,
-                             const DwnGroupHead *head = nullptr) {
+                             const DwnGroupHead *head = nullptr, const float *alpha_n = nullptr,
+                             const float *beta_n = nullptr) {
     const long long NO = (long long)N * O;
     const int L = 1 << k;
     const uint8_t *addrT = (const uint8_t *)saved;
@@ -924,7 +929,8 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
                  (dwn_stable_table<<<dl_ceil_div(NO, 4), 256, 0, s>>>(luts, scale, D, gluts, (int)NO, k, O)));
     else if (gx)
         DL_TIMED("dwn_efd_table", s,
-                 (dwn_efd_table<<<dl_ceil_div(NO, 4), 256, 0, s>>>(luts, D, gluts, (int)NO, k, alpha, beta, sform ? 1 : 0)));
+                 (dwn_efd_table<<<dl_ceil_div(NO, 4), 256, 0, s>>>(luts, D, gluts, (int)NO, k, alpha, beta, sform ? 1 : 0,
+                                                                  alpha_n, beta_n, O)));
     else
         dl_fill_zero(gluts, NO * L, s);
     if (head)
@@ -973,6 +979,29 @@ extern "C" int dl_dwn_layer_bwd(const float *x, const void *saved, const int32_t
     if (!saved || !ws) return DL_ERR_NULL;
     if (ws_bytes < dl_dwn_bwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
     return dwn_backward_fast(saved, inv_ptr, inv_pos, luts, gy, 0, alpha, beta, nullptr, gx, 0, gluts, ws, B, I, N, k, O, s);
+}
+
+// The same backward with every node's own alpha and beta (device arrays [N]); beta_abs_max = max |beta_n| decides
+// which form of the coefficient table is safe for all nodes.
+extern "C" int dl_dwn_layer_bwd_nodes(const float *x, const void *saved, const int32_t *idx32, const int32_t *inv_ptr,
+                                      const int32_t *inv_pos, const float *luts, const float *gy, const float *alpha_n,
+                                      const float *beta_n, float beta_abs_max, float *gx, float *gluts, void *ws,
+                                      size_t ws_bytes, int B, int I, int N, int k, int O, void *stream) {
+    if (!idx32 || !luts || !gy || !gluts || !alpha_n || !beta_n) return DL_ERR_NULL;
+    if (gx && (!inv_ptr || !inv_pos)) return DL_ERR_NULL;
+    int rc = dwn_check(B, I, N, k, O);
+    if (rc) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    if (!dwn_fast(N, k, O)) {
+        if (!x) return DL_ERR_NULL;
+        return dwn_generic_backward(x, idx32, inv_ptr, inv_pos, luts, gy, 0.0f, 0.0f, nullptr, gx, gluts, B, I, N, k, O, s,
+                                    alpha_n, beta_n);
+    }
+    if (!saved || !ws) return DL_ERR_NULL;
+    if (ws_bytes < dl_dwn_bwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
+    // beta handed to the form choice only: |beta| <= 1/2 for every node -> the shared 64-entry form
+    return dwn_backward_fast(saved, inv_ptr, inv_pos, luts, gy, 0, 0.0f, beta_abs_max, nullptr, gx, 0, gluts, ws, B, I, N, k,
+                             O, s, nullptr, alpha_n, beta_n);
 }
 
 extern "C" int dl_dwn_stable_layer_bwd(const float *x, const void *saved, const int32_t *idx32, const int32_t *inv_ptr,

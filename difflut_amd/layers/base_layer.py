@@ -13,7 +13,13 @@ users, optimisers and state_dict see (`nodes.{i}.luts`, ...) are views into that
     `.grad` reads row i of `flat.grad`, so optimisers update the shared storage in place
     and no per-node gradient copies are made;
   * `Module._apply` (.to/.cuda/.float) re-allocates parameters one by one, so the layer
-    re-ties them after every `_apply`.
+    re-ties them after every `_apply`; `copy.deepcopy` and unpickling re-tie in `__setstate__`, so the
+    objects `parameters()` yields are final before the first forward (an optimizer built right after
+    a copy or a load keeps working).
+The per-node scalar buffers the fused kernels need (`alpha`, `beta`, `temperature`) are banked the same way
+(`ScalarBank`: one [N] tensor, each node's 0-dim buffer a view of it), so a state dict or an in-place edit that
+gives nodes different values is seen by the layer: DWN layers then hand the kernels the per-node arrays, the
+other fused paths refuse to run rather than use one node's value for all.
 """
 import warnings
 from abc import ABC, abstractmethod
@@ -71,10 +77,15 @@ class ParameterBank:
     def __init__(self, nodes, name):
         self.nodes, self.name = nodes, name
         self.flat = None
+        self._stale = False  # set when another bank takes over one of my nodes, or a node's parameter is reassigned
         self.tie()
 
     def tie(self, keep_grad=None):
         params = [node._parameters[self.name] for node in self.nodes]
+        for p in params:  # a bank that held one of these nodes (a sub-layer's own, a level's) no longer does
+            other = getattr(p, "_bank", None)
+            if other is not None and other is not self:
+                other._stale = True
         flat = torch.stack([p.data for p in params]).contiguous()
         flat.requires_grad_(True)
         if keep_grad is not None:
@@ -83,8 +94,11 @@ class ParameterBank:
         view = flat.detach()
         for row, node in enumerate(self.nodes):
             node._parameters[self.name] = BankedParameter(view[row], self, row)
+        self._stale = False
 
     def tied(self):
+        if self._stale:
+            return False
         first = self.nodes[0]._parameters[self.name]
         last = self.nodes[-1]._parameters[self.name]
         step = self.flat[0].numel() * self.flat.element_size()
@@ -96,6 +110,52 @@ class ParameterBank:
         if not self.tied():
             self.tie()
         return self.flat
+
+
+class ScalarBank:
+    """The 0-dim buffer `name` of N nodes as one tensor [N]; each node's buffer is a view of its entry, so
+    `load_state_dict` and in-place edits land in the bank.  `summary()` is the host's view of it, read back
+    only when the bank's version changes: (all entries equal, first value, largest magnitude)."""
+
+    def __init__(self, nodes, name):
+        self.nodes, self.name = nodes, name
+        self.flat, self._stale, self._key, self._summary = None, False, None, None
+        self.tie()
+
+    def tie(self):
+        bufs = [node._buffers[self.name] for node in self.nodes]
+        for b in bufs:
+            other = getattr(b, "_scalar_bank", None)
+            if other is not None and other is not self:
+                other._stale = True
+        self.flat = torch.stack([b.detach().reshape(()).to(torch.float32) for b in bufs]).contiguous()
+        for row, node in enumerate(self.nodes):
+            view = self.flat[row]
+            view._scalar_bank = self
+            node._buffers[self.name] = view
+        self._stale, self._key = False, None
+
+    def tied(self):
+        if self._stale:
+            return False
+        first, last = self.nodes[0]._buffers[self.name], self.nodes[-1]._buffers[self.name]
+        base, step = self.flat.data_ptr(), self.flat.element_size()
+        return (first.device == self.flat.device and first.data_ptr() == base
+                and last.data_ptr() == base + step * (len(self.nodes) - 1))
+
+    def tensor(self):
+        if not self.tied():
+            self.tie()
+        return self.flat
+
+    def summary(self):
+        flat = self.tensor()
+        key = (flat._version, flat.data_ptr())
+        if key != self._key:
+            host = flat.detach().cpu()
+            self._summary = (bool((host == host[0]).all()), float(host[0]), float(host.abs().max()))
+            self._key = key
+        return self._summary
 
 
 class LUTLayerMixin(nn.Module):
@@ -173,12 +233,15 @@ class BaseLUTLayer(ABC, LUTLayerMixin, nn.Module):
         self.nodes = nn.ModuleList([node_type(**kwargs) for _ in range(output_size)])
         self.n = self.nodes[0].num_inputs
         self.output_dim_per_node = self.nodes[0].num_outputs
-        self._banks = {}
+        self._banks, self._scalars = {}, {}
         self._fused = self._detect_fused_kind()
         if self._fused == "dwn":
             self._banks["luts"] = ParameterBank(self.nodes, "luts")
+            self._scalars["alpha"] = ScalarBank(self.nodes, "alpha")
+            self._scalars["beta"] = ScalarBank(self.nodes, "beta")
         elif self._fused == "probabilistic":
             self._banks["raw_weights"] = ParameterBank(self.nodes, "raw_weights")
+            self._scalars["temperature"] = ScalarBank(self.nodes, "temperature")
         elif self._fused == "dwn_stable":
             self._banks["raw_luts"] = ParameterBank(self.nodes, "raw_luts")
             self._banks["gradient_scale"] = ParameterBank(self.nodes, "gradient_scale")
@@ -206,7 +269,39 @@ class BaseLUTLayer(ABC, LUTLayerMixin, nn.Module):
         super()._apply(fn, *args, **kwargs)
         for name, bank in self._banks.items():
             bank.tie(keep_grad=None if grads[name] is None else fn(grads[name]))
+        for bank in self._scalars.values():
+            bank.tie()
         return self
+
+    def __setstate__(self, state):
+        # copy.deepcopy and unpickling hand back plain per-node Parameters: tie them to their banks now, so that
+        # what parameters() yields is not replaced by the first forward
+        super().__setstate__(state)
+        self.__dict__.setdefault("_scalars", {})
+        for bank in self._banks.values():
+            bank.nodes = self.nodes
+            bank.tie()
+        for bank in self._scalars.values():
+            bank.nodes = self.nodes
+            bank.tie()
+
+    def efd_scalars(self):
+        """(alpha, beta) of a DWN layer whose nodes all share them, as Python floats.  The paths that take one pair for
+        the whole layer (chained layers, convolutional levels) call this and refuse per-node values."""
+        (a_same, alpha, _), (b_same, beta, _) = self._scalars["alpha"].summary(), self._scalars["beta"].summary()
+        if not (a_same and b_same):
+            raise RuntimeError("the nodes of this layer carry different alpha / beta values; chained and convolutional "
+                               "execution takes one pair per layer - call the layer on its own (RandomLayer.forward "
+                               "passes every node's pair to the kernels)")
+        return alpha, beta
+
+    def temperature_value(self):
+        """The temperature shared by the nodes of a probabilistic layer; per-node temperatures are refused."""
+        same, value, _ = self._scalars["temperature"].summary()
+        if not same:
+            raise RuntimeError("the nodes of this layer carry different temperatures; the fused probabilistic kernels "
+                               "take one temperature per layer")
+        return value
 
     def bank_parameters(self):
         """The layer's trainable tensors with every node parameter as ONE leaf [N, ...] (the storage the
@@ -223,22 +318,26 @@ class BaseLUTLayer(ABC, LUTLayerMixin, nn.Module):
 
     def _run_nodes(self, x, plan):
         """All nodes on x [batch, width] through `plan` (index table over width) -> [batch, N*O]."""
-        first = self.nodes[0]
         if self._fused == "dwn":
             from .. import ops
 
             luts = self._banks["luts"].tensor()
             if self.training:
-                alpha, beta = first.efd_scalars()
-                return ops.DWNLayerFunction.apply(x, luts, plan, alpha, beta)
+                (a_same, alpha, _), (b_same, beta, b_max) = (self._scalars["alpha"].summary(),
+                                                             self._scalars["beta"].summary())
+                if a_same and b_same:
+                    return ops.DWNLayerFunction.apply(x, luts, plan, alpha, beta)
+                # every node's own pair (dwn_node.py:450 reads them per node)
+                return ops.DWNLayerFunction.apply(x, luts, plan, self._scalars["alpha"].tensor(),
+                                                  self._scalars["beta"].tensor(), b_max)
             return ops.dwn_layer_eval(x, luts.detach(), plan)
         if self._fused == "probabilistic":
             from .. import ops
 
             raw = self._banks["raw_weights"].tensor()
             if self.training:
-                return ops.ProbLayerFunction.apply(x, raw, plan, first.temperature_value())
-            return ops.prob_layer_eval(x, raw.detach(), plan, first.temperature_value())
+                return ops.ProbLayerFunction.apply(x, raw, plan, self.temperature_value())
+            return ops.prob_layer_eval(x, raw.detach(), plan, self.temperature_value())
         if self._fused in ("dwn_stable", "hybrid"):
             from .. import ops
 

@@ -129,6 +129,22 @@ class ConvolutionalLayer(LUTLayerMixin, nn.Module):
         self._plans = None
         return self
 
+    def __setstate__(self, state):
+        # after copy.deepcopy / unpickling the per-node Parameters are plain again: tie them to the level banks now
+        super().__setstate__(state)
+        if self._kind is not None:
+            self._tie_levels()
+        self._plans = None
+
+    def _level_scalars(self, level, what):
+        """The value all sub-layers of a depth level share (`efd_scalars` or `temperature_value`): a level runs as one
+        layer call with one value, so differing nodes are refused rather than overridden."""
+        values = {getattr(layer, what)() for layer in self._level_layers(level)}
+        if len(values) != 1:
+            raise RuntimeError(f"the sub-layers of depth level {level} carry different {what.split('_')[0]} values; a level "
+                               "runs as one fused layer call and takes one value")
+        return values.pop()
+
     def bank_parameters(self):
         """One leaf [nodes of the level, ...] per depth level and node parameter (what the fused calls
         differentiate); hand these to an optimizer instead of the per-node `parameters()`."""
@@ -165,25 +181,26 @@ class ConvolutionalLayer(LUTLayerMixin, nn.Module):
         device = patches.device if patches is not None else image.device
         plans = self._level_plans(device)
         banks = [{name: bank.tensor() for name, bank in level.items()} for level in self._level_banks]
-        firsts = [self._level_layers(level)[0].nodes[0] for level in range(self.tree_depth + 1)]
+        levels = range(self.tree_depth + 1)
         kind, h = self._kind, patches
         if image is not None:
-            scalars = [node.efd_scalars() for node in firsts]
+            scalars = [self._level_scalars(level, "efd_scalars") for level in levels]
             return ops.DWNStackFunction.apply(image, self._geometry(), plans, scalars, None, *[b["luts"] for b in banks])
         if kind == "dwn" and self.training and self.n_inputs_per_node <= ops.FAST_K:
-            scalars = [node.efd_scalars() for node in firsts]
+            scalars = [self._level_scalars(level, "efd_scalars") for level in levels]
             return ops.DWNStackFunction.apply(h, None, plans, scalars, None, *[b["luts"] for b in banks])
-        for plan, bank, node in zip(plans, banks, firsts):
+        for level, plan, bank in zip(levels, plans, banks):
             if kind == "dwn":
                 if self.training:
-                    h = ops.DWNLayerFunction.apply(h, bank["luts"], plan, *node.efd_scalars())
+                    h = ops.DWNLayerFunction.apply(h, bank["luts"], plan, *self._level_scalars(level, "efd_scalars"))
                 else:
                     h = ops.dwn_layer_eval(h, bank["luts"].detach(), plan)
             elif kind == "probabilistic":
+                temperature = self._level_scalars(level, "temperature_value")
                 if self.training:
-                    h = ops.ProbLayerFunction.apply(h, bank["raw_weights"], plan, node.temperature_value())
+                    h = ops.ProbLayerFunction.apply(h, bank["raw_weights"], plan, temperature)
                 else:
-                    h = ops.prob_layer_eval(h, bank["raw_weights"].detach(), plan, node.temperature_value())
+                    h = ops.prob_layer_eval(h, bank["raw_weights"].detach(), plan, temperature)
             elif not self.training:
                 with torch.no_grad():
                     h = ops.dwn_layer_eval(h, ops.TableSigmoidFunction.apply(bank["raw_luts"]), plan)

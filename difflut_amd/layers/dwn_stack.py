@@ -89,7 +89,7 @@ class DWNStack(nn.Module):
         if thresholds is None:
             self.layers[0]._validate_input_dims(x)
         plans = [layer.mapping_plan() for layer in self.layers]
-        scalars = [layer.nodes[0].efd_scalars() for layer in self.layers]
+        scalars = [layer.efd_scalars() for layer in self.layers]  # raises when a layer's nodes disagree
         luts = [layer._banks["luts"].tensor() for layer in self.layers]
         if self.head is not None and self._fusable_head():
             return ops.DWNStackFunction.apply(x, thresholds, plans, scalars, (self.head.k, self.head.tau), *luts)

@@ -54,6 +54,18 @@ class BaseNode(nn.Module, ABC):
             raise TypeError(f"init_kwargs must be a dict, but got {type(self.init_kwargs).__name__}")
         self.regularizers = self._checked_regularizers(regularizers)
 
+    def __setattr__(self, name, value):
+        # a parameter or scalar buffer that a layer keeps in a bank is being replaced: the bank must re-tie
+        params = self.__dict__.get("_parameters")
+        if params is not None:
+            old = params.get(name)
+            if old is None:
+                old = self.__dict__["_buffers"].get(name)
+            bank = getattr(old, "_bank", None) or getattr(old, "_scalar_bank", None)
+            if bank is not None:
+                bank._stale = True
+        super().__setattr__(name, value)
+
     @property
     def num_inputs(self):
         return self.input_dim

@@ -125,7 +125,9 @@ class DWNLayerFunction(torch.autograd.Function):
     """y[b, n*O+d] = luts[n,d,addr(b,n)] with the extended-finite-difference backward."""
 
     @staticmethod
-    def forward(ctx, x, luts, plan, alpha, beta):
+    def forward(ctx, x, luts, plan, alpha, beta, beta_abs_max=None):
+        """alpha, beta: Python floats for the whole layer, or device tensors [N] with every node's own values
+        (then beta_abs_max = max |beta|, a host value)."""
         nat.require_device(x, luts)
         x, luts = _f32(x), _f32(luts)
         B, I = x.shape
@@ -141,8 +143,16 @@ class DWNLayerFunction(torch.autograd.Function):
         ws = _bytes(lib.dl_dwn_fwd_workspace_bytes(*dims), x.device)
         nat.check(lib.dl_dwn_layer_fwd(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(luts), nat.ptr(y), nat.ptr(saved),
                                        nat.ptr(ws), ws.numel(), *dims, nat.stream()))
+        if torch.is_tensor(alpha) or torch.is_tensor(beta):
+            alpha = torch.as_tensor(alpha, dtype=torch.float32, device=x.device).expand(N).contiguous()
+            beta = torch.as_tensor(beta, dtype=torch.float32, device=x.device).expand(N).contiguous()
+            if beta_abs_max is None:
+                beta_abs_max = float(beta.abs().max())
+            ctx.ab = (alpha, beta, float(beta_abs_max))
+        else:
+            ctx.ab = (float(alpha), float(beta))
         ctx.save_for_backward(luts, saved, x if k > FAST_K else None)
-        ctx.plan, ctx.ab, ctx.dims = plan, (float(alpha), float(beta)), dims
+        ctx.plan, ctx.dims = plan, dims
         return y
 
     @staticmethod
@@ -155,10 +165,16 @@ class DWNLayerFunction(torch.autograd.Function):
         gx = torch.empty((B, I), dtype=torch.float32, device=gy.device) if ctx.needs_input_grad[0] else None
         gl = torch.empty_like(luts)
         ws = _bytes(lib.dl_dwn_bwd_workspace_bytes(*ctx.dims), gy.device)
-        nat.check(lib.dl_dwn_layer_bwd(nat.ptr(x), nat.ptr(saved), nat.ptr(plan.idx32), nat.ptr(plan.inv_ptr),
-                                       nat.ptr(plan.inv_pos), nat.ptr(luts), nat.ptr(gy), ctx.ab[0], ctx.ab[1],
-                                       nat.ptr(gx), nat.ptr(gl), nat.ptr(ws), ws.numel(), *ctx.dims, nat.stream()))
-        return gx, gl, None, None, None
+        if len(ctx.ab) == 3:
+            nat.check(lib.dl_dwn_layer_bwd_nodes(nat.ptr(x), nat.ptr(saved), nat.ptr(plan.idx32), nat.ptr(plan.inv_ptr),
+                                                 nat.ptr(plan.inv_pos), nat.ptr(luts), nat.ptr(gy), nat.ptr(ctx.ab[0]),
+                                                 nat.ptr(ctx.ab[1]), ctx.ab[2], nat.ptr(gx), nat.ptr(gl), nat.ptr(ws),
+                                                 ws.numel(), *ctx.dims, nat.stream()))
+        else:
+            nat.check(lib.dl_dwn_layer_bwd(nat.ptr(x), nat.ptr(saved), nat.ptr(plan.idx32), nat.ptr(plan.inv_ptr),
+                                           nat.ptr(plan.inv_pos), nat.ptr(luts), nat.ptr(gy), ctx.ab[0], ctx.ab[1],
+                                           nat.ptr(gx), nat.ptr(gl), nat.ptr(ws), ws.numel(), *ctx.dims, nat.stream()))
+        return gx, gl, None, None, None, None
 
 
 class DWNStackFunction(torch.autograd.Function):

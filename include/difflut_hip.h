@@ -104,6 +104,14 @@ int dl_dwn_layer_bwd(const float *x, const void *saved, const int32_t *idx32,
                      const float *luts, const float *gy, float alpha, float beta,
                      float *gx, float *gluts, void *ws, size_t ws_bytes,
                      int B, int I, int N, int k, int O, void *stream);
+/* dl_dwn_layer_bwd with every node's own alpha and beta: the reference keeps them as per-node buffers and reads
+ * each node's pair in its forward (dwn_node.py:417-418, 450), so a state dict may carry different values per node.
+ * alpha_n, beta_n: device arrays [N]; beta_abs_max = max_n |beta_n[n]| (host value). */
+int dl_dwn_layer_bwd_nodes(const float *x, const void *saved, const int32_t *idx32,
+                           const int32_t *inv_ptr, const int32_t *inv_pos,
+                           const float *luts, const float *gy, const float *alpha_n, const float *beta_n,
+                           float beta_abs_max, float *gx, float *gluts, void *ws, size_t ws_bytes,
+                           int B, int I, int N, int k, int O, void *stream);
 /* Chained DWN layers.  No counterpart in the reference, which materialises the [B, N] fp32
  * activations between layers (random_layer.py:306-340 per layer): a following DWN layer only
  * thresholds them, so layer l can hand layer l+1 its output as bit-planes

@@ -267,3 +267,90 @@ def test_argument_checks_of_the_later_entry_points_need_no_gpu():
     dims = (4096, 16384, 8192, 6, 1)
     assert lib.dl_hybrid_bwd_workspace_bytes(*dims) < lib.dl_prob_bwd_workspace_bytes(*dims)
     assert lib.dl_hybrid_bwd_workspace_bytes(*dims) >= 4096 * (16384 + 8192 + 6 * 8192) * 4
+
+
+# ------------------------------------------------------------------------------ parameter and scalar banks
+def _small_dwn_layer(n=12, k=3, inputs=20):
+    from difflut_amd.layers import RandomLayer
+    from difflut_amd.nodes import DWNNode, NodeConfig
+    return RandomLayer(inputs, n, DWNNode, NodeConfig(input_dim=k, output_dim=1), seed=5)
+
+
+@pytest.mark.parametrize("how", ["deepcopy", "pickle"])
+def test_parameters_are_final_after_copy_so_an_optimizer_built_at_once_trains(how):
+    """copy.deepcopy / pickle hand back a layer whose per-node Parameters are already views of the bank: an optimizer
+    built before any forward holds the tensors the layer uses, and a step moves the bank."""
+    import copy
+    import pickle
+    layer = _small_dwn_layer()
+    twin = copy.deepcopy(layer) if how == "deepcopy" else pickle.loads(pickle.dumps(layer))
+    params = list(twin.parameters())
+    ids = [id(p) for p in params]
+    opt = torch.optim.SGD(params, lr=0.5)
+    bank = twin._banks["luts"]
+    flat = bank.tensor()                      # what the first forward asks for
+    assert [id(p) for p in twin.parameters()] == ids and bank.tensor() is flat
+    assert bank.nodes[3]._parameters["luts"].data_ptr() == flat[3].data_ptr()
+    before = flat.detach().clone()
+    flat.grad = torch.ones_like(flat)         # what a backward leaves
+    assert params[3].grad is not None and torch.equal(params[3].grad, torch.ones_like(params[3]))
+    opt.step()
+    assert torch.equal(flat.detach(), before - 0.5)
+    assert torch.equal(twin.nodes[3].luts.detach(), before[3] - 0.5)
+    # the original is untouched and still tied to its own bank
+    assert layer._banks["luts"].tied() and not torch.equal(layer._banks["luts"].flat.detach(), flat.detach())
+
+
+def test_bank_notices_nodes_taken_over_or_replaced():
+    """A bank whose nodes were re-tied by another bank (a sub-layer called on its own inside a convolutional level) or
+    whose parameter was reassigned is stale, whichever node it was - not only the first or the last."""
+    from difflut_amd.layers.base_layer import ParameterBank
+    layer = _small_dwn_layer()
+    bank = layer._banks["luts"]
+    assert bank.tied()
+    middle = ParameterBank(list(layer.nodes)[4:8], "luts")   # takes nodes 4..7 away
+    assert middle.tied() and not bank.tied()
+    flat = bank.tensor()                                      # re-ties all twelve
+    assert bank.tied() and not middle.tied()
+    assert layer.nodes[5].luts.data_ptr() == flat[5].data_ptr()
+    layer.nodes[6].luts = torch.nn.Parameter(torch.zeros(1, 8))
+    assert not bank.tied()
+    assert torch.equal(bank.tensor()[6], torch.zeros(1, 8))
+
+
+def test_scalar_buffers_are_banked_and_differences_are_seen():
+    layer = _small_dwn_layer()
+    alpha, beta = layer._scalars["alpha"], layer._scalars["beta"]
+    same, value, _ = alpha.summary()
+    assert same and value == pytest.approx(0.5 * 0.75 ** 2)
+    assert layer.efd_scalars() == (pytest.approx(0.5 * 0.75 ** 2), pytest.approx(1 / 3))
+    assert set(layer.state_dict()) >= {"nodes.0.alpha", "nodes.11.beta"} and layer.state_dict()["nodes.0.alpha"].shape == ()
+    # a state dict with another value for one node in the middle lands in the bank
+    state = layer.state_dict()
+    state["nodes.7.alpha"] = torch.tensor(0.25)
+    layer.load_state_dict(state)
+    assert alpha.tied() and float(alpha.flat[7]) == 0.25
+    assert alpha.summary()[0] is False
+    with pytest.raises(RuntimeError, match="different alpha"):
+        layer.efd_scalars()
+    # in-place edits too; making all equal again is seen as well
+    with torch.no_grad():
+        for node in layer.nodes:
+            node.alpha.fill_(0.25)
+    assert alpha.summary()[:2] == (True, 0.25)
+    # replacing a node's buffer object re-ties on the next use
+    layer.nodes[2].beta = torch.tensor(0.9)
+    assert not beta.tied()
+    assert beta.summary() == (False, pytest.approx(1 / 3), pytest.approx(0.9))
+    assert layer.nodes[2].beta.data_ptr() == beta.flat[2].data_ptr()
+
+
+def test_probabilistic_layer_refuses_per_node_temperatures():
+    from difflut_amd.layers import RandomLayer
+    from difflut_amd.nodes import NodeConfig, ProbabilisticNode
+    layer = RandomLayer(16, 8, ProbabilisticNode, NodeConfig(input_dim=2, output_dim=1), seed=1)
+    assert layer.temperature_value() == 1.0
+    with torch.no_grad():
+        layer.nodes[5].temperature.fill_(2.0)
+    with pytest.raises(RuntimeError, match="different temperatures"):
+        layer.temperature_value()
