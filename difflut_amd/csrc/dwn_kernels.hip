@@ -16,7 +16,8 @@
 //                           beta^popc((a^kappa)&~(1<<j)), a' = address with bit j squeezed out;
 //                           also clears the table-gradient output
 //             transpose_hist : gy [B,N*O] -> gyT [B/64][N*O][64]; per-node 2^k-bin histogram of gy
-//                           in LDS, one float atomic per bin per block into gluts
+//                           in LDS; blocks of one column tile leave partials that the last of them adds in a
+//                           fixed order (no floating-point atomics)
 //             bwd_gx      : for every input i the (node,slot) pairs that read it (CSR):
 //                           gx[b,i] = sum gyT[c][b] * D[c][j][a'(b)]  - a gather in fixed order
 // k > 6 goes to the one-thread-per-element kernels of dwn_generic.hip.
@@ -33,15 +34,6 @@ __device__ __forceinline__ unsigned dwn_shift_in(unsigned addr, u64 mask) {
     u64 carry_out;
     asm("v_addc_co_u32_e64 %0, %1, %2, %2, %3" : "=v"(out), "=s"(carry_out) : "v"(addr), "s"(mask));
     return out;
-}
-
-// ---------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void dl_fill_zero_kernel(float *p, long long n) {
-    long long i = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) p[i] = 0.0f;
-}
-static void dl_fill_zero(float *p, long long n, hipStream_t s) {
-    if (n > 0) DL_TIMED("dl_fill_zero", s, (dl_fill_zero_kernel<<<dl_ceil_div(n, 256), 256, 0, s>>>(p, n)));
 }
 
 // ---------------------------------------------------------------------------------
@@ -249,9 +241,44 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
     }
 }
 
+// gluts[e] = scale * (partial[0][e] + partial[1][e] + ...), four entries per thread, the chunks' loads in flight together.
+// `block` = index among the blocks that reduce (the table kernels below append these blocks to their own grid, so that
+// the backward needs one launch for both).
+struct DwnReduce {
+    const float *partial;  // null: nothing to reduce
+    float *gluts;
+    long long NOL;
+    int chunks;
+    const float *scale;
+    int L, O;
+};
+__device__ __forceinline__ void dwn_reduce_block(const DwnReduce &r, int block) {
+    const long long e4 = ((long long)block * 256 + threadIdx.x) * 4;
+    if (e4 >= r.NOL) return;
+    float sum[4] = {0.f, 0.f, 0.f, 0.f};
+    if (r.NOL % 4 == 0) {
+        for (int ch0 = 0; ch0 < r.chunks; ch0 += 8) {
+            float4 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                v[u] = ch0 + u < r.chunks ? *reinterpret_cast<const float4 *>(r.partial + (size_t)(ch0 + u) * r.NOL + e4)
+                                          : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) { sum[0] += v[u].x; sum[1] += v[u].y; sum[2] += v[u].z; sum[3] += v[u].w; }
+        }
+    } else {
+        for (int ch = 0; ch < r.chunks; ++ch)
+            for (int q = 0; q < 4; ++q)
+                if (e4 + q < r.NOL) sum[q] += r.partial[(size_t)ch * r.NOL + e4 + q];
+    }
+    for (int q = 0; q < 4; ++q)
+        if (e4 + q < r.NOL) r.gluts[e4 + q] = sum[q] * (r.scale ? r.scale[((e4 + q) / r.L) / r.O] : 1.0f);
+}
+static inline int dwn_reduce_blocks(const DwnReduce &r) { return r.partial ? dl_ceil_div(r.NOL, 1024) : 0; }
+__global__ __launch_bounds__(256) void dwn_reduce_partials(DwnReduce r) { dwn_reduce_block(r, blockIdx.x); }
+
 // ---------------------------------------------------------------------------------
-// efd_table: one wavefront per table (column), lane = table entry; also clears the table's
-// gradient row.  Two forms of the EFD coefficients, both in double with one rounding to float:
+// efd_table: one wavefront per table (column), lane = table entry.  Two forms of the EFD coefficients, both in double with one rounding to float:
 //   D form: for every input j the table is smoothed along all OTHER inputs
 //           (v <- v + beta * v[entry ^ bit]) and differenced along j; lanes whose bit j is clear
 //           hold D[c][j][a'] = alpha * (v[a | bit j] - v[a & ~bit j]).          192 floats/table
@@ -264,8 +291,10 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
 // alpha_n / beta_n (nullable): the nodes' own alpha and beta [N] instead of one value for the layer.
 __global__ __launch_bounds__(256) void dwn_efd_table(const float *__restrict__ luts, float *__restrict__ D,
                                                       float *__restrict__ gluts, int NO, int K, float alpha, float beta,
-                                                      int sform, const float *__restrict__ alpha_n = nullptr,
+                                                      int sform, DwnReduce red, int table_blocks,
+                                                      const float *__restrict__ alpha_n = nullptr,
                                                       const float *__restrict__ beta_n = nullptr, int O = 1) {
+    if ((int)blockIdx.x >= table_blocks) return dwn_reduce_block(red, blockIdx.x - table_blocks);
     const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int a = threadIdx.x & 63;
     if (c >= NO) return;
@@ -274,7 +303,6 @@ __global__ __launch_bounds__(256) void dwn_efd_table(const float *__restrict__ l
     const int L = 1 << K, Lh = L >> 1;
     const bool live = a < L;
     const double v0 = live ? (double)luts[(size_t)c * L + a] : 0.0;
-    if (live) gluts[(size_t)c * L + a] = 0.0f;
     if (sform) {
         double v = v0;
         for (int m = 0; m < K; ++m) v += (double)beta * __shfl_xor(v, 1 << m);
@@ -300,10 +328,11 @@ __global__ __launch_bounds__(256) void dwn_efd_table(const float *__restrict__ l
 // That weight is not a product over inputs, so the sums are taken directly, in double: one wavefront
 // per table keeps it in LDS and shares out the k * 2^(k-1) outputs (j, a'), one 2^(k-1)-term sum
 //   D[c][j][a'] = scale * sum_kappa' (lut[kappa' with bit j set] - lut[kappa' with bit j clear]) / (popc(a' ^ kappa') + 1)
-// each.  Also clears the table's gradient row.
+// each.
 __global__ __launch_bounds__(256) void dwn_stable_table(const float *__restrict__ luts, const float *__restrict__ scale,
                                                          float *__restrict__ D, float *__restrict__ gluts, int NO, int K,
-                                                         int O) {
+                                                         int O, DwnReduce red, int table_blocks) {
+    if ((int)blockIdx.x >= table_blocks) return dwn_reduce_block(red, blockIdx.x - table_blocks);
     __shared__ double rec[8];
     __shared__ float tab[4][64];
     if (threadIdx.x < 8) rec[threadIdx.x] = 1.0 / (double)(threadIdx.x + 1);
@@ -312,7 +341,6 @@ __global__ __launch_bounds__(256) void dwn_stable_table(const float *__restrict_
     const int L = 1 << K, Lh = L >> 1;
     if (c < NO && lane < L) {
         tab[w][lane] = luts[(size_t)c * L + lane];
-        gluts[(size_t)c * L + lane] = 0.0f;
     }
     __syncthreads();
     if (c >= NO) return;
@@ -367,11 +395,28 @@ __device__ __forceinline__ int dwn_quad_xor(int v) {
     constexpr int ctrl = X == 1 ? 0xB1 : (X == 2 ? 0x4E : 0x1B);  // quad_perm [1,0,3,2] / [2,3,0,1] / [3,2,1,0]
     return __builtin_amdgcn_update_dpp(0, v, ctrl, 0xf, 0xf, true);
 }
+// End of a histogram block: the table gradient in a fixed order of additions.  With one chunk of batch tiles per
+// column tile the block's bins are the result.  With several, every block stores its bins as a partial
+// ([chunk][column][bin]) and dwn_reduce_partials adds them in chunk order afterwards, so the sums do not depend on the
+// order the blocks ran in (no floating-point atomics).  scale (nullable): the stabilised node's per-node factor.
+__device__ __forceinline__ void dwn_hist_flush(const float (*hist)[65], int c0, int cend, int L, long long NOL, int chunks,
+                                               float *__restrict__ partial, float *__restrict__ gluts,
+                                               const float *__restrict__ scale, int O) {
+    if (chunks == 1) {
+        for (int e = threadIdx.x; e < cend * L; e += 256)
+            gluts[(size_t)c0 * L + e] = hist[e / L][e % L] * (scale ? scale[(c0 + e / L) / O] : 1.0f);
+        return;
+    }
+    float *mine = partial + (size_t)blockIdx.y * NOL + (size_t)c0 * L;
+    for (int e = threadIdx.x; e < cend * L; e += 256) mine[e] = hist[e / L][e % L];
+}
+
 template <bool WRITE_T>
 __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__restrict__ gy, const uint8_t *__restrict__ addrT,
                                                                float *__restrict__ gyT, float *__restrict__ gluts,
                                                                int B, int NO, int O, int L, int BP, int BT,
-                                                               int tiles_per_chunk, const float *__restrict__ scale = nullptr) {
+                                                               int tiles_per_chunk, float *__restrict__ partial,
+                                                               const float *__restrict__ scale = nullptr) {
     __shared__ float tile[64][DWN_HC + 1];       // [row][column]
     __shared__ float hist[DWN_HC][65];           // [column][bin]
     __shared__ uint8_t atile[DWN_HC][64 + 4];    // [column][row] addresses
@@ -453,8 +498,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
     }
     __syncthreads();
     // scale (nullable): the stabilised node multiplies a node's table gradient by its gradient_scale
-    for (int e = threadIdx.x; e < cend * L; e += 256)
-        atomicAdd(&gluts[(size_t)c0 * L + e], hist[e / L][e % L] * (scale ? scale[(c0 + e / L) / O] : 1.0f));
+    dwn_hist_flush(hist, c0, cend, L, (long long)NO * L, (int)gridDim.y, partial, gluts, scale, O);
 }
 
 // hist_tiled: the histogram alone, for gy that arrives tile-major ([B/64][N*O][64]).  Nothing has to be
@@ -467,8 +511,8 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
 template <bool GROUPS = false>
 __global__ __launch_bounds__(256) void dwn_bwd_hist_tiled(const float *__restrict__ gy, const uint8_t *__restrict__ addrT,
                                                            float *__restrict__ gluts, int NO, int O, int L, int BT,
-                                                           int tiles_per_chunk, float *__restrict__ gyT = nullptr, int B = 0,
-                                                           int groups = 0, int gsize = 1, float inv_tau = 1.0f) {
+                                                           int tiles_per_chunk, float *__restrict__ partial, float *__restrict__ gyT = nullptr,
+                                                           int B = 0, int groups = 0, int gsize = 1, float inv_tau = 1.0f) {
     __shared__ float hist[DWN_HC][65];  // [column][bin]
     const int c0 = blockIdx.x * DWN_HC;
     const int lane = threadIdx.x & 63;
@@ -532,7 +576,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_hist_tiled(const float *__restric
         }
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < cend * L; e += 256) atomicAdd(&gluts[(size_t)c0 * L + e], hist[e / L][e % L]);
+    dwn_hist_flush(hist, c0, cend, L, (long long)NO * L, (int)gridDim.y, partial, gluts, nullptr, O);
 }
 
 // ---------------------------------------------------------------------------------
@@ -724,6 +768,21 @@ static inline size_t dwn_table_bytes(int N, int k, int O) {
 static inline size_t dwn_gyT_bytes(int B, int N, int O) {
     return dl_align256((size_t)N * O * dwn_bt(B) * 64 * sizeof(float));
 }
+// grid of the histogram kernels: column tiles x chunks of batch tiles.  Enough blocks to fill 256 CUs several times
+// over; four blocks fit a CU (LDS), so at most about 1024 of them - all resident at once, no second, mostly empty round.
+static inline void dwn_hist_grid(long long NO, int BT, int &col_tiles, int &chunks, int &tpc) {
+    col_tiles = dl_ceil_div(NO, DWN_HC);
+    chunks = col_tiles >= 1024 ? 1 : 1024 / col_tiles;
+    if (chunks > BT) chunks = BT;
+    tpc = dl_ceil_div(BT, chunks);
+    chunks = dl_ceil_div(BT, tpc);
+}
+// chunk partials of the table gradient (none when one chunk covers the batch)
+static inline size_t dwn_partial_bytes(int B, int N, int k, int O) {
+    int col_tiles, chunks, tpc;
+    dwn_hist_grid((long long)N * O, dwn_bt(B), col_tiles, chunks, tpc);
+    return chunks > 1 ? dl_align256((size_t)chunks * N * O * sizeof(float) << k) : 0;
+}
 
 static int dwn_check(int B, int I, int N, int k, int O) {
     if (B <= 0 || I <= 0 || N <= 0 || k <= 0 || O <= 0) return DL_ERR_SHAPE;
@@ -748,7 +807,8 @@ extern "C" size_t dl_dwn_fwd_workspace_bytes(int B, int I, int N, int k, int O) 
 }
 extern "C" size_t dl_dwn_bwd_workspace_bytes(int B, int I, int N, int k, int O) {
     (void)I;
-    return dwn_fast(N, k, O) ? dwn_table_bytes(N, k, O) + dwn_gyT_bytes(B, N, O) : 256;
+    return dwn_fast(N, k, O) ? dwn_table_bytes(N, k, O) + dwn_gyT_bytes(B, N, O) + dwn_partial_bytes(B, N, k, O)
+                             : 256;
 }
 
 template <int K>
@@ -913,39 +973,36 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
     float *D = (float *)ws;
     float *gyT = (float *)((char *)ws + dwn_table_bytes(N, k, O));
     const int BT = dwn_bt(B), BP = BT * 64;
-    // enough blocks to fill 256 CUs several times over, few enough that the per-block
-    // histogram flush (one atomic per bin) stays small next to the streaming work
-    const int col_tiles = dl_ceil_div(NO, DWN_HC);
-    // four blocks fit a CU (LDS): at most 1024 blocks, so that all of them are resident at once and
-    // no second, mostly empty round of blocks follows
-    int chunks = col_tiles >= 1024 ? 1 : 1024 / col_tiles;
-    if (chunks > BT) chunks = BT;
-    const int tpc = dl_ceil_div(BT, chunks);
-    chunks = dl_ceil_div(BT, tpc);
+    float *partial = (float *)((char *)ws + dwn_table_bytes(N, k, O) + dwn_gyT_bytes(B, N, O));
+    int col_tiles, chunks, tpc;
+    dwn_hist_grid(NO, BT, col_tiles, chunks, tpc);
     const dim3 hgrid(col_tiles, chunks);
     const bool sform = !scale && beta >= -0.5f && beta <= 0.5f;
-    if (gx && scale)
-        DL_TIMED("dwn_stable_table", s,
-                 (dwn_stable_table<<<dl_ceil_div(NO, 4), 256, 0, s>>>(luts, scale, D, gluts, (int)NO, k, O)));
-    else if (gx)
-        DL_TIMED("dwn_efd_table", s,
-                 (dwn_efd_table<<<dl_ceil_div(NO, 4), 256, 0, s>>>(luts, D, gluts, (int)NO, k, alpha, beta, sform ? 1 : 0,
-                                                                  alpha_n, beta_n, O)));
-    else
-        dl_fill_zero(gluts, NO * L, s);
     if (head)
         DL_TIMED("dwn_bwd_hist_groups", s, (dwn_bwd_hist_tiled<true><<<hgrid, 256, 0, s>>>(
-                                               gy, addrT, gluts, (int)NO, O, L, BT, tpc, gx ? gyT : nullptr, B, head->groups,
+                                               gy, addrT, gluts, (int)NO, O, L, BT, tpc, partial, gx ? gyT : nullptr, B, head->groups,
                                                head->gsize, head->inv_tau)));
     else if (gy_tiled)
         DL_TIMED("dwn_bwd_hist_tiled", s,
-                 (dwn_bwd_hist_tiled<false><<<hgrid, 256, 0, s>>>(gy, addrT, gluts, (int)NO, O, L, BT, tpc)));
+                 (dwn_bwd_hist_tiled<false><<<hgrid, 256, 0, s>>>(gy, addrT, gluts, (int)NO, O, L, BT, tpc, partial)));
     else if (gx)
         DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<true><<<hgrid, 256, 0, s>>>(
-                                                  gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc, scale)));
+                                                  gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc, partial, scale)));
     else
         DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<false><<<hgrid, 256, 0, s>>>(
-                                                  gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc, scale)));
+                                                  gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc, partial, scale)));
+    // the coefficient tables of the gather and the fixed-order sum of the histogram partials share one launch
+    // (the row-major histogram's scale is applied in the sum; the tile-major ones scale afterwards)
+    DwnReduce red = {chunks > 1 ? partial : nullptr, gluts, NO * L, chunks, (head || gy_tiled) ? nullptr : scale, L, O};
+    const int table_blocks = dl_ceil_div(NO, 4), red_blocks = dwn_reduce_blocks(red);
+    if (gx && scale)
+        DL_TIMED("dwn_stable_table", s, (dwn_stable_table<<<table_blocks + red_blocks, 256, 0, s>>>(luts, scale, D, gluts, (int)NO, k,
+                                                                                                  O, red, table_blocks)));
+    else if (gx)
+        DL_TIMED("dwn_efd_table", s, (dwn_efd_table<<<table_blocks + red_blocks, 256, 0, s>>>(
+                                         luts, D, gluts, (int)NO, k, alpha, beta, sform ? 1 : 0, red, table_blocks, alpha_n, beta_n, O)));
+    else if (red_blocks)
+        DL_TIMED("dwn_reduce_partials", s, (dwn_reduce_partials<<<red_blocks, 256, 0, s>>>(red)));
     if (gx) {
         const float *src = gy_tiled ? gy : gyT;
         switch (k) {
