@@ -27,12 +27,31 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
-# HBM bytes per launch of a workload's dominant kernel, from rocprofv3 counter runs of this file
-# (FETCH_SIZE scaled by 2.0 after calibration against a plain copy, plus WRITE_SIZE; the runs and
-# the calibration are written up under profiles/).  Measured, not computed: None where no run exists.
-MEASURED_TRAFFIC = {
-    ("dwn_k6_b4096_i16384_n8192", "dwn_bwd_gx"): 901565644,  # (301.9 * 2 + 256.0) MiB
-}
+PROFILE_DIR = os.path.join(ROOT, "profiles")
+KERNEL_SOURCE = os.path.join(ROOT, "difflut_amd", "csrc", "dwn_kernels.hip")
+
+
+def source_hash(path=KERNEL_SOURCE):
+    import hashlib
+    with open(path, "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()[:16]
+
+
+def measured_traffic(workload, kernel):
+    """HBM bytes per launch of `kernel` from the rocprofv3 counter summary committed under profiles/ (FETCH_SIZE scaled
+    by the copy calibration written there, plus WRITE_SIZE).  The summary names the hash of the kernel source it was
+    measured on; when the source has changed since, the figure is stale and None is reported instead."""
+    import re
+    path = os.path.join(PROFILE_DIR, f"{workload}_kernels.md")
+    if not os.path.exists(path):
+        return None
+    text = open(path).read()
+    m = re.search(r"kernel_source_sha256_16:\s*([0-9a-f]{16})", text)
+    t = re.search(rf"traffic_bytes_per_launch:\s*{re.escape(kernel)}\s+(\d+)", text)
+    if not m or not t or m.group(1) != source_hash():
+        return None
+    return int(t.group(1))
+
 
 WORKLOADS = {
     # name: (B, I, N, k, O)
@@ -72,6 +91,24 @@ def algorithmic_bytes(B, I, N, k, O):
         "dl_fill_zero": tables,
     }
     return fwd, bwd, per_kernel
+
+
+def stack_bytes(B, F, nbits, widths, k, train):
+    """HBM bytes the chained bit-plane formulation has to move for one batch (a lower bound for THESE kernels, so the
+    fraction of the roofline cannot exceed 1): raw features in; every layer's input once written and once read as
+    bit-planes (1 bit per value); tables read; logits.  Training adds: the saved address of every (node, row), one
+    byte, written forward and read by the histogram and by the gather; the fp32 gradient with respect to every hidden
+    activation, written once and read twice (histogram, gather) in tile-major form; the gradient of the logits; and
+    nine passes over the tables in all (forward, backward, gradient, Adam read p/g/m/v, write p/m/v)."""
+    ins = [F * nbits] + widths[:-1]
+    tables = sum(widths) * (1 << k) * 4
+    planes = sum(ins) * B // 8
+    nbytes = B * F * 4 + 2 * planes + tables + B * 10 * 4
+    if train:
+        nbytes += 3 * B * sum(widths)                   # saved addresses: written, read twice
+        nbytes += 3 * 4 * B * sum(widths[:-1])          # hidden-activation gradients: written, read twice
+        nbytes += 2 * B * 10 * 4 + 8 * tables
+    return nbytes
 
 
 def time_steps(step, steps, warmup):
@@ -140,8 +177,7 @@ def run_stack(args):
 
         ms = time_steps(infer, args.steps, args.warmup)
         evals = B * sum(widths)
-        ins = [F * 4] + widths[:-1]
-        nbytes = sum(4 * B * (i + n) for i, n in zip(ins, widths)) + sum(widths) * (1 << k) * 4
+        nbytes = stack_bytes(B, F, 4, widths, k, train=False)
         out = {"metric": "LUT-node evals/sec, inference (thermometer -> 4 DWN k=6 layers -> GroupSum)",
                "value": evals / (ms * 1e-3), "unit": "node-evals/s", "ms_per_step": ms, "dtype": "f32 tables, 1-bit activations",
                "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
@@ -151,10 +187,10 @@ def run_stack(args):
                "roofline_step": {"bound": "hbm", "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                  "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                                  "algorithmic_bytes_per_step": nbytes,
-                                 "note": "bytes of the layer-by-layer fp32 formulation (x and y per layer, tables once)"},
+                                 "note": "bytes of the bit-plane formulation (features, 1-bit activations written and read, "
+                                         "tables, logits); the kernels are bound by L2 gather latency, not by HBM"},
                "kernel_ms": kernel_times(infer, min(args.steps, 5))}
-        print(json.dumps(out))
-        return
+        return out
 
     def step():
         opt.zero_grad(set_to_none=True)
@@ -171,11 +207,14 @@ def run_stack(args):
 
     ms = time_steps(step, args.steps, args.warmup)
     evals = B * sum(widths)
-    # compulsory fp32 traffic of the layer-by-layer formulation: per layer x and y forward, gy, x and gx
-    # backward (no gx for the first layer), plus nine passes over the tables (forward, backward, gradient, Adam)
-    ins = [F * 4] + widths[:-1]
-    nbytes = sum(4 * B * (2 * i + 2 * n + (i if li else 0)) for li, (i, n) in enumerate(zip(ins, widths)))
-    nbytes += 9 * sum(widths) * (1 << k) * 4
+    if args.layer_by_layer:
+        # fp32 traffic of the layer-by-layer formulation: per layer x and y forward, gy, x and gx backward (no gx for
+        # the first layer), plus nine passes over the tables (forward, backward, gradient, Adam)
+        ins = [F * 4] + widths[:-1]
+        nbytes = sum(4 * B * (2 * i + 2 * n + (i if li else 0)) for li, (i, n) in enumerate(zip(ins, widths)))
+        nbytes += 9 * sum(widths) * (1 << k) * 4
+    else:
+        nbytes = stack_bytes(B, F, 4, widths, k, train=True)
     out = {"metric": "LUT-node evals/sec, training step (thermometer -> 4 DWN k=6 layers -> GroupSum -> CE, Adam)",
            "value": evals / (ms * 1e-3), "unit": "node-evals/s", "ms_per_step": ms, "dtype": "f32",
            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
@@ -185,7 +224,7 @@ def run_stack(args):
            "roofline_step": {"bound": "hbm", "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                              "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes_per_step": nbytes},
            "kernel_ms": kernel_times(step, min(args.steps, 5))}
-    print(json.dumps(out))
+    return out
 
 
 def run_conv(args):
@@ -219,18 +258,16 @@ def run_conv(args):
     ms = time_steps(step, args.steps, args.warmup)
     rows = B * out * out
     nodes = sum(layer.hidden_layers) * T
-    # compulsory traffic of the convolution as a whole: the image in, its gradient out, the output and its gradient
-    nbytes = 2 * x.numel() * 4 + 2 * gy.numel() * 4 + 4 * nodes * (1 << k) * 4
     out_d = {"metric": "LUT-node evals/sec fwd+bwd (ConvolutionalLayer, DWN k=6 trees of depth 2, 32 channels, 5x5x4 patches)",
              "value": rows * nodes / (ms * 1e-3), "unit": "node-evals/s", "ms_per_step": ms, "dtype": "f32",
              "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
              "vs_baseline": None, "data": "synthetic",
              "config": {"workload": args.workload, "images": B, "in_channels": C, "out_channels": T, "image": [H, W],
                         "receptive_field": rf, "tree_depth": depth, "patch_rows": rows, "nodes": nodes},
-             "roofline_step": {"bound": "hbm", "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                               "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes_per_step": nbytes},
+             # no roofline fraction: image and output are a few MB, the step is bound by the first level's input
+             # gradient (6912 connections onto 100 inputs: lane reads and L2 gathers), see profiles/
              "kernel_ms": kernel_times(step, min(args.steps, 5))}
-    print(json.dumps(out_d))
+    return out_d
 
 
 def run_learnable(args):
@@ -274,7 +311,7 @@ def run_learnable(args):
            "roofline_step": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
                              "frac": flops / (ms * 1e-3) / 1e12 / peak, "algorithmic_flops_per_step": flops},
            "kernel_ms": kernel_times(step, min(args.steps, 5))}
-    print(json.dumps(out))
+    return out
 
 
 def maybe_graph(step, args):
@@ -299,7 +336,7 @@ def run_secondary(args):
     soft connectivity (512 x 3136 -> 48000 rows), all through the C ABI."""
     from difflut_amd import _native as nat
     from difflut_amd import ops
-    from oracle import difflut_oracle as orc
+    from difflut_amd.layers.random_layer import draw_mapping
 
     lib = nat.lib()
     dev = torch.device("cuda:0")
@@ -308,7 +345,7 @@ def run_secondary(args):
     if args.workload.startswith("prob"):
         dims = (B, I, N, k, O)
         x = torch.sigmoid(torch.randn(B, I, device=dev))
-        plan = ops.MappingPlan(orc.random_mapping(I, N, k, seed=42).to(dev), I)
+        plan = ops.MappingPlan(draw_mapping(I, N, k, seed=42).to(dev), I)
         raw = torch.rand(N, 1 << k, O, device=dev)
         gy = torch.randn(B, N * O, device=dev)
         y = torch.empty(B, N * O, device=dev); gx = torch.empty(B, I, device=dev); graw = torch.empty_like(raw)
@@ -336,7 +373,7 @@ def run_secondary(args):
         dims = (B, I, N, k, O)
         count = N * O * (1 << k)
         x = torch.rand(B, I, device=dev)  # real-valued: the hybrid backward differentiates at x itself
-        plan = ops.MappingPlan(orc.random_mapping(I, N, k, seed=42).to(dev), I)
+        plan = ops.MappingPlan(draw_mapping(I, N, k, seed=42).to(dev), I)
         raw = torch.randn(N, O, 1 << k, device=dev)
         scale = torch.full((N,), 1.25, device=dev)
         gy = torch.randn(B, N * O, device=dev)
@@ -399,7 +436,68 @@ def run_secondary(args):
                 "vs_baseline": None, "data": "synthetic",
                 "config": {"workload": args.workload, "launch": "hip graph replay" if args.graph else "direct"},
                 "kernel_ms": kernel_times(step, min(args.steps, 10))})
-    print(json.dumps(out))
+    return out
+
+
+def layer_api_step(args, x, gy, idx, luts):
+    """forward + backward of the headline layer through RandomLayer / DWNNode modules and autograd."""
+    from difflut_amd import REGISTRY
+    from difflut_amd.nodes.node_config import NodeConfig
+    B, I, N, k, O = WORKLOADS[args.workload]
+    layer = REGISTRY.get_layer("random")(I, N, REGISTRY.get_node("dwn"), NodeConfig(input_dim=k, output_dim=O), seed=42,
+                                         mapping_indices=idx).to(x.device).train()
+    bank = layer.bank_parameters()[0]
+    with torch.no_grad():
+        bank.copy_(luts)
+    xg = x.clone().requires_grad_()
+
+    def step():
+        xg.grad = None
+        bank.grad = None
+        layer(xg).backward(gy)
+
+    ms = time_steps(step, args.steps, args.warmup)
+    fwd_b, bwd_b, _ = algorithmic_bytes(B, I, N, k, O)
+    gbs = (fwd_b + bwd_b) / (ms * 1e-3) / 1e9
+    return {"ms_per_step": ms, "value": B * N / (ms * 1e-3), "unit": "node-evals/s",
+            "call": "RandomLayer(...).forward(x).backward(gy), tensors allocated per call by torch's caching allocator",
+            "roofline_step": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                              "algorithmic_bytes_per_step": fwd_b + bwd_b}}
+
+
+def secondary_configs(args):
+    """The other benchmark configurations, a few steps each, after the headline's timed region: the probabilistic layer,
+    the LearnableLayer with fp32 and with bf16 soft connectivity, and the deep-stack training step.  Each entry carries
+    its own metric, time per step and a roofline fraction against the bytes or flops its formulation has to move."""
+    import copy
+    import gc
+    res = {}
+    plan = [("prob_k4_b1024_i4096_n4096", {}), ("learnable_layer_b512_i3136_n8000", {"precision": 0}),
+            ("learnable_layer_b512_i3136_n8000", {"precision": 1}), ("dwn_stack_b8192_train_step", {})]
+    for workload, extra in plan:
+        sub = copy.copy(args)
+        sub.workload, sub.steps, sub.warmup, sub.graph, sub.layer_by_layer = workload, min(args.steps, 10), 3, False, False
+        for key, value in extra.items():
+            setattr(sub, key, value)
+        gc.collect()
+        torch.cuda.empty_cache()
+        r = dispatch_other(sub)
+        name = workload + ("_bf16" if extra.get("precision") == 1 else "")
+        res[name] = {key: r[key] for key in ("metric", "value", "unit", "ms_per_step", "dtype", "roofline_step") if key in r}
+    return res
+
+
+def dispatch_other(args):
+    """Every workload but the headline one: its result line as a dict (None for the headline)."""
+    if args.workload.startswith("dwn_stack"):
+        return run_stack(args)
+    if args.workload.startswith("conv"):
+        return run_conv(args)
+    if args.workload.startswith("learnable"):
+        return run_learnable(args)
+    if not args.workload.startswith("dwn"):
+        return run_secondary(args)
+    return None
 
 
 def main():
@@ -412,6 +510,8 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=4096, help="batch rows of the workload the CPU baseline runs")
     ap.add_argument("--precision", type=int, default=0, help="soft-connectivity workload: 0 fp32, 1 bf16 operands")
     ap.add_argument("--layer-by-layer", action="store_true", help="stack workload: call the layers one by one")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="default workload: skip the other benchmark configurations reported under 'secondary'")
     ap.add_argument("--graph", action="store_true",
                     help="C-ABI workloads other than the default: replay the step from a captured HIP graph")
     args = ap.parse_args()
@@ -422,25 +522,21 @@ def main():
 
     from difflut_amd import _native as nat
     from difflut_amd import ops
-    from oracle import difflut_oracle as orc
+    from difflut_amd.layers.random_layer import draw_mapping
 
     lib = nat.lib()  # raises if the HIP library has not been built
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a ROCm device")
-    if args.workload.startswith("dwn_stack"):
-        return run_stack(args)
-    if args.workload.startswith("conv"):
-        return run_conv(args)
-    if args.workload.startswith("learnable"):
-        return run_learnable(args)
-    if not args.workload.startswith("dwn"):
-        return run_secondary(args)
+    other = dispatch_other(args)
+    if other is not None:
+        print(json.dumps(other))
+        return
     dev = torch.device("cuda:0")
     B, I, N, k, O = WORKLOADS[args.workload]
     dims = (B, I, N, k, O)
     torch.manual_seed(0)
     x = torch.bernoulli(torch.full((B, I), 0.5, device=dev))
-    idx = orc.random_mapping(I, N, k, seed=42)  # same draw as RandomLayer(seed=42)
+    idx = draw_mapping(I, N, k, seed=42)  # the table RandomLayer(seed=42) registers
     plan = ops.MappingPlan(idx.to(dev), I)
     luts = torch.rand(N, O, 1 << k, device=dev) * 2 - 1
     gy = torch.randn(B, N * O, device=dev)
@@ -503,13 +599,21 @@ def main():
         "config": {"workload": args.workload, "batch": B, "inputs": I, "nodes": N, "k": k, "output_dim": O,
                    "pass": "forward + EFD backward (input and table gradients)", "seed": 0, "mapping_seed": 42},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": dom_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": dom_gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get((args.workload, dominant)),
+                     "frac": dom_gbs / HBM_PEAK_GBS, "traffic": measured_traffic(args.workload, dominant),
                      "algorithmic_bytes_per_launch": split[dominant],
                      "avg_launch_ms": avg[dominant]},
         "roofline_step": {"bound": "hbm", "achieved": step_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                           "frac": step_gbs / HBM_PEAK_GBS, "algorithmic_bytes_per_step": fwd_b + bwd_b},
         "kernel_ms": avg,
     }
+
+    # the same step through the layer API (what a user of the reference calls): RandomLayer.forward allocates its
+    # output, saved addresses and workspaces per call and goes through autograd
+    out["layer_api"] = layer_api_step(args, x, gy, idx, luts)
+    y_host = y[:min(B, args.cpu_rows)].cpu().numpy()  # for the check of the CPU baseline's output below
+    del y, gx, gl, saved, ws_f, ws_b
+    if not args.no_secondary and args.workload == "dwn_k6_b4096_i16384_n8192":
+        out["secondary"] = secondary_configs(args)
 
     if not args.no_cpu_baseline:
         from oracle import c_oracle
@@ -524,7 +628,7 @@ def main():
         yc = c_oracle.dwn_layer_forward(xs, idn, ls)
         c_oracle.dwn_layer_backward(xs, idn, ls, gs, alpha, beta)
         cpu_s = time.perf_counter() - t0
-        assert np.array_equal(yc.reshape(rows, -1), y[:rows].cpu().numpy())  # the checker, not the measured thing
+        assert np.array_equal(yc.reshape(rows, -1), y_host)  # the checker, not the measured thing
         out["cpu_baseline"] = {"value": rows * N / cpu_s, "unit": "node-evals/s", "cores": cores, "kind": "port",
                                "sample": f"first {rows} of {B} batch rows, all {N} nodes, forward+backward, "
                                          f"{cpu_s:.2f} s wall"}
