@@ -65,6 +65,7 @@ SIGNATURES = {
     "dl_thermometer_planes": (_I, [_P, _P, _P, _I, _I, _I, _P]),
     "dl_unfold_rows": (ctypes.c_longlong, [_I] * 9),
     "dl_unfold": (_I, [_P, _P, _P] + [_I] * 10 + [_P]),
+    "dl_unfold_flip": (_I, [_P, _P, _P, _P] + [_I] * 10 + [_P]),
     "dl_fold": (_I, [_P, _I, _P] + [_I] * 10 + [_P]),
     "dl_group_sum_fwd": (_I, [_P, _P, _I, _I, _I, _F, _P]),
     "dl_cross_entropy_workspace_bytes": (_Z, [_I]),

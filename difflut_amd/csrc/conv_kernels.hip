@@ -22,8 +22,10 @@ __device__ __forceinline__ void conv_fill_columns(const ConvGeom &g, int cols, i
 }
 
 // grid = ceil(rows / 64) blocks of 256 threads; block t writes rows 64 t .. 64 t + 63 (all columns), coalesced.
+// flip (nullable, [rows][cols] bytes): bit-flip augmentation of the patch matrix, v -> v + (1 - 2 v) where set
+// (base_layer.py:149-264 applied to the patches, convolutional.py:205-207).
 __global__ __launch_bounds__(256) void conv_unfold_rows(const float *__restrict__ x, float *__restrict__ patches, ConvGeom g,
-                                                         long long rows, int cols) {
+                                                         long long rows, int cols, const uint8_t *__restrict__ flip) {
     __shared__ int off[CONV_MAX_COLS], dydx[CONV_MAX_COLS];
     __shared__ long long base[64];
     __shared__ int y0s[64], x0s[64];
@@ -46,14 +48,17 @@ __global__ __launch_bounds__(256) void conv_unfold_rows(const float *__restrict_
         const int r = e / cols, c = e - r * cols;
         const int y = y0s[r] + (dydx[c] >> 16), xx = x0s[r] + (dydx[c] & 0xffff);
         const bool in = y >= 0 && y < g.H && xx >= 0 && xx < g.W;
-        out[e] = in ? x[base[r] + off[c]] : 0.0f;
+        float v = in ? x[base[r] + off[c]] : 0.0f;
+        if (flip && flip[r0 * cols + e]) v = v + (1.0f - 2.0f * v);
+        out[e] = v;
     }
 }
 
 // The same patches as the bit-planes a DWN layer reads: word (t, c) holds in bit r (patches[64 t + r][c] >= 0.5).
 // grid = ceil(rows / 64) blocks of 256 threads; lane = row, the four wavefronts share the columns.
 __global__ __launch_bounds__(256) void conv_unfold_planes(const float *__restrict__ x, unsigned long long *__restrict__ planes,
-                                                           ConvGeom g, long long rows, int cols) {
+                                                           ConvGeom g, long long rows, int cols,
+                                                           const uint8_t *__restrict__ flip) {
     __shared__ int off[CONV_MAX_COLS], dydx[CONV_MAX_COLS];
     conv_fill_columns(g, cols, off, dydx);
     __syncthreads();
@@ -75,8 +80,9 @@ __global__ __launch_bounds__(256) void conv_unfold_planes(const float *__restric
             const int c = cb + q;
             const int y = y0 + (dydx[c] >> 16), xx = x0 + (dydx[c] & 0xffff);
             const bool in = live && y >= 0 && y < g.H && xx >= 0 && xx < g.W;
-            const float v = in ? img[off[c]] : 0.0f;
-            const unsigned long long mask = __ballot(v >= 0.5f);
+            float v = in ? img[off[c]] : 0.0f;
+            if (flip && live && flip[r * cols + c]) v = v + (1.0f - 2.0f * v);  // the value the reference thresholds
+            const unsigned long long mask = __ballot(live && v >= 0.5f);
             if (q == lane) mine = mask;
         }
         if (lane < cnt) out[cb + lane] = mine;
@@ -130,8 +136,15 @@ extern "C" long long dl_unfold_rows(int B, int H, int W, int KH, int KW, int SH,
     return (long long)B * g.OH * g.OW;
 }
 
+extern "C" int dl_unfold_flip(const float *x, const uint8_t *flip, float *patches, void *planes, int B, int C, int H, int W,
+                              int KH, int KW, int SH, int SW, int PH, int PW, void *stream);
 extern "C" int dl_unfold(const float *x, float *patches, void *planes, int B, int C, int H, int W, int KH, int KW, int SH,
                          int SW, int PH, int PW, void *stream) {
+    return dl_unfold_flip(x, nullptr, patches, planes, B, C, H, W, KH, KW, SH, SW, PH, PW, stream);
+}
+
+extern "C" int dl_unfold_flip(const float *x, const uint8_t *flip, float *patches, void *planes, int B, int C, int H, int W,
+                              int KH, int KW, int SH, int SW, int PH, int PW, void *stream) {
     if (!x || (!patches && !planes)) return DL_ERR_NULL;
     ConvGeom g;
     int rc = conv_geom(g, B, C, H, W, KH, KW, SH, SW, PH, PW);
@@ -139,10 +152,10 @@ extern "C" int dl_unfold(const float *x, float *patches, void *planes, int B, in
     hipStream_t s = (hipStream_t)stream;
     const long long rows = (long long)B * g.OH * g.OW;
     const int cols = C * KH * KW, grid = dl_ceil_div(rows, 64);
-    if (patches) DL_TIMED("conv_unfold_rows", s, (conv_unfold_rows<<<grid, 256, 0, s>>>(x, patches, g, rows, cols)));
+    if (patches) DL_TIMED("conv_unfold_rows", s, (conv_unfold_rows<<<grid, 256, 0, s>>>(x, patches, g, rows, cols, flip)));
     if (planes)
         DL_TIMED("conv_unfold_planes", s,
-                 (conv_unfold_planes<<<grid, 256, 0, s>>>(x, (unsigned long long *)planes, g, rows, cols)));
+                 (conv_unfold_planes<<<grid, 256, 0, s>>>(x, (unsigned long long *)planes, g, rows, cols, flip)));
     return dl_launch_status();
 }
 

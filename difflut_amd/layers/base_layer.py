@@ -185,20 +185,30 @@ class LUTLayerMixin(nn.Module):
          self.grad_epsilon) = values
         self._flip_mask_buffer = None
 
+    def _flip_mask(self, shape, device):
+        """The positions the bit-flip augmentation inverts this call (training only; None = none): below 5 % an exact
+        count of positions drawn without replacement, otherwise one Bernoulli draw per entry - the two branches and
+        their generator calls of base_layer.py:149-264."""
+        if self.flip_probability <= 0.0 or not self.training:
+            return None
+        numel = 1
+        for d in shape:
+            numel *= d
+        if self.flip_probability < 0.05:
+            count = int(numel * self.flip_probability)
+            if count == 0:
+                return None
+            mask = torch.zeros(numel, dtype=torch.bool, device=device)
+            mask[torch.randperm(numel, device=device)[:count]] = True
+            return mask.view(shape)
+        return torch.bernoulli(torch.full(tuple(shape), self.flip_probability, device=device, dtype=torch.float32)).bool()
+
     def _apply_bit_flip(self, x):
         """Training only: x -> 1 - x on a random subset; the flip is detached so gradients flow as if
-        no bit had been flipped.  Below 5 % an exact count of positions is drawn (base_layer.py:149-264)."""
-        if self.flip_probability <= 0.0 or not self.training:
+        no bit had been flipped."""
+        mask = self._flip_mask(x.shape, x.device)
+        if mask is None:
             return x
-        if self.flip_probability < 0.05:
-            count = int(x.numel() * self.flip_probability)
-            if count == 0:
-                return x
-            mask = torch.zeros(x.numel(), dtype=torch.bool, device=x.device)
-            mask[torch.randperm(x.numel(), device=x.device)[:count]] = True
-            mask = mask.view_as(x)
-        else:
-            mask = torch.rand(x.shape, device=x.device) < self.flip_probability
         delta = torch.where(mask, 1.0 - 2.0 * x.detach(), torch.zeros_like(x))
         return x + delta
 

@@ -173,11 +173,11 @@ class ConvolutionalLayer(LUTLayerMixin, nn.Module):
 
     def _chained(self):
         """DWN trees in training mode run as one chained call that reads the image itself."""
-        return (self._kind == "dwn" and self.training and self.n_inputs_per_node <= ops.FAST_K
-                and self.flip_probability <= 0.0)
+        return self._kind == "dwn" and self.training and self.n_inputs_per_node <= ops.FAST_K
 
-    def _run_levels(self, patches, image=None):
-        """patches [rows, input_size] (or, chained, the image batch) -> [rows, out_channels] through the depth levels."""
+    def _run_levels(self, patches, image=None, flip=None):
+        """patches [rows, input_size] (or, chained, the image batch and the flip mask of its patch matrix) ->
+        [rows, out_channels] through the depth levels."""
         device = patches.device if patches is not None else image.device
         plans = self._level_plans(device)
         banks = [{name: bank.tensor() for name, bank in level.items()} for level in self._level_banks]
@@ -185,7 +185,8 @@ class ConvolutionalLayer(LUTLayerMixin, nn.Module):
         kind, h = self._kind, patches
         if image is not None:
             scalars = [self._level_scalars(level, "efd_scalars") for level in levels]
-            return ops.DWNStackFunction.apply(image, self._geometry(), plans, scalars, None, *[b["luts"] for b in banks])
+            source = self._geometry() if flip is None else (*self._geometry(), flip)
+            return ops.DWNStackFunction.apply(image, source, plans, scalars, None, *[b["luts"] for b in banks])
         if kind == "dwn" and self.training and self.n_inputs_per_node <= ops.FAST_K:
             scalars = [self._level_scalars(level, "efd_scalars") for level in levels]
             return ops.DWNStackFunction.apply(h, None, plans, scalars, None, *[b["luts"] for b in banks])
@@ -236,12 +237,13 @@ class ConvolutionalLayer(LUTLayerMixin, nn.Module):
         out_h = (x.shape[2] + 2 * self.padding[0] - self.receptive_field[0]) // self.stride[0] + 1
         out_w = (x.shape[3] + 2 * self.padding[1] - self.receptive_field[1]) // self.stride[1] + 1
         positions = out_h * out_w
+        # bit-flip augmentation of the patch matrix (convolutional.py:205-207): the mask is drawn here, the patch
+        # extraction applies it on the way (also when the patches only ever exist as bit-planes)
+        flip = self._flip_mask((batch * positions, self.input_size), x.device)
         if self._kind is not None and self._chained():
-            out = self._run_levels(None, image=x)  # patches only ever exist as bit-planes
+            out = self._run_levels(None, image=x, flip=flip)
         else:
-            patches = ops.UnfoldFunction.apply(x, self._geometry())  # (batch * positions, channels * kh * kw)
-            if self.training and self.flip_probability > 0.0:
-                patches = self._apply_bit_flip(patches)
+            patches = ops.UnfoldFunction.apply(x, self._geometry(), flip)  # (batch * positions, channels * kh * kw)
             out = self._run_levels(patches) if self._kind is not None else self._loop_trees(patches)
         out = out.view(batch, positions, self.out_channels).transpose(1, 2)
         out = out.reshape(batch, self.out_channels, out_h, out_w)

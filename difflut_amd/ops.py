@@ -92,14 +92,25 @@ class GatherFunction(torch.autograd.Function):
 
 
 # ----------------------------------------------------------------------------- patches of the convolutional layer
+def _flip_bytes(flip, shape):
+    """A flip mask as the contiguous byte matrix the kernels read (None stays None)."""
+    if flip is None:
+        return None
+    if tuple(flip.shape) != tuple(shape):
+        raise RuntimeError(f"flip mask {tuple(flip.shape)} does not match the patch matrix {tuple(shape)}")
+    flip = flip.contiguous()
+    return flip.view(torch.uint8) if flip.dtype == torch.bool else flip.to(torch.uint8)
+
+
 class UnfoldFunction(torch.autograd.Function):
     """x [B,C,H,W] -> patches [B*OH*OW, C*KH*KW] (nn.Unfold, transposed and flattened as
     difflut/layers/convolutional.py:199-205 does); backward folds the patch gradients back.
-    `geom` = (KH, KW, SH, SW, PH, PW)."""
+    `geom` = (KH, KW, SH, SW, PH, PW).  `flip` (optional bool/uint8 [rows, C*KH*KW]): entries of the patch matrix that
+    the bit-flip augmentation turns into 1 - value; noise, so the backward ignores it."""
 
     @staticmethod
-    def forward(ctx, x, geom):
-        nat.require_device(x)
+    def forward(ctx, x, geom, flip=None):
+        nat.require_device(x, flip)
         x = _f32(x)
         B, C, H, W = x.shape
         lib = nat.lib()
@@ -108,7 +119,8 @@ class UnfoldFunction(torch.autograd.Function):
             raise RuntimeError(f"receptive field {geom[:2]} with stride {geom[2:4]}, padding {geom[4:]} does not fit a "
                                f"{H}x{W} image")
         patches = torch.empty((rows, C * geom[0] * geom[1]), dtype=torch.float32, device=x.device)
-        nat.check(lib.dl_unfold(nat.ptr(x), nat.ptr(patches), None, B, C, H, W, *geom, nat.stream()))
+        flip = _flip_bytes(flip, patches.shape)
+        nat.check(lib.dl_unfold_flip(nat.ptr(x), nat.ptr(flip), nat.ptr(patches), None, B, C, H, W, *geom, nat.stream()))
         ctx.shape, ctx.geom = (B, C, H, W), geom
         return patches
 
@@ -117,7 +129,7 @@ class UnfoldFunction(torch.autograd.Function):
         gp = _f32(gp)
         gx = torch.empty(ctx.shape, dtype=torch.float32, device=gp.device)
         nat.check(nat.lib().dl_fold(nat.ptr(gp), 0, nat.ptr(gx), *ctx.shape, *ctx.geom, nat.stream()))
-        return gx, None
+        return gx, None, None
 
 
 # ----------------------------------------------------------------------------- DWN
@@ -191,11 +203,13 @@ class DWNStackFunction(torch.autograd.Function):
         None                  x [B, I] itself;
         a tensor [F, nbits]   thermometer thresholds: x is raw data [B, F], its code is produced directly
                               as bit-planes and x gets no gradient (the code is a step function of it);
-        a tuple (KH, KW, SH, SW, PH, PW)   x is an image batch [B, C, H, W]: the first layer reads its patch
+        a tuple (KH, KW, SH, SW, PH, PW[, flip])   x is an image batch [B, C, H, W]: the first layer reads its patch
                               matrix (rows = output positions), again produced directly as bit-planes; the
-                              input gradient is folded back from the tile-major patch gradient."""
+                              input gradient is folded back from the tile-major patch gradient.  `flip`
+                              (bool [rows, C*KH*KW], optional): patch entries the bit-flip augmentation inverts."""
         thresholds = source if torch.is_tensor(source) else None
-        geom = source if isinstance(source, tuple) else None
+        geom = tuple(source[:6]) if isinstance(source, tuple) else None
+        flip = source[6] if isinstance(source, tuple) and len(source) > 6 else None
         nat.require_device(x, thresholds, *luts)
         x = _f32(x)
         luts = tuple(_f32(t) for t in luts)
@@ -209,7 +223,8 @@ class DWNStackFunction(torch.autograd.Function):
                                    f"a {H}x{W} image")
             width = C * geom[0] * geom[1]
             planes = _bytes(lib.dl_dwn_planes_bytes(B, width), x.device)
-            nat.check(lib.dl_unfold(nat.ptr(x), None, nat.ptr(planes), Bi, C, H, W, *geom, nat.stream()))
+            flip = _flip_bytes(flip, (B, width))
+            nat.check(lib.dl_unfold_flip(nat.ptr(x), nat.ptr(flip), None, nat.ptr(planes), Bi, C, H, W, *geom, nat.stream()))
             ctx.image = ((Bi, C, H, W), geom)
         elif thresholds is None:
             B, width = x.shape

@@ -326,6 +326,12 @@ int dl_unfold(const float *x, float *patches, void *planes, int B, int C, int H,
               int KH, int KW, int SH, int SW, int PH, int PW, void *stream);
 int dl_fold(const float *gpatches, int tiled, float *gx, int B, int C, int H, int W,
             int KH, int KW, int SH, int SW, int PH, int PW, void *stream);
+/* dl_unfold with the layer's bit-flip augmentation applied to the patch matrix on the way
+ * (LUTLayerMixin._apply_bit_flip, difflut/layers/base_layer.py:149-264, called on the patches at
+ * convolutional.py:205-207): flip [rows, C KH KW] bytes (nullable), non-zero = that entry becomes v + (1 - 2 v)
+ * before it is written or thresholded.  The flip is noise, not a function of x: dl_fold is its backward too. */
+int dl_unfold_flip(const float *x, const uint8_t *flip, float *patches, void *planes, int B, int C, int H, int W,
+                   int KH, int KW, int SH, int SW, int PH, int PW, void *stream);
 
 /* ------------------------------------------------------------------------
  * Per-kernel timing.  No counterpart in the reference (it has no tracing at all).

@@ -278,3 +278,106 @@ def test_conv_layer_with_grouped_connections_against_tree_loops(kind):
     np.testing.assert_allclose(xt.grad.cpu().numpy(), orc.conv_fold(gp, x.shape, (3, 3), (1, 1), (0, 0)), rtol=1e-5, atol=5e-6)
     got = np.stack([getattr(node, pname).grad.cpu().numpy() for node in layer.first_layer_chunks[2].nodes])
     np.testing.assert_allclose(got, gch[2], rtol=1e-5, atol=5e-6)
+
+
+# ------------------------------------------------------------------------------ bit-flip augmentation, gradient rescaling
+def _conv_oracle(layer, kind, x, flip_mask, gy):
+    """Forward and backward of the tree loops on the patch matrix with `flip_mask` applied (None: no flip)."""
+    pname, fwd, bwd = _oracle_fns(kind)
+    B, C, H, W = x.shape
+    rf2, st2, pd2 = layer.receptive_field, layer.stride, layer.padding
+    oh, ow = (H + 2 * pd2[0] - rf2[0]) // st2[0] + 1, (W + 2 * pd2[1] - rf2[1]) // st2[1] + 1
+    chunks, trees = _tables(layer, pname)
+    patches = orc.conv_unfold(x, rf2, st2, pd2)
+    if flip_mask is not None:  # x + (1 - 2 x) in fp32, as base_layer.py:214-221 computes the flipped value
+        patches = np.where(flip_mask, patches + (np.float32(1.0) - np.float32(2.0) * patches), patches).astype(np.float32)
+    out, acts = orc.conv_trees_forward(patches, chunks, trees, layer.hidden_layers[0], fwd)
+    want = out.reshape(B, oh * ow, layer.out_channels).transpose(0, 2, 1).reshape(B, layer.out_channels, oh, ow)
+    gout = gy.reshape(B, layer.out_channels, oh * ow).transpose(0, 2, 1).reshape(-1, layer.out_channels)
+    gp, gch, gtr = orc.conv_trees_backward(patches, chunks, trees, layer.hidden_layers[0], acts, gout, bwd)
+    return want, orc.conv_fold(gp, x.shape, rf2, st2, pd2), gch, gtr
+
+
+def _check_conv_grads(layer, kind, xt, gx, gch, gtr):
+    pname = _oracle_fns(kind)[0]
+    np.testing.assert_allclose(xt.grad.cpu().numpy(), gx, rtol=1e-5, atol=5e-6)
+    for c, (sub, want_g) in enumerate(zip(layer.first_layer_chunks, gch)):
+        got = np.stack([getattr(node, pname).grad.cpu().numpy() for node in sub.nodes])
+        np.testing.assert_allclose(got, want_g, rtol=1e-5, atol=5e-6, err_msg=f"chunk {c}")
+    for t in (0, layer.out_channels - 1):
+        for l, sub in enumerate(layer.trees[t]):
+            got = np.stack([getattr(node, pname).grad.cpu().numpy() for node in sub.nodes])
+            np.testing.assert_allclose(got, gtr[t][l], rtol=1e-5, atol=5e-6, err_msg=f"tree {t} layer {l}")
+
+
+@pytest.mark.parametrize("kind,prob", [("dwn", 0.3), ("dwn", 0.02), ("probabilistic", 0.3), ("hybrid", 0.1)])
+def test_conv_layer_with_bit_flip_against_tree_loops_on_the_same_mask(kind, prob):
+    """flip_probability > 0 (convolutional.py:205-207): the mask the layer draws is reproduced from the same seed with
+    the same generator calls and handed to the oracle.  For DWN trees the chained bit-plane path stays on (the flip is
+    applied where the patch bits are formed); outputs bit-exact, gradients flow as if nothing had been flipped."""
+    torch.manual_seed(11)
+    layer = _build(kind, 2, 2, 5, 3, 1, 1, 2)
+    layer.flip_probability = prob
+    layer.train()
+    B, C, H, W = 3, 2, 7, 6
+    rng = np.random.default_rng(8)
+    x = rng.integers(0, 2, (B, C, H, W)).astype(np.float32) if kind != "probabilistic" else \
+        (0.02 + 0.96 * rng.random((B, C, H, W))).astype(np.float32)
+    if kind == "dwn":
+        x[0, 0, 0, :3] = [0.5, 0.49999997, 0.50000006]  # values whose flipped form sits at the threshold
+    rows, cols = B * 7 * 6, C * 9   # padding 1: output 7 x 6
+    xt = torch.tensor(x, device=DEV, requires_grad=True)
+    torch.manual_seed(77)
+    y = layer(xt)
+    torch.manual_seed(77)
+    if prob < 0.05:
+        mask = torch.zeros(rows * cols, dtype=torch.bool, device=DEV)
+        mask[torch.randperm(rows * cols, device=DEV)[:int(rows * cols * prob)]] = True
+        mask = mask.view(rows, cols)
+    else:
+        mask = torch.bernoulli(torch.full((rows, cols), prob, device=DEV, dtype=torch.float32)).bool()
+    assert 0 < int(mask.sum()) < rows * cols
+    gy = rng.standard_normal(tuple(y.shape)).astype(np.float32)
+    y.backward(torch.tensor(gy, device=DEV))
+    want, gx, gch, gtr = _conv_oracle(layer, kind, x, mask.cpu().numpy(), gy)
+    if kind == "dwn":
+        assert layer._chained()
+        assert np.array_equal(y.detach().cpu().numpy(), want)
+    else:
+        np.testing.assert_allclose(y.detach().cpu().numpy(), want, rtol=1e-5, atol=1e-6)
+    _check_conv_grads(layer, kind, xt, gx, gch, gtr)
+    # and the flip really changed something: the unflipped oracle differs
+    plain = _conv_oracle(layer, kind, x, None, gy)[0]
+    assert not np.array_equal(plain, want)
+    # eval mode never flips
+    layer.eval()
+    with torch.no_grad():
+        assert torch.equal(layer(xt), layer(xt))
+
+
+@pytest.mark.parametrize("mode", ["layerwise", "batchwise"])
+@pytest.mark.parametrize("subtract_mean", [False, True])
+@pytest.mark.parametrize("kind", ["dwn", "probabilistic"])
+def test_conv_layer_gradient_stabilization_against_formula(kind, mode, subtract_mean):
+    """grad_stabilization (base_layer.py:266-339 through the hook of convolutional.py:252-265): the gradient that
+    reaches the trees is (g - mean) * sqrt(target / (mean((g - mean)^2) + eps)), over the whole output or per image.
+    The oracle's tree loops are fed the rescaled gradient computed in float64 from that formula."""
+    torch.manual_seed(13)
+    layer = _build(kind, 2, 2, 4, 3, 1, 0, 3)
+    layer.grad_stabilization, layer.grad_target_std, layer.grad_subtract_mean, layer.grad_epsilon = mode, 0.7, subtract_mean, 1e-8
+    layer.train()
+    B, C, H, W = 4, 2, 6, 7
+    rng = np.random.default_rng(3)
+    x = (0.02 + 0.96 * rng.random((B, C, H, W))).astype(np.float32)
+    xt = torch.tensor(x, device=DEV, requires_grad=True)
+    y = layer(xt)
+    gy = (rng.standard_normal(tuple(y.shape)) * 3.0 + 0.5).astype(np.float32)
+    y.backward(torch.tensor(gy, device=DEV))
+    g = gy.reshape(B, -1).astype(np.float64)
+    axis = None if mode == "layerwise" else 1
+    if subtract_mean:
+        g = g - g.mean(axis=axis, keepdims=axis is not None)
+    var = (g ** 2).mean(axis=axis, keepdims=axis is not None)
+    g = (g * np.sqrt(0.7 / (var + 1e-8))).astype(np.float32).reshape(gy.shape)
+    want, gx, gch, gtr = _conv_oracle(layer, kind, x, None, g)
+    _check_conv_grads(layer, kind, xt, gx, gch, gtr)
