@@ -44,53 +44,57 @@ __device__ __forceinline__ unsigned dwn_shift_in(unsigned addr, u64 mask) {
 // piece of a row of x.  Rows past B give 0 bits.
 // CHECK: also clears *all_binary (preset to 1 by the caller) when some value is neither 0 nor 1.
 #define DWN_PACK_ROWS 16
+static inline int dwn_pack_grid_y(int BT) { return 4 * BT < 65535 ? 4 * BT : 65535; }
 template <int VEC, bool CHECK = false>
 __global__ __launch_bounds__(256) void dwn_pack_planes(const float *__restrict__ x, u64 *__restrict__ planes,
                                                         int B, int I, int *__restrict__ all_binary = nullptr) {
     constexpr int PIECES = 64 / DWN_PACK_ROWS;
-    const int t = blockIdx.y / PIECES, piece = blockIdx.y % PIECES;
     bool odd = false;  // saw a value other than 0 and 1
     const int i0 = (blockIdx.x * 256 + threadIdx.x) * VEC;
     if (i0 >= I) return;
-    const int r0 = t * 64 + piece * DWN_PACK_ROWS;
-    const int rows = min(DWN_PACK_ROWS, B - r0);  // <= 0 for pieces past the batch
-    const float *base = x + (size_t)r0 * I + i0;
-    unsigned acc[VEC];
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) acc[v] = 0u;
-    if (rows == DWN_PACK_ROWS) {
-#pragma unroll
-        for (int r = 0; r < DWN_PACK_ROWS; ++r) {
-            const float *src = base + (size_t)r * I;
-            if constexpr (VEC == 4) {
-                typedef float f4v __attribute__((ext_vector_type(4)));
-                const f4v q = __builtin_nontemporal_load(reinterpret_cast<const f4v *>(src));  // x is read once
-                acc[0] |= (q.x >= 0.5f ? 1u : 0u) << r;
-                acc[1] |= (q.y >= 0.5f ? 1u : 0u) << r;
-                acc[2] |= (q.z >= 0.5f ? 1u : 0u) << r;
-                acc[3] |= (q.w >= 0.5f ? 1u : 0u) << r;
-                if (CHECK)
-                    odd = odd || !((q.x == 0.0f || q.x == 1.0f) && (q.y == 0.0f || q.y == 1.0f) &&
-                                   (q.z == 0.0f || q.z == 1.0f) && (q.w == 0.0f || q.w == 1.0f));
-            } else {
-                const float v0 = __builtin_nontemporal_load(src);
-                acc[0] |= (v0 >= 0.5f ? 1u : 0u) << r;
-                if (CHECK) odd = odd || !(v0 == 0.0f || v0 == 1.0f);
+    const int pieces_total = PIECES * ((B + 63) / 64);
+    for (int by = blockIdx.y; by < pieces_total; by += gridDim.y) {  // grid.y is capped at 65535 (pieces of 16 rows)
+        const int t = by / PIECES, piece = by % PIECES;
+        const int r0 = t * 64 + piece * DWN_PACK_ROWS;
+        const int rows = min(DWN_PACK_ROWS, B - r0);  // <= 0 for pieces past the batch
+        const float *base = x + (size_t)r0 * I + i0;
+        unsigned acc[VEC];
+    #pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[v] = 0u;
+        if (rows == DWN_PACK_ROWS) {
+    #pragma unroll
+            for (int r = 0; r < DWN_PACK_ROWS; ++r) {
+                const float *src = base + (size_t)r * I;
+                if constexpr (VEC == 4) {
+                    typedef float f4v __attribute__((ext_vector_type(4)));
+                    const f4v q = __builtin_nontemporal_load(reinterpret_cast<const f4v *>(src));  // x is read once
+                    acc[0] |= (q.x >= 0.5f ? 1u : 0u) << r;
+                    acc[1] |= (q.y >= 0.5f ? 1u : 0u) << r;
+                    acc[2] |= (q.z >= 0.5f ? 1u : 0u) << r;
+                    acc[3] |= (q.w >= 0.5f ? 1u : 0u) << r;
+                    if (CHECK)
+                        odd = odd || !((q.x == 0.0f || q.x == 1.0f) && (q.y == 0.0f || q.y == 1.0f) &&
+                                       (q.z == 0.0f || q.z == 1.0f) && (q.w == 0.0f || q.w == 1.0f));
+                } else {
+                    const float v0 = __builtin_nontemporal_load(src);
+                    acc[0] |= (v0 >= 0.5f ? 1u : 0u) << r;
+                    if (CHECK) odd = odd || !(v0 == 0.0f || v0 == 1.0f);
+                }
+            }
+        } else {
+            for (int r = 0; r < rows; ++r) {
+    #pragma unroll
+                for (int v = 0; v < VEC; ++v) {
+                    const float val = base[(size_t)r * I + v];
+                    acc[v] |= (val >= 0.5f ? 1u : 0u) << r;
+                    if (CHECK) odd = odd || !(val == 0.0f || val == 1.0f);
+                }
             }
         }
-    } else {
-        for (int r = 0; r < rows; ++r) {
-#pragma unroll
-            for (int v = 0; v < VEC; ++v) {
-                const float val = base[(size_t)r * I + v];
-                acc[v] |= (val >= 0.5f ? 1u : 0u) << r;
-                if (CHECK) odd = odd || !(val == 0.0f || val == 1.0f);
-            }
-        }
+        unsigned short *out = reinterpret_cast<unsigned short *>(planes + (size_t)t * I + i0) + piece;
+    #pragma unroll
+        for (int v = 0; v < VEC; ++v) out[v * PIECES] = (unsigned short)acc[v];
     }
-    unsigned short *out = reinterpret_cast<unsigned short *>(planes + (size_t)t * I + i0) + piece;
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) out[v * PIECES] = (unsigned short)acc[v];
     if (CHECK && odd) *all_binary = 0;  // every writer stores the same value
 }
 __global__ void dwn_set_flag(int *flag, int value) {
@@ -855,9 +859,9 @@ static int dwn_forward_fast(const float *x, const int32_t *idx32, const float *l
                             int B, int I, int N, int k, int O, hipStream_t s) {
     const int BT = dwn_bt(B);
     if (I % 4 == 0 && ((uintptr_t)x & 15) == 0)
-        DL_TIMED("dwn_pack_planes", s, (dwn_pack_planes<4><<<dim3(dl_ceil_div(I, 1024), 4 * BT), 256, 0, s>>>(x, planes, B, I)));
+        DL_TIMED("dwn_pack_planes", s, (dwn_pack_planes<4><<<dim3(dl_ceil_div(I, 1024), dwn_pack_grid_y(BT)), 256, 0, s>>>(x, planes, B, I)));
     else
-        DL_TIMED("dwn_pack_planes", s, (dwn_pack_planes<1><<<dim3(dl_ceil_div(I, 256), 4 * BT), 256, 0, s>>>(x, planes, B, I)));
+        DL_TIMED("dwn_pack_planes", s, (dwn_pack_planes<1><<<dim3(dl_ceil_div(I, 256), dwn_pack_grid_y(BT)), 256, 0, s>>>(x, planes, B, I)));
     uint8_t *addrT = (uint8_t *)saved;
     switch (k) {
         case 1: dwn_launch_lookup<1>(planes, idx32, luts, y, addrT, nullptr, B, I, N, O, s); break;
@@ -1221,9 +1225,9 @@ extern "C" int dl_dwn_pack_planes(const float *x, void *planes, int B, int I, vo
     hipStream_t s = (hipStream_t)stream;
     const int BT = dwn_bt(B);
     if (I % 4 == 0 && ((uintptr_t)x & 15) == 0)
-        DL_TIMED("dwn_pack_planes", s, (dwn_pack_planes<4><<<dim3(dl_ceil_div(I, 1024), 4 * BT), 256, 0, s>>>(x, (u64 *)planes, B, I)));
+        DL_TIMED("dwn_pack_planes", s, (dwn_pack_planes<4><<<dim3(dl_ceil_div(I, 1024), dwn_pack_grid_y(BT)), 256, 0, s>>>(x, (u64 *)planes, B, I)));
     else
-        DL_TIMED("dwn_pack_planes", s, (dwn_pack_planes<1><<<dim3(dl_ceil_div(I, 256), 4 * BT), 256, 0, s>>>(x, (u64 *)planes, B, I)));
+        DL_TIMED("dwn_pack_planes", s, (dwn_pack_planes<1><<<dim3(dl_ceil_div(I, 256), dwn_pack_grid_y(BT)), 256, 0, s>>>(x, (u64 *)planes, B, I)));
     return dl_launch_status();
 }
 
@@ -1367,10 +1371,10 @@ extern "C" int dl_dwn_layer_eval_ws(const float *x, const int32_t *idx32, const 
     dwn_set_flag<<<1, 64, 0, s>>>(flag, 1);
     if (I % 4 == 0 && ((uintptr_t)x & 15) == 0)
         DL_TIMED("dwn_pack_planes", s,
-                 (dwn_pack_planes<4, true><<<dim3(dl_ceil_div(I, 1024), 4 * BT), 256, 0, s>>>(x, planes, B, I, flag)));
+                 (dwn_pack_planes<4, true><<<dim3(dl_ceil_div(I, 1024), dwn_pack_grid_y(BT)), 256, 0, s>>>(x, planes, B, I, flag)));
     else
         DL_TIMED("dwn_pack_planes", s,
-                 (dwn_pack_planes<1, true><<<dim3(dl_ceil_div(I, 256), 4 * BT), 256, 0, s>>>(x, planes, B, I, flag)));
+                 (dwn_pack_planes<1, true><<<dim3(dl_ceil_div(I, 256), dwn_pack_grid_y(BT)), 256, 0, s>>>(x, planes, B, I, flag)));
     uint8_t *none = (uint8_t *)const_cast<float *>(luts);
     switch (k) {
         case 1: dwn_launch_lookup<1>(planes, idx32, luts, y, none, nullptr, B, I, N, O, s, 0, 0, true, flag); break;

@@ -6,26 +6,28 @@
 // x is read through the cache (random but inside one 4*I-byte row), writes are coalesced.
 template <typename index_t>
 __global__ __launch_bounds__(256) void gather_fwd_kernel(const float *__restrict__ x, const index_t *__restrict__ idx,
-                                                          float *__restrict__ m, int I, long long NK) {
-    const int b = blockIdx.y;
-    const float *xrow = x + (size_t)b * I;
-    float *out = m + (size_t)b * NK;
-    for (long long p = (long long)blockIdx.x * 1024 + threadIdx.x; p < min(NK, ((long long)blockIdx.x + 1) * 1024);
-         p += 256)
-        out[p] = xrow[idx[p]];
+                                                          float *__restrict__ m, int B, int I, long long NK) {
+    for (int b = blockIdx.y; b < B; b += gridDim.y) {  // grid.y is capped at 65535 rows
+        const float *xrow = x + (size_t)b * I;
+        float *out = m + (size_t)b * NK;
+        for (long long p = (long long)blockIdx.x * 1024 + threadIdx.x; p < min(NK, ((long long)blockIdx.x + 1) * 1024);
+             p += 256)
+            out[p] = xrow[idx[p]];
+    }
 }
 
 // gx[b,i] = sum over CSR entries of input i of gm[b, pos]; fixed order, no atomics.
 __global__ __launch_bounds__(256) void gather_bwd_kernel(const float *__restrict__ gm, const int *__restrict__ inv_ptr,
                                                           const int *__restrict__ inv_pos, float *__restrict__ gx,
-                                                          int I, long long NK) {
-    const int b = blockIdx.y;
+                                                          int B, int I, long long NK) {
     const int i = blockIdx.x * 256 + threadIdx.x;
     if (i >= I) return;
-    const float *row = gm + (size_t)b * NK;
-    float acc = 0.0f;
-    for (int e = inv_ptr[i]; e < inv_ptr[i + 1]; ++e) acc += row[inv_pos[e]];
-    gx[(size_t)b * I + i] = acc;
+    for (int b = blockIdx.y; b < B; b += gridDim.y) {  // grid.y is capped at 65535 rows
+        const float *row = gm + (size_t)b * NK;
+        float acc = 0.0f;
+        for (int e = inv_ptr[i]; e < inv_ptr[i + 1]; ++e) acc += row[inv_pos[e]];
+        gx[(size_t)b * I + i] = acc;
+    }
 }
 
 // One wavefront per row of W; lowest index wins ties.
@@ -168,11 +170,11 @@ extern "C" int dl_gather_fwd(const float *x, const void *idx, int idx_bits, floa
     if (B <= 0 || I <= 0 || N <= 0 || k <= 0) return DL_ERR_SHAPE;
     if (idx_bits != 16 && idx_bits != 32) return DL_ERR_UNSUPPORTED;
     const long long NK = (long long)N * k;
-    dim3 grid(dl_ceil_div(NK, 1024), B);
+    dim3 grid(dl_ceil_div(NK, 1024), B < 65535 ? B : 65535);
     if (idx_bits == 16)
-        gather_fwd_kernel<int16_t><<<grid, 256, 0, (hipStream_t)stream>>>(x, (const int16_t *)idx, m, I, NK);
+        gather_fwd_kernel<int16_t><<<grid, 256, 0, (hipStream_t)stream>>>(x, (const int16_t *)idx, m, B, I, NK);
     else
-        gather_fwd_kernel<int32_t><<<grid, 256, 0, (hipStream_t)stream>>>(x, (const int32_t *)idx, m, I, NK);
+        gather_fwd_kernel<int32_t><<<grid, 256, 0, (hipStream_t)stream>>>(x, (const int32_t *)idx, m, B, I, NK);
     return dl_launch_status();
 }
 
@@ -180,8 +182,8 @@ extern "C" int dl_gather_bwd(const float *gm, const int32_t *inv_ptr, const int3
                              int N, int k, void *stream) {
     if (!gm || !inv_ptr || !inv_pos || !gx) return DL_ERR_NULL;
     if (B <= 0 || I <= 0 || N <= 0 || k <= 0) return DL_ERR_SHAPE;
-    gather_bwd_kernel<<<dim3(dl_ceil_div(I, 256), B), 256, 0, (hipStream_t)stream>>>(gm, inv_ptr, inv_pos, gx, I,
-                                                                                    (long long)N * k);
+    gather_bwd_kernel<<<dim3(dl_ceil_div(I, 256), B < 65535 ? B : 65535), 256, 0, (hipStream_t)stream>>>(
+        gm, inv_ptr, inv_pos, gx, B, I, (long long)N * k);
     return dl_launch_status();
 }
 
@@ -214,6 +216,7 @@ extern "C" int dl_thermometer_planes(const float *x, const float *thr, void *pla
                                      void *stream) {
     if (!x || !thr || !planes) return DL_ERR_NULL;
     if (B <= 0 || F <= 0 || nbits <= 0) return DL_ERR_SHAPE;
+    if (B > 4000000) return DL_ERR_UNSUPPORTED;  // batch tiles ride in grid.y (at most 65535 of them)
     hipStream_t s = (hipStream_t)stream;
     DL_TIMED("thermometer_planes", s,
              (thermometer_planes_kernel<<<dim3(dl_ceil_div(F, 64), dl_ceil_div(B, 64)), 256, 0, s>>>(

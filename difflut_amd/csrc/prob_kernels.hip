@@ -527,6 +527,7 @@ __global__ __launch_bounds__(256) void prob_fill_zero(float *p, long long n) {
 static int prob_check(int B, int I, int N, int k, int O) {
     if (B <= 0 || I <= 0 || N <= 0 || k <= 0 || O <= 0) return DL_ERR_SHAPE;
     if (k > DL_MAX_K) return DL_ERR_UNSUPPORTED;
+    if (B > 4000000) return DL_ERR_UNSUPPORTED;  // batch tiles ride in grid.y (at most 65535 of them, extra rows included)
     return DL_OK;
 }
 // the tiled path addresses a batch tile of xT with 32-bit byte offsets (input * 256)

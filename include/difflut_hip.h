@@ -18,6 +18,12 @@
  * All float tensors are fp32, row-major, contiguous.  Workspaces, `saved` buffers, bit-planes and tile-major
  * tensors must be 16-byte aligned (what hipMalloc and torch's allocator return is enough); fp32 tensors
  * take vectorised paths when they are 16-byte aligned and their row length is a multiple of 4.
+ *
+ * Size limits (DL_ERR_UNSUPPORTED beyond them, checked on the host before anything is launched):
+ * k <= DL_MAX_K; N * O * 2^k < 2^31 table entries per layer; I <= 2^28 for the k <= 6 DWN kernels;
+ * B <= 4 000 000 rows for the probabilistic entry points and dl_thermometer_planes (their batch tiles are a
+ * grid dimension); C * KH * KW <= 4096 patch columns for dl_unfold / dl_fold.  The gathers, the bit-plane
+ * packing and the DWN layers take any B that fits an int.
  */
 #ifndef DIFFLUT_HIP_H
 #define DIFFLUT_HIP_H

@@ -453,3 +453,37 @@ def test_argument_errors_are_reported_not_launched():
         _ops().DWNLayerFunction.apply(torch.zeros(2, 2), torch.zeros(1, 1, 4), None, 0.1, 0.1)
     with pytest.raises(IndexError):
         _ops().MappingPlan(torch.tensor([[0, 7]], device=DEV, dtype=torch.int32), 4)
+
+
+def test_row_counts_beyond_one_grid_dimension():
+    """B > 65535 rows for the gathers (RandomLayer.get_mapping, LearnableLayer eval) and more than 2^20 rows for the
+    bit-plane packing (patch matrices of large image batches): the kernels walk the rows a grid dimension cannot hold."""
+    from difflut_amd import _native as nat
+    lib = nat.lib()
+    rng = np.random.default_rng(5)
+    B, I, N, k = 70001, 9, 5, 2
+    x = rng.random((B, I)).astype(np.float32)
+    idx = rng.integers(0, I, (N, k)).astype(np.int16)
+    xd, idd = dev(x), torch.as_tensor(idx).to(DEV)
+    m = torch.empty(B, N * k, device=DEV)
+    nat.check(lib.dl_gather_fwd(xd.data_ptr(), idd.data_ptr(), 16, m.data_ptr(), B, I, N, k, nat.stream()))
+    assert np.array_equal(m.cpu().numpy(), x[:, idx.reshape(-1).astype(np.int64)])
+    plan = _ops().MappingPlan(idd.to(torch.int32), I)
+    gm = rng.standard_normal((B, N * k)).astype(np.float32)
+    gx = torch.empty(B, I, device=DEV)
+    nat.check(lib.dl_gather_bwd(dev(gm).data_ptr(), plan.inv_ptr.data_ptr(), plan.inv_pos.data_ptr(), gx.data_ptr(), B, I, N, k,
+                                nat.stream()))
+    want = np.zeros((B, I), np.float32)
+    for p, i in enumerate(idx.reshape(-1)):
+        want[:, i] += gm[:, p]
+    np.testing.assert_allclose(gx.cpu().numpy(), want, rtol=1e-6, atol=1e-6)
+    # bit-planes of 1 050 000 rows x 8 columns: 65 625 pieces of 16 rows
+    R, C = 1050000, 8
+    v = torch.rand(R, C, device=DEV)
+    planes = torch.zeros(lib.dl_dwn_planes_bytes(R, C) // 8, dtype=torch.int64, device=DEV)
+    nat.check(lib.dl_dwn_pack_planes(v.data_ptr(), planes.data_ptr(), R, C, nat.stream()))
+    BT = (R + 63) // 64
+    bits = torch.zeros(BT * 64, C, dtype=torch.int64, device=DEV)
+    bits[:R] = (v >= 0.5).long()
+    want_planes = (bits.view(BT, 64, C) << torch.arange(64, device=DEV).view(1, 64, 1)).sum(1)  # wraps into the sign bit
+    assert torch.equal(planes[:BT * C].view(BT, C), want_planes)

@@ -354,3 +354,27 @@ def test_probabilistic_layer_refuses_per_node_temperatures():
         layer.nodes[5].temperature.fill_(2.0)
     with pytest.raises(RuntimeError, match="different temperatures"):
         layer.temperature_value()
+
+
+def test_size_limits_and_argument_errors_are_reported_before_any_launch():
+    """Error codes of the C ABI on the host side: nothing below reaches a kernel launch, so it runs without a GPU."""
+    from difflut_amd import _native as nat
+    lib = nat.lib()
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.addressof(buf)
+    NULL, SHAPE, UNSUPPORTED, WORKSPACE = -1, -2, -3, -4
+    assert lib.dl_gather_fwd(None, p, 16, p, 4, 4, 4, 2, None) == NULL
+    assert lib.dl_gather_fwd(p, p, 8, p, 4, 4, 4, 2, None) == UNSUPPORTED            # index width
+    assert lib.dl_gather_bwd(p, p, p, p, 0, 4, 4, 2, None) == SHAPE
+    assert lib.dl_dwn_layer_fwd(p, p, p, p, p, p, 64, 4, 4, 4, 17, 1, None) == UNSUPPORTED   # k > DL_MAX_K
+    assert lib.dl_dwn_layer_fwd(p, p, p, p, p, p, 8, 4096, 16384, 8192, 6, 1, None) == WORKSPACE
+    assert lib.dl_dwn_layer_bwd(None, p, p, p, p, p, p, 0.1, 0.3, p, p, p, 8, 4096, 16384, 8192, 6, 1, None) == WORKSPACE
+    assert lib.dl_prob_layer_fwd(p, p, p, 1.0, p, p, 64, 4000001, 4, 4, 2, 1, None) == UNSUPPORTED  # batch tiles > grid.y
+    assert lib.dl_thermometer_planes(p, p, p, 4000001, 4, 2, None) == UNSUPPORTED
+    # 256 channels with a 5x5 field: more patch columns than the per-block offset table holds
+    assert lib.dl_unfold(p, p, None, 1, 256, 8, 8, 5, 5, 1, 1, 0, 0, None) == UNSUPPORTED
+    assert lib.dl_unfold(p, p, None, 1, 1, 3, 3, 5, 5, 1, 1, 0, 0, None) == SHAPE           # field larger than the image
+    assert lib.dl_unfold_rows(2, 8, 8, 3, 3, 1, 1, 0, 0) == 2 * 36
+    assert lib.dl_dwn_layer_fwd_static(p, p, p, p, p, 4097, 16384, 8, 6, 1, None) == -6
+    for code in (NULL, SHAPE, UNSUPPORTED, WORKSPACE, -5, -6):
+        assert len(lib.dl_error_string(code)) > 10
