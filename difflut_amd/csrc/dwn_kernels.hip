@@ -12,14 +12,15 @@
 //   forward   pack_planes : x [B,I] fp32 -> planes [B/64][I] u64 (bit r = x[64t+r][i] >= 0.5)
 //             lookup_fwd  : planes + idx + luts -> y [B,N*O] (LDS-transposed tiles) and
 //                           addrT [B/64][N][64] u8, the address of every (node,row), kept for backward
-//   backward  efd_table   : luts -> D[n][d][j][a'] = alpha * sum_kappa s(kappa_j) lut[kappa]
-//                           beta^popc((a^kappa)&~(1<<j)), a' = address with bit j squeezed out;
-//                           also clears the table-gradient output
-//             transpose_hist : gy [B,N*O] -> gyT [B/64][N*O][64]; per-node 2^k-bin histogram of gy
-//                           in LDS; blocks of one column tile leave partials that the last of them adds in a
-//                           fixed order (no floating-point atomics)
+//   backward  transpose_hist : gy [B,N*O] -> gyT [B/64][N*O][64]; per-node 2^k-bin histogram of gy
+//                           in LDS; blocks of one column tile leave partials per chunk of batch tiles.
+//                           The same launch carries the blocks that build the gather's coefficient tables
+//                           (efd_table_block): luts -> D[n][d][j][a'] = alpha * sum_kappa s(kappa_j) lut[kappa]
+//                           beta^popc((a^kappa)&~(1<<j)), a' = address with bit j squeezed out
 //             bwd_gx      : for every input i the (node,slot) pairs that read it (CSR):
-//                           gx[b,i] = sum gyT[c][b] * D[c][j][a'(b)]  - a gather in fixed order
+//                           gx[b,i] = sum gyT[c][b] * D[c][j][a'(b)]  - a gather in fixed order; its launch
+//                           also carries the blocks that add the histogram partials in chunk order (no
+//                           floating-point atomics anywhere)
 // k > 6 goes to the one-thread-per-element kernels of dwn_generic.hip.
 #include "dl_common.h"
 #include <mutex>
@@ -293,21 +294,29 @@ __global__ __launch_bounds__(256) void dwn_reduce_partials(DwnReduce r) { dwn_re
 //           memory, shared by the k slots of a node - but it amplifies rounding by
 //           (1+|beta|)^k / (1-beta), so it is only used for |beta| <= 1/2 (the default is 1/3).
 // alpha_n / beta_n (nullable): the nodes' own alpha and beta [N] instead of one value for the layer.
-__global__ __launch_bounds__(256) void dwn_efd_table(const float *__restrict__ luts, float *__restrict__ D,
-                                                      float *__restrict__ gluts, int NO, int K, float alpha, float beta,
-                                                      int sform, DwnReduce red, int table_blocks,
-                                                      const float *__restrict__ alpha_n = nullptr,
-                                                      const float *__restrict__ beta_n = nullptr, int O = 1) {
-    if ((int)blockIdx.x >= table_blocks) return dwn_reduce_block(red, blockIdx.x - table_blocks);
-    const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
+struct DwnTables {
+    const float *luts;   // null: no coefficient table wanted
+    float *D;
+    const float *scale;  // stabilised node: per-node factor (selects dwn_stable_table_block)
+    const float *alpha_n, *beta_n;
+    float alpha, beta;
+    int NO, K, O, sform;
+};
+static inline int dwn_table_blocks(const DwnTables &t) { return t.luts ? dl_ceil_div(t.NO, 4) : 0; }
+
+// 256 threads = four tables; `block` = index among the blocks that build tables
+__device__ __forceinline__ void dwn_efd_table_block(const DwnTables &tb, int block) {
+    const int c = block * 4 + (threadIdx.x >> 6);
     const int a = threadIdx.x & 63;
-    if (c >= NO) return;
-    if (alpha_n) alpha = alpha_n[c / O];
-    if (beta_n) beta = beta_n[c / O];
+    if (c >= tb.NO) return;
+    const int K = tb.K;
+    const float alpha = tb.alpha_n ? tb.alpha_n[c / tb.O] : tb.alpha;
+    const float beta = tb.beta_n ? tb.beta_n[c / tb.O] : tb.beta;
     const int L = 1 << K, Lh = L >> 1;
     const bool live = a < L;
-    const double v0 = live ? (double)luts[(size_t)c * L + a] : 0.0;
-    if (sform) {
+    const double v0 = live ? (double)tb.luts[(size_t)c * L + a] : 0.0;
+    float *__restrict__ D = tb.D;
+    if (tb.sform) {
         double v = v0;
         for (int m = 0; m < K; ++m) v += (double)beta * __shfl_xor(v, 1 << m);
         if (live) D[(size_t)c * L + a] = (float)((double)alpha / (1.0 - (double)beta) * v);
@@ -332,23 +341,21 @@ __global__ __launch_bounds__(256) void dwn_efd_table(const float *__restrict__ l
 // That weight is not a product over inputs, so the sums are taken directly, in double: one wavefront
 // per table keeps it in LDS and shares out the k * 2^(k-1) outputs (j, a'), one 2^(k-1)-term sum
 //   D[c][j][a'] = scale * sum_kappa' (lut[kappa' with bit j set] - lut[kappa' with bit j clear]) / (popc(a' ^ kappa') + 1)
-// each.
-__global__ __launch_bounds__(256) void dwn_stable_table(const float *__restrict__ luts, const float *__restrict__ scale,
-                                                         float *__restrict__ D, float *__restrict__ gluts, int NO, int K,
-                                                         int O, DwnReduce red, int table_blocks) {
-    if ((int)blockIdx.x >= table_blocks) return dwn_reduce_block(red, blockIdx.x - table_blocks);
+// each.  Called by every thread of the block.
+__device__ __forceinline__ void dwn_stable_table_block(const DwnTables &tb, int block) {
     __shared__ double rec[8];
     __shared__ float tab[4][64];
     if (threadIdx.x < 8) rec[threadIdx.x] = 1.0 / (double)(threadIdx.x + 1);
     const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int c = blockIdx.x * 4 + w;
+    const int c = block * 4 + w;
+    const int K = tb.K, NO = tb.NO;
     const int L = 1 << K, Lh = L >> 1;
     if (c < NO && lane < L) {
-        tab[w][lane] = luts[(size_t)c * L + lane];
+        tab[w][lane] = tb.luts[(size_t)c * L + lane];
     }
     __syncthreads();
     if (c >= NO) return;
-    const double sc = (double)scale[c / O];
+    const double sc = (double)tb.scale[c / tb.O];
     for (int o = lane; o < K * Lh; o += 64) {
         const int j = o / Lh, ap = o - j * Lh;
         const int low = (1 << j) - 1;
@@ -357,8 +364,12 @@ __global__ __launch_bounds__(256) void dwn_stable_table(const float *__restrict_
             const int lo = (kp & low) | ((kp & ~low) << 1);  // kappa' with a clear bit j put in
             acc += ((double)tab[w][lo | (1 << j)] - (double)tab[w][lo]) * rec[__popc(ap ^ kp)];
         }
-        D[((size_t)c * K + j) * Lh + ap] = (float)(sc * acc);
+        tb.D[((size_t)c * K + j) * Lh + ap] = (float)(sc * acc);
     }
+}
+__device__ __forceinline__ void dwn_table_block(const DwnTables &tb, int block) {
+    if (tb.scale) dwn_stable_table_block(tb, block);
+    else dwn_efd_table_block(tb, block);
 }
 
 // gluts[c][a] *= scale[c / O]: the stabilised node scales its table gradient as well
@@ -420,10 +431,11 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
                                                                float *__restrict__ gyT, float *__restrict__ gluts,
                                                                int B, int NO, int O, int L, int BP, int BT,
                                                                int tiles_per_chunk, float *__restrict__ partial,
-                                                               const float *__restrict__ scale = nullptr) {
+                                                               const float *__restrict__ scale, int chunks, DwnTables tb) {
     __shared__ float tile[64][DWN_HC + 1];       // [row][column]
     __shared__ float hist[DWN_HC][65];           // [column][bin]
     __shared__ uint8_t atile[DWN_HC][64 + 4];    // [column][row] addresses
+    if ((int)blockIdx.y >= chunks) return dwn_table_block(tb, ((int)blockIdx.y - chunks) * gridDim.x + blockIdx.x);
     const int c0 = blockIdx.x * DWN_HC;
     const int lane = threadIdx.x & 63;
     const int wave = dl_uniform(threadIdx.x >> 6);
@@ -502,7 +514,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
     }
     __syncthreads();
     // scale (nullable): the stabilised node multiplies a node's table gradient by its gradient_scale
-    dwn_hist_flush(hist, c0, cend, L, (long long)NO * L, (int)gridDim.y, partial, gluts, scale, O);
+    dwn_hist_flush(hist, c0, cend, L, (long long)NO * L, chunks, partial, gluts, scale, O);
 }
 
 // hist_tiled: the histogram alone, for gy that arrives tile-major ([B/64][N*O][64]).  Nothing has to be
@@ -515,9 +527,11 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
 template <bool GROUPS = false>
 __global__ __launch_bounds__(256) void dwn_bwd_hist_tiled(const float *__restrict__ gy, const uint8_t *__restrict__ addrT,
                                                            float *__restrict__ gluts, int NO, int O, int L, int BT,
-                                                           int tiles_per_chunk, float *__restrict__ partial, float *__restrict__ gyT = nullptr,
-                                                           int B = 0, int groups = 0, int gsize = 1, float inv_tau = 1.0f) {
+                                                           int tiles_per_chunk, float *__restrict__ partial, int chunks, DwnTables tb,
+                                                           float *__restrict__ gyT = nullptr, int B = 0, int groups = 0, int gsize = 1,
+                                                           float inv_tau = 1.0f) {
     __shared__ float hist[DWN_HC][65];  // [column][bin]
+    if ((int)blockIdx.y >= chunks) return dwn_table_block(tb, ((int)blockIdx.y - chunks) * gridDim.x + blockIdx.x);
     const int c0 = blockIdx.x * DWN_HC;
     const int lane = threadIdx.x & 63;
     const int wave = dl_uniform(threadIdx.x >> 6);
@@ -580,7 +594,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_hist_tiled(const float *__restric
         }
     }
     __syncthreads();
-    dwn_hist_flush(hist, c0, cend, L, (long long)NO * L, (int)gridDim.y, partial, gluts, nullptr, O);
+    dwn_hist_flush(hist, c0, cend, L, (long long)NO * L, chunks, partial, gluts, nullptr, O);
 }
 
 // ---------------------------------------------------------------------------------
@@ -597,9 +611,11 @@ template <int K, bool O1, bool SFORM, int WI = DWN_WI>
 __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT, const uint8_t *__restrict__ addrT,
                                                    const float *__restrict__ D, const int *__restrict__ inv_ptr,
                                                    const int *__restrict__ inv_pos, float *__restrict__ gx,
-                                                   int B, int I, int N, int O, int BT, int out_tiled) {
+                                                   int B, int I, int N, int O, int BT, int out_tiled, int gather_blocks,
+                                                   DwnReduce red) {
     constexpr int IS = 4 * WI;  // inputs per block
     __shared__ float tile[IS][65];  // [input][row]
+    if ((int)blockIdx.x >= gather_blocks) return dwn_reduce_block(red, (int)blockIdx.x - gather_blocks);
     constexpr int Lh = 1 << (K - 1);
     int slab, t;
     if (!dl_xcd_map((I + IS - 1) / IS, BT, slab, t)) return;
@@ -930,27 +946,29 @@ extern "C" int dl_dwn_layer_fwd_static(const float *x, const int32_t *idx32, con
 
 template <int K>
 static void dwn_launch_gx(const float *gyT, const uint8_t *addrT, const float *D, const int *inv_ptr, const int *inv_pos,
-                          float *gx, int B, int I, int N, int O, bool sform, int out_tiled, hipStream_t s) {
+                          float *gx, int B, int I, int N, int O, bool sform, int out_tiled, const DwnReduce &red,
+                          hipStream_t s) {
     const int BT = dwn_bt(B);
+    const int rb = dwn_reduce_blocks(red);  // the fixed-order sum of the histogram partials rides behind the gather's blocks
     // Long CSR lists per input (average N*k/I: ~70 on the first level of a convolutional layer, 15 under a learnable
     // mapping) want fewer inputs per wavefront: more, shorter and evenly filled blocks.  Measured at B = 4096, k = 6:
     // lists of 3 - 16 inputs per wavefront is best (169 vs 221 us); 7.7 - 4 inputs (67 vs 73 us); 15 - 4 (134 vs
     // 179 us); 31 - 4 (368 vs 442 us); 69 with tile-major output - 1 (249 vs 265 vs 375 us).
     if (O == 1 && sform && out_tiled && (long long)N * K >= 32LL * I) {
         const int grid_s = dl_xcd_grid(dl_ceil_div(I, 4), BT);
-        DL_TIMED("dwn_bwd_gx", s, (dwn_bwd_gx<K, true, true, 1><<<grid_s, 256, 0, s>>>(gyT, addrT, D, inv_ptr, inv_pos, gx, B,
-                                                                                     I, N, O, BT, out_tiled)));
+        DL_TIMED("dwn_bwd_gx", s, (dwn_bwd_gx<K, true, true, 1><<<grid_s + rb, 256, 0, s>>>(gyT, addrT, D, inv_ptr, inv_pos, gx, B,
+                                                                                          I, N, O, BT, out_tiled, grid_s, red)));
         return;
     }
     if (O == 1 && sform && (long long)N * K >= 6LL * I) {
         const int grid_s = dl_xcd_grid(dl_ceil_div(I, 4 * DWN_WI_SMALL), BT);
-        DL_TIMED("dwn_bwd_gx", s, (dwn_bwd_gx<K, true, true, DWN_WI_SMALL><<<grid_s, 256, 0, s>>>(
-                                      gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, BT, out_tiled)));
+        DL_TIMED("dwn_bwd_gx", s, (dwn_bwd_gx<K, true, true, DWN_WI_SMALL><<<grid_s + rb, 256, 0, s>>>(
+                                      gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, BT, out_tiled, grid_s, red)));
         return;
     }
     const int grid = dl_xcd_grid(dl_ceil_div(I, 4 * DWN_WI), BT);
 #define DWN_GX(O1_, S_) \
-    DL_TIMED("dwn_bwd_gx", s, (dwn_bwd_gx<K, O1_, S_><<<grid, 256, 0, s>>>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, BT, out_tiled)))
+    DL_TIMED("dwn_bwd_gx", s, (dwn_bwd_gx<K, O1_, S_><<<grid + rb, 256, 0, s>>>(gyT, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, BT, out_tiled, grid, red)))
     if (O == 1 && sform) DWN_GX(true, true);
     else if (O == 1) DWN_GX(true, false);
     else if (sform) DWN_GX(false, true);
@@ -980,42 +998,38 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
     float *partial = (float *)((char *)ws + dwn_table_bytes(N, k, O) + dwn_gyT_bytes(B, N, O));
     int col_tiles, chunks, tpc;
     dwn_hist_grid(NO, BT, col_tiles, chunks, tpc);
-    const dim3 hgrid(col_tiles, chunks);
     const bool sform = !scale && beta >= -0.5f && beta <= 0.5f;
+    // The coefficient tables of the gather depend on the tables only, so their blocks ride in the histogram's launch
+    // (extra rows of its grid, dispatched last: they fill the tail in which the histogram blocks drain); the
+    // fixed-order sum of the histogram partials rides in the gather's launch the same way.
+    DwnTables tb = {gx ? luts : nullptr, D, scale, alpha_n, beta_n, alpha, beta, (int)NO, k, O, sform ? 1 : 0};
+    const dim3 hgrid(col_tiles, chunks + dl_ceil_div(dwn_table_blocks(tb), col_tiles));
     if (head)
         DL_TIMED("dwn_bwd_hist_groups", s, (dwn_bwd_hist_tiled<true><<<hgrid, 256, 0, s>>>(
-                                               gy, addrT, gluts, (int)NO, O, L, BT, tpc, partial, gx ? gyT : nullptr, B, head->groups,
-                                               head->gsize, head->inv_tau)));
+                                               gy, addrT, gluts, (int)NO, O, L, BT, tpc, partial, chunks, tb, gx ? gyT : nullptr, B,
+                                               head->groups, head->gsize, head->inv_tau)));
     else if (gy_tiled)
         DL_TIMED("dwn_bwd_hist_tiled", s,
-                 (dwn_bwd_hist_tiled<false><<<hgrid, 256, 0, s>>>(gy, addrT, gluts, (int)NO, O, L, BT, tpc, partial)));
+                 (dwn_bwd_hist_tiled<false><<<hgrid, 256, 0, s>>>(gy, addrT, gluts, (int)NO, O, L, BT, tpc, partial, chunks, tb)));
     else if (gx)
         DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<true><<<hgrid, 256, 0, s>>>(
-                                                  gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc, partial, scale)));
+                                                  gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc, partial, scale, chunks, tb)));
     else
         DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<false><<<hgrid, 256, 0, s>>>(
-                                                  gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc, partial, scale)));
-    // the coefficient tables of the gather and the fixed-order sum of the histogram partials share one launch
+                                                  gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc, partial, scale, chunks, tb)));
     // (the row-major histogram's scale is applied in the sum; the tile-major ones scale afterwards)
     DwnReduce red = {chunks > 1 ? partial : nullptr, gluts, NO * L, chunks, (head || gy_tiled) ? nullptr : scale, L, O};
-    const int table_blocks = dl_ceil_div(NO, 4), red_blocks = dwn_reduce_blocks(red);
-    if (gx && scale)
-        DL_TIMED("dwn_stable_table", s, (dwn_stable_table<<<table_blocks + red_blocks, 256, 0, s>>>(luts, scale, D, gluts, (int)NO, k,
-                                                                                                  O, red, table_blocks)));
-    else if (gx)
-        DL_TIMED("dwn_efd_table", s, (dwn_efd_table<<<table_blocks + red_blocks, 256, 0, s>>>(
-                                         luts, D, gluts, (int)NO, k, alpha, beta, sform ? 1 : 0, red, table_blocks, alpha_n, beta_n, O)));
-    else if (red_blocks)
-        DL_TIMED("dwn_reduce_partials", s, (dwn_reduce_partials<<<red_blocks, 256, 0, s>>>(red)));
+    if (!gx && dwn_reduce_blocks(red))
+        DL_TIMED("dwn_reduce_partials", s, (dwn_reduce_partials<<<dwn_reduce_blocks(red), 256, 0, s>>>(red)));
     if (gx) {
         const float *src = gy_tiled ? gy : gyT;
         switch (k) {
-            case 1: dwn_launch_gx<1>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, s); break;
-            case 2: dwn_launch_gx<2>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, s); break;
-            case 3: dwn_launch_gx<3>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, s); break;
-            case 4: dwn_launch_gx<4>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, s); break;
-            case 5: dwn_launch_gx<5>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, s); break;
-            default: dwn_launch_gx<6>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, s); break;
+            case 1: dwn_launch_gx<1>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, red, s); break;
+            case 2: dwn_launch_gx<2>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, red, s); break;
+            case 3: dwn_launch_gx<3>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, red, s); break;
+            case 4: dwn_launch_gx<4>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, red, s); break;
+            case 5: dwn_launch_gx<5>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, red, s); break;
+            default: dwn_launch_gx<6>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, red, s); break;
         }
     }
     if (scale && (gy_tiled || head))  // the row-major histogram applies the scale when it flushes
