@@ -85,10 +85,8 @@ def algorithmic_bytes(B, I, N, k, O):
     per_kernel = {
         "dwn_pack_planes": x,                         # reads every input once
         "dwn_lookup_fwd": y + tables + mapping,       # writes every output once
-        "dwn_bwd_transpose_hist": y + tables,         # reads gy once, writes the table gradients
-        "dwn_bwd_gx": x + tables + mapping,           # writes every input gradient once
-        "dwn_efd_table": tables,
-        "dl_fill_zero": tables,
+        "dwn_bwd_transpose_hist": y + tables,         # reads gy once, reads the tables (its launch builds the coefficients)
+        "dwn_bwd_gx": x + tables + mapping,           # writes every input gradient once and the table gradients
     }
     return fwd, bwd, per_kernel
 
