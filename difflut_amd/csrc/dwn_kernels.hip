@@ -410,6 +410,24 @@ __device__ __forceinline__ int dwn_quad_xor(int v) {
     constexpr int ctrl = X == 1 ? 0xB1 : (X == 2 ? 0x4E : 0x1B);  // quad_perm [1,0,3,2] / [2,3,0,1] / [3,2,1,0]
     return __builtin_amdgcn_update_dpp(0, v, ctrl, 0xf, 0xf, true);
 }
+// The four lanes of a quad hold four rows of one column: (address a, value v), lane rank hr = lane & 3.  Lanes with equal
+// addresses are merged: `sum` = v plus the values of the partners with the same address (adding 0 for the others keeps
+// the order of additions), and the function says whether this lane is the one that adds `sum` to the bin - the
+// lowest-ranked lane of its group.  Partner hr ^ 1 ranks lower when hr is odd, partners hr ^ 2 and hr ^ 3 when hr >= 2;
+// written on booleans so that the comparisons stay lane masks in scalar registers.
+__device__ __forceinline__ bool dwn_quad_merge(unsigned a, float v, int hr, float &sum) {
+    const unsigned a1 = (unsigned)dwn_quad_xor<1>((int)a), a2 = (unsigned)dwn_quad_xor<2>((int)a),
+                   a3 = (unsigned)dwn_quad_xor<3>((int)a);
+    const float v1 = __int_as_float(dwn_quad_xor<1>(__float_as_int(v))), v2 = __int_as_float(dwn_quad_xor<2>(__float_as_int(v))),
+                v3 = __int_as_float(dwn_quad_xor<3>(__float_as_int(v)));
+    const bool e1 = a1 == a, e2 = a2 == a, e3 = a3 == a;
+    sum = v;
+    sum += e1 ? v1 : 0.0f;
+    sum += e2 ? v2 : 0.0f;
+    sum += e3 ? v3 : 0.0f;
+    const bool odd = (hr & 1) != 0, upper = (hr & 2) != 0;
+    return !((e1 & odd) | ((e2 | e3) & upper));
+}
 // End of a histogram block: the table gradient in a fixed order of additions.  With one chunk of batch tiles per
 // column tile the block's bins are the result.  With several, every block stores its bins as a partial
 // ([chunk][column][bin]) and dwn_reduce_partials adds them in chunk order afterwards, so the sums do not depend on the
@@ -434,7 +452,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
                                                                const float *__restrict__ scale, int chunks, DwnTables tb) {
     __shared__ float tile[64][DWN_HC + 1];       // [row][column]
     __shared__ float hist[DWN_HC][65];           // [column][bin]
-    __shared__ uint8_t atile[DWN_HC][64 + 4];    // [column][row] addresses
+    __shared__ __align__(16) uint8_t atile[DWN_HC][64 + 4];  // [column][row] addresses
     if ((int)blockIdx.y >= chunks) return dwn_table_block(tb, ((int)blockIdx.y - chunks) * gridDim.x + blockIdx.x);
     const int c0 = blockIdx.x * DWN_HC;
     const int lane = threadIdx.x & 63;
@@ -448,7 +466,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
     const int N = NO / O;
     const int wc0 = wave * (DWN_HC / 4);  // my wavefront's first column
     float4 pre[4];
-    unsigned apre[DWN_HC / 4];  // addresses of my 16 columns for the tile being fetched (lane = row)
+    unsigned apre[DWN_HC / 16];  // addresses of my 16 columns for the tile being fetched: four rows per lane and pass
     auto fetch = [&](int t) {
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
@@ -469,9 +487,9 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
             }
         }
 #pragma unroll
-        for (int u = 0; u < DWN_HC / 4; ++u) {
-            const int c = min(c0 + wc0 + u, NO - 1);
-            apre[u] = addrT[((size_t)t * N + c / O) * 64 + lane];
+        for (int p = 0; p < DWN_HC / 16; ++p) {  // pass p: column wc0 + 4p + lane / 16, rows 4 (lane % 16) .. + 3, one 32-bit load
+            const int c = min(c0 + wc0 + 4 * p + (lane >> 4), NO - 1);
+            apre[p] = *reinterpret_cast<const unsigned *>(addrT + ((size_t)t * N + c / O) * 64 + 4 * (lane & 15));
         }
     };
     if (t_begin < t_end) fetch(t_begin);
@@ -484,7 +502,8 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
             dst[0] = pre[p].x; dst[1] = pre[p].y; dst[2] = pre[p].z; dst[3] = pre[p].w;
         }
 #pragma unroll
-        for (int u = 0; u < DWN_HC / 4; ++u) atile[wc0 + u][lane] = (uint8_t)apre[u];
+        for (int p = 0; p < DWN_HC / 16; ++p)
+            *reinterpret_cast<unsigned *>(&atile[wc0 + 4 * p + (lane >> 4)][4 * (lane & 15)]) = apre[p];
         __syncthreads();
         if (t + 1 < t_end) fetch(t + 1);
         if (WRITE_T) {
@@ -498,17 +517,8 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
             for (int r0 = 0; r0 < 64; r0 += 4) {
                 const float v = tile[r0 + hr][hc];  // rows past B carry 0
                 const unsigned a = atile[hc][r0 + hr];
-                float sum = v;
-                bool leader = true;
-                const unsigned a1 = (unsigned)dwn_quad_xor<1>((int)a), a2 = (unsigned)dwn_quad_xor<2>((int)a),
-                               a3 = (unsigned)dwn_quad_xor<3>((int)a);
-                const float v1 = __int_as_float(dwn_quad_xor<1>(__float_as_int(v))),
-                            v2 = __int_as_float(dwn_quad_xor<2>(__float_as_int(v))),
-                            v3 = __int_as_float(dwn_quad_xor<3>(__float_as_int(v)));
-                if (a1 == a) { sum += v1; leader = leader && (hr ^ 1) > hr; }
-                if (a2 == a) { sum += v2; leader = leader && (hr ^ 2) > hr; }
-                if (a3 == a) { sum += v3; leader = leader && (hr ^ 3) > hr; }
-                if (leader) hist[hc][a] += sum;
+                float sum;
+                if (dwn_quad_merge(a, v, hr, sum)) hist[hc][a] += sum;
             }
         }
     }
@@ -576,17 +586,8 @@ __global__ __launch_bounds__(256) void dwn_bwd_hist_tiled(const float *__restric
                 for (int e = 0; e < 4; ++e) {
                     const float v = vs[e];
                     const unsigned a = (aw[m] >> (8 * e)) & 0xffu;
-                    float sum = v;
-                    bool leader = true;
-                    const unsigned a1 = (unsigned)dwn_quad_xor<1>((int)a), a2 = (unsigned)dwn_quad_xor<2>((int)a),
-                                   a3 = (unsigned)dwn_quad_xor<3>((int)a);
-                    const float v1 = __int_as_float(dwn_quad_xor<1>(__float_as_int(v))),
-                                v2 = __int_as_float(dwn_quad_xor<2>(__float_as_int(v))),
-                                v3 = __int_as_float(dwn_quad_xor<3>(__float_as_int(v)));
-                    if (a1 == a) { sum += v1; leader = leader && (hr ^ 1) > hr; }
-                    if (a2 == a) { sum += v2; leader = leader && (hr ^ 2) > hr; }
-                    if (a3 == a) { sum += v3; leader = leader && (hr ^ 3) > hr; }
-                    if (leader) hist[hc][a] += sum;
+                    float sum;
+                    if (dwn_quad_merge(a, v, hr, sum)) hist[hc][a] += sum;
                 }
             }
 #pragma unroll
