@@ -239,6 +239,18 @@ __global__ __launch_bounds__(64 * DWN_FW) void dwn_lookup_fwd(const u64 *__restr
         return;
     }
     if (CHAIN && !y) return;
+    if (cend == DWN_TC && t * 64 + 64 <= B && (NO & 3) == 0 && (((uintptr_t)y) & 15) == 0) {
+        // whole tile: 16-byte stores, a wavefront covers two 512-byte row pieces per instruction
+        typedef float f4v __attribute__((ext_vector_type(4)));
+#pragma unroll
+        for (int pass = 0; pass < 64 * DWN_TC / 4 / (64 * DWN_FW); ++pass) {
+            const int e = pass * 64 * DWN_FW + threadIdx.x;
+            const int r = e / (DWN_TC / 4), c4 = (e % (DWN_TC / 4)) * 4;
+            const f4v v = {tile[c4][r], tile[c4 + 1][r], tile[c4 + 2][r], tile[c4 + 3][r]};
+            __builtin_nontemporal_store(v, reinterpret_cast<f4v *>(&y[(size_t)(t * 64 + r) * NO + c0 + c4]));
+        }
+        return;
+    }
     for (int e = threadIdx.x; e < 64 * DWN_TC; e += 64 * DWN_FW) {
         const int r = e / DWN_TC, cc = e % DWN_TC;
         const int b = t * 64 + r;
@@ -770,6 +782,18 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT,
         return;
     }
     __syncthreads();
+    if (IS % 4 == 0 && iend == IS && t * 64 + 64 <= B && (I & 3) == 0 && (((uintptr_t)gx) & 15) == 0) {
+        typedef float f4v __attribute__((ext_vector_type(4)));  // whole tile: 16-byte stores
+#pragma unroll
+        for (int pass = 0; pass < (64 * IS / 4 + 255) / 256; ++pass) {
+            const int e = pass * 256 + threadIdx.x;
+            if (64 * IS / 4 % 256 != 0 && e >= 64 * IS / 4) break;
+            const int r = e / (IS / 4), i4 = (e % (IS / 4)) * 4;
+            const f4v v = {tile[i4][r], tile[i4 + 1][r], tile[i4 + 2][r], tile[i4 + 3][r]};
+            __builtin_nontemporal_store(v, reinterpret_cast<f4v *>(&gx[(size_t)(t * 64 + r) * I + i0 + i4]));
+        }
+        return;
+    }
     for (int e = threadIdx.x; e < 64 * IS; e += 256) {
         const int r = e / IS, ii = e % IS;
         const int b = t * 64 + r;
