@@ -110,22 +110,35 @@ def stack_bytes(B, F, nbits, widths, k, train):
 
 
 PRERUN_MS = 60.0
+PRERUN_MAX_MS = 800.0
 
 
-def steady_state(step, ms=PRERUN_MS):
-    """Brings the device to its sustained clocks before anything is timed: after an idle phase (the setup above every
-    timed loop is mostly host work) the first ~60 steps of the headline workload run up to 14 % slower (0.337 ms
-    against 0.295 ms per step, settled after about 20 ms).  The step is run, untimed, for `ms` milliseconds; the
-    warm-up steps asked for on the command line and the timed steps follow without a pause."""
+def steady_state(step, ms=PRERUN_MS, max_ms=PRERUN_MAX_MS, chunk=8):
+    """Brings device and host to their sustained state before anything is timed.  After an idle phase (the setup above
+    every timed loop is mostly host work) the first ~60 steps of the headline workload run up to 14 % slower (0.337 ms
+    against 0.295 ms per step, settled after about 20 ms), and the first ~200 steps of a freshly built layer object
+    through autograd and torch's allocator read 9 % slower than all later ones.  The step is run, untimed, in chunks
+    of `chunk` for at least `ms` milliseconds and until the last three chunks agree within 1 % with each other and with
+    the fastest chunk so far (at most `max_ms`); the warm-up steps asked for on the command line and the timed steps
+    follow without a pause.  Returns the number of steps run."""
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    n = 0
-    while (time.perf_counter() - t0) * 1e3 < ms:
-        for _ in range(4):
+    t_begin = time.perf_counter()
+    times = []
+    while True:
+        t0 = time.perf_counter()
+        for _ in range(chunk):
             step()
         torch.cuda.synchronize()
-        n += 4
-    return n
+        now = time.perf_counter()
+        times.append(now - t0)
+        elapsed = (now - t_begin) * 1e3
+        if elapsed >= max_ms:
+            break
+        if elapsed >= ms and len(times) >= 4:
+            last = times[-3:]
+            if max(last) <= 1.01 * min(last) and max(last) <= 1.01 * min(times):
+                break
+    return chunk * len(times)
 
 
 def time_steps(step, steps, warmup):
@@ -474,13 +487,10 @@ def layer_api_step(args, x, gy, idx, luts):
         bank.grad = None
         layer(xg).backward(gy)
 
-    # the first timed loop of a fresh layer in a process reads about 9 % slower than every later one (0.323 against
-    # 0.297 ms, torch's allocator and autograd warming up); it is run and reported as `first_loop_ms_per_step`
-    first = time_steps(step, args.steps, args.warmup)
     ms = time_steps(step, args.steps, args.warmup)
     fwd_b, bwd_b, _ = algorithmic_bytes(B, I, N, k, O)
     gbs = (fwd_b + bwd_b) / (ms * 1e-3) / 1e9
-    return {"ms_per_step": ms, "first_loop_ms_per_step": first, "value": B * N / (ms * 1e-3), "unit": "node-evals/s",
+    return {"ms_per_step": ms, "value": B * N / (ms * 1e-3), "unit": "node-evals/s",
             "call": "RandomLayer(...).forward(x).backward(gy), tensors allocated per call by torch's caching allocator",
             "roofline_step": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
                               "algorithmic_bytes_per_step": fwd_b + bwd_b}}
@@ -618,8 +628,9 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "steady_state_prerun": {"ms": PRERUN_MS, "steps": prerun_steps,
-                                "why": "untimed steps before the warm-up: device clocks settle about 20 ms after idle"},
+        "steady_state_prerun": {"min_ms": PRERUN_MS, "max_ms": PRERUN_MAX_MS, "steps": prerun_steps,
+                                "why": "untimed steps before the warm-up, until chunks of 8 steps agree within 1 %: "
+                                       "device clocks settle about 20 ms after idle"},
         "config": {"workload": args.workload, "batch": B, "inputs": I, "nodes": N, "k": k, "output_dim": O,
                    "pass": "forward + EFD backward (input and table gradients)", "seed": 0, "mapping_seed": 42},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": dom_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
