@@ -163,19 +163,27 @@ __global__ __launch_bounds__(64 * PROB_FW) void prob_fwd_t(const float *__restri
     }
 }
 
-// one wavefront per (column, chunk of batch tiles); 4 wavefronts per block.
+// one wavefront per (column, chunk of batch tiles); W wavefronts per block.
 // HYB (hybrid node): the table is used as given and the input gradient carries the factor
 // q / (q + 1e-8), q = x_j (1 - x_j), of that node's backward.
-template <int K, bool HYB>
-__global__ __launch_bounds__(256) void prob_bwd_t(const float *__restrict__ xT, const float *__restrict__ gyT,
-                                                   const int *__restrict__ idx32, const float *__restrict__ sig,
-                                                   float *__restrict__ gmT, float *__restrict__ gpart, int I, int N,
-                                                   int O, int BT, int tiles_per_chunk, int want_gm) {
+// W = 4: gy arrives tile-major (gyT [B/64][N*O][64], written by prob_to_tiles).  W = 16 (k <= 4, where 16 wavefronts
+// of this kernel fit a CU's registers): gy is the row-major gradient itself; the block's 16 columns are 64 contiguous
+// bytes of a row, the 64 x 16 piece of a batch tile is fetched one value per thread a tile ahead and turned through
+// the LDS (two buffers, one barrier per tile), so the re-tiling pass and its launch are not needed.
+template <int K, bool HYB, int W = 4>
+__global__ __launch_bounds__(64 * W) void prob_bwd_t(const float *__restrict__ xT, const float *__restrict__ gyT,
+                                                     const int *__restrict__ idx32, const float *__restrict__ sig,
+                                                     float *__restrict__ gmT, float *__restrict__ gpart, int I, int N,
+                                                     int O, int BT, int tiles_per_chunk, int want_gm, int B = 0) {
     constexpr int L = 1 << K;
+    constexpr bool GYROW = W == 16;
+    __shared__ float gturn[GYROW ? 2 : 1][GYROW ? W : 1][GYROW ? 65 : 1];  // [buffer][column][row]
     const int NO = N * O;
     const int lane = threadIdx.x & 63;
-    const int c = blockIdx.x * 4 + dl_uniform(threadIdx.x >> 6);
-    if (c >= NO) return;
+    const int c_raw = blockIdx.x * W + dl_uniform(threadIdx.x >> 6);
+    if (!GYROW && c_raw >= NO) return;
+    const bool live = c_raw < NO;        // GYROW: wavefronts past the last column still serve the barriers
+    const int c = live ? c_raw : NO - 1;
     const int chunk = blockIdx.y;
     const int n = c / O;
     const int lane4 = lane * 4;
@@ -189,18 +197,30 @@ __global__ __launch_bounds__(256) void prob_bwd_t(const float *__restrict__ xT, 
     for (int a = 0; a < L; ++a) acc[a] = 0.0f;
     const int t0 = chunk * tiles_per_chunk, t1 = min(BT, t0 + tiles_per_chunk);
     float nxs[K], ng = 0.0f;  // operands of the next batch tile, requested one tile ahead
+    const int trow = threadIdx.x >> 4, tcol = threadIdx.x & 15;  // GYROW: my value of the 64 x 16 piece
     auto request = [&](int t) {
         const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc((void *)(xT + (size_t)t * I * 64), 0, I * 256, PROB_RSRC);
 #pragma unroll
         for (int j = 0; j < K; ++j) nxs[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_x, lane4, off[j], 0));
-        ng = gyT[((size_t)t * NO + c) * 64 + lane];
+        if (GYROW) {
+            const int b = t * 64 + trow, cc = blockIdx.x * W + tcol;
+            ng = (b < B && cc < NO) ? gyT[(size_t)b * NO + cc] : 0.0f;
+        } else {
+            ng = gyT[((size_t)t * NO + c) * 64 + lane];
+        }
     };
     if (t0 < t1) request(t0);
     for (int t = t0; t < t1; ++t) {
         float xs[K];
 #pragma unroll
         for (int j = 0; j < K; ++j) xs[j] = nxs[j];
-        const float g = ng;
+        float g = ng;
+        if (GYROW) {
+            const int buf = (t - t0) & 1;
+            gturn[buf][tcol][trow] = ng;
+            __syncthreads();  // the other buffer is rewritten only after the next barrier: its readers are done by then
+            g = gturn[buf][threadIdx.x >> 6][lane];
+        }
         if (t + 1 < t1) request(t + 1);
         // forward fold, keeping the differences d_j[a] = lvl_j[2a+1] - lvl_j[2a] of every level
         float diff[L > 1 ? L - 1 : 1];  // level j occupies [L - (L >> j), L - (L >> (j+1)))
@@ -246,7 +266,7 @@ __global__ __launch_bounds__(256) void prob_bwd_t(const float *__restrict__ xT, 
         }
 #pragma unroll
         for (int a = 0; a < L; ++a) acc[a] = fmaf(g, bar[a], acc[a]);
-        if (want_gm) {
+        if (want_gm && live) {
 #pragma unroll
             for (int j = 0; j < K; ++j) gmT[(((size_t)t * NO + c) * K + j) * 64 + lane] = g * dx[j];
         }
@@ -272,7 +292,7 @@ __global__ __launch_bounds__(256) void prob_bwd_t(const float *__restrict__ xT, 
     int a = 0;
 #pragma unroll
     for (int r = 0; r < K; ++r) a |= ((lane >> (5 - r)) & 1) << r;
-    if ((lane & ((64 >> K) - 1)) == 0) gpart[((size_t)chunk * NO + c) * L + a] = mine;
+    if (live && (lane & ((64 >> K) - 1)) == 0) gpart[((size_t)chunk * NO + c) * L + a] = mine;
 }
 
 // graw[n,a,d] = sigmoid'(w/T)/T * sum over chunks of gpart[chunk][c][a];
@@ -631,13 +651,24 @@ extern "C" int dl_prob_layer_bwd(const float *x, const void *saved, const int32_
         DL_TIMED("prob_sig_table", s, (prob_sig_table<<<dl_ceil_div(WT, 256), 256, 0, s>>>(raw_w, inv_t, sig, N, L, O)));
         DL_TIMED("prob_to_tiles_x", s, (prob_to_tiles<<<dim3(dl_ceil_div(I, 64), BT), 256, 0, s>>>(x, xT, B, I)));
     }
-    DL_TIMED("prob_to_tiles_gy", s, (prob_to_tiles<<<dim3(dl_ceil_div(NO, 64), BT), 256, 0, s>>>(gy, gyT, B, NO)));
+    if (k <= 4) {  // 16 wavefronts per block take gy as it is (see prob_bwd_t)
+#define CALL(KK)                                                                                                       \
+    DL_TIMED("prob_bwd_t", s,                                                                                          \
+             (prob_bwd_t<KK, false, 16><<<dim3(dl_ceil_div(NO, 16), chunks), 1024, 0, s>>>(xT, gy, idx32, sig, gmT, gpart, I, N, \
+                                                                                        O, BT, tpc, gx != nullptr, B)))
+        switch (k) {
+            case 1: CALL(1); break; case 2: CALL(2); break; case 3: CALL(3); break; default: CALL(4); break;
+        }
+#undef CALL
+    } else {
+        DL_TIMED("prob_to_tiles_gy", s, (prob_to_tiles<<<dim3(dl_ceil_div(NO, 64), BT), 256, 0, s>>>(gy, gyT, B, NO)));
 #define CALL(KK)                                                                                                    \
     DL_TIMED("prob_bwd_t", s,                                                                                       \
              (prob_bwd_t<KK, false><<<dim3(dl_ceil_div(NO, 4), chunks), 256, 0, s>>>(xT, gyT, idx32, sig, gmT, gpart, I, N, O, \
                                                                                   BT, tpc, gx != nullptr)))
-    PROB_DISPATCH(k, CALL)
+        PROB_DISPATCH(k, CALL)
 #undef CALL
+    }
     const ProbReduce R = {gpart, sig, inv_t, graw, N, L, O, chunks};
     prob_launch_gather_and_reduce(gmT, inv_ptr, inv_pos, gx, B, I, N, k, O, BT, R, WT, s);
     return dl_launch_status();
