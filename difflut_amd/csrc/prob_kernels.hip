@@ -19,7 +19,7 @@ typedef float prob_f4 __attribute__((ext_vector_type(4)));
 // re-tiled once: xT [B/64][I][64], gyT [B/64][N*O][64], gmT [B/64][N*O*k][64], so the row of an
 // input (or a column's gradient) for a batch tile is 256 contiguous bytes, whatever the mapping.
 //   sig_table   : sig[c][a] = sigmoid(raw[n,a,d] / T), c = n*O + d                (tiny)
-//   to_tiles    : [B][C] -> [B/64][C][64], rows past B are zero                    (x, gy)
+//   to_tiles    : [B][C] -> [B/64][C][64], rows past B are zero        (x; gy only for k > 4, see bwd_t)
 //   fwd_t       : per (column, batch tile): fold the table along x_0, x_1, ... ; y leaves through
 //                 an LDS transpose as whole rows
 //   bwd_t       : one wavefront per column over a chunk of batch tiles.  The fold is run forward
