@@ -156,6 +156,16 @@ __global__ __launch_bounds__(64 * PROB_FW) void prob_fwd_t(const float *__restri
         }
     }
     __syncthreads();
+    if (cend == PROB_TC && t * 64 + 64 <= B && (NO & 3) == 0 && (((uintptr_t)y) & 15) == 0) {  // whole tile: 16-byte stores
+#pragma unroll
+        for (int pass = 0; pass < 64 * PROB_TC / 4 / (64 * PROB_FW); ++pass) {
+            const int e = pass * 64 * PROB_FW + threadIdx.x;
+            const int r = e / (PROB_TC / 4), c4 = (e % (PROB_TC / 4)) * 4;
+            const prob_f4 v = {tile[c4][r], tile[c4 + 1][r], tile[c4 + 2][r], tile[c4 + 3][r]};
+            __builtin_nontemporal_store(v, reinterpret_cast<prob_f4 *>(&y[(size_t)(t * 64 + r) * NO + c0 + c4]));
+        }
+        return;
+    }
     for (int e = threadIdx.x; e < 64 * PROB_TC; e += 64 * PROB_FW) {
         const int r = e / PROB_TC, cc = e % PROB_TC;
         const int b = t * 64 + r;
