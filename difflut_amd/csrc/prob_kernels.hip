@@ -19,7 +19,7 @@ typedef float prob_f4 __attribute__((ext_vector_type(4)));
 // re-tiled once: xT [B/64][I][64], gyT [B/64][N*O][64], gmT [B/64][N*O*k][64], so the row of an
 // input (or a column's gradient) for a batch tile is 256 contiguous bytes, whatever the mapping.
 //   sig_table   : sig[c][a] = sigmoid(raw[n,a,d] / T), c = n*O + d                (tiny)
-//   to_tiles    : [B][C] -> [B/64][C][64], rows past B are zero        (x; gy only for k > 4, see bwd_t)
+//   to_tiles    : [B][C] -> [B/64][C][64], rows past B are zero        (x; gy only for k > 5, see bwd_t)
 //   fwd_t       : per (column, batch tile): fold the table along x_0, x_1, ... ; y leaves through
 //                 an LDS transpose as whole rows
 //   bwd_t       : one wavefront per column over a chunk of batch tiles.  The fold is run forward
@@ -176,7 +176,7 @@ __global__ __launch_bounds__(64 * PROB_FW) void prob_fwd_t(const float *__restri
 // one wavefront per (column, chunk of batch tiles); W wavefronts per block.
 // HYB (hybrid node): the table is used as given and the input gradient carries the factor
 // q / (q + 1e-8), q = x_j (1 - x_j), of that node's backward.
-// W = 4: gy arrives tile-major (gyT [B/64][N*O][64], written by prob_to_tiles).  W = 16 (k <= 4, where 16 wavefronts
+// W = 4: gy arrives tile-major (gyT [B/64][N*O][64], written by prob_to_tiles).  W = 16 (k <= 5, where 16 wavefronts
 // of this kernel fit a CU's registers): gy is the row-major gradient itself; the block's 16 columns are 64 contiguous
 // bytes of a row, the 64 x 16 piece of a batch tile is fetched one value per thread a tile ahead and turned through
 // the LDS (two buffers, one barrier per tile), so the re-tiling pass and its launch are not needed.
@@ -661,13 +661,14 @@ extern "C" int dl_prob_layer_bwd(const float *x, const void *saved, const int32_
         DL_TIMED("prob_sig_table", s, (prob_sig_table<<<dl_ceil_div(WT, 256), 256, 0, s>>>(raw_w, inv_t, sig, N, L, O)));
         DL_TIMED("prob_to_tiles_x", s, (prob_to_tiles<<<dim3(dl_ceil_div(I, 64), BT), 256, 0, s>>>(x, xT, B, I)));
     }
-    if (k <= 4) {  // 16 wavefronts per block take gy as it is (see prob_bwd_t)
+    if (k <= 5) {  // 16 wavefronts per block take gy as it is (see prob_bwd_t)
 #define CALL(KK)                                                                                                       \
     DL_TIMED("prob_bwd_t", s,                                                                                          \
              (prob_bwd_t<KK, false, 16><<<dim3(dl_ceil_div(NO, 16), chunks), 1024, 0, s>>>(xT, gy, idx32, sig, gmT, gpart, I, N, \
                                                                                         O, BT, tpc, gx != nullptr, B)))
         switch (k) {
-            case 1: CALL(1); break; case 2: CALL(2); break; case 3: CALL(3); break; default: CALL(4); break;
+            case 1: CALL(1); break; case 2: CALL(2); break; case 3: CALL(3); break; case 4: CALL(4); break;
+            default: CALL(5); break;
         }
 #undef CALL
     } else {
