@@ -42,6 +42,7 @@ SIGNATURES = {
     "dl_dwn_groups_workspace_bytes": (_Z, [_I] * 4),
     "dl_dwn_layer_fwd_planes_groups": (_I, [_P, _P, _P, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _I, _F, _P]),
     "dl_dwn_layer_bwd_groups": (_I, [_P, _P, _P, _P, _P, _I, _F, _F, _F, _P, _I, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
+    "dl_dwn_layer_bwd_chain_nodes": (_I, [_P, _P, _P, _P, _P, _I, _I, _F, _P, _P, _F, _P, _I, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
     "dl_dwn_stable_layer_bwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
     "dl_table_sigmoid_fwd": (_I, [_P, _P, ctypes.c_longlong, _P]),
     "dl_table_sigmoid_bwd": (_I, [_P, _P, _P, ctypes.c_longlong, _P]),
@@ -51,6 +52,9 @@ SIGNATURES = {
     "dl_prob_bwd_workspace_bytes": (_Z, [_I] * 5),
     "dl_prob_layer_fwd": (_I, [_P, _P, _P, _F, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
     "dl_prob_layer_bwd": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
+    "dl_prob_layer_fwd_nodes": (_I, [_P, _P, _P, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
+    "dl_prob_layer_bwd_nodes": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
+    "dl_prob_layer_eval_ws_nodes": (_I, [_P, _P, _P, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
     "dl_prob_eval_workspace_bytes": (_Z, [_I] * 5),
     "dl_prob_layer_eval_ws": (_I, [_P, _P, _P, _F, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
     "dl_prob_layer_eval": (_I, [_P, _P, _P, _F, _P, _I, _I, _I, _I, _I, _P]),

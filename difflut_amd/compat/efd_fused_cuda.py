@@ -9,6 +9,13 @@ def _dims(input, mapping, luts):
     return B, I, N, k, luts.shape[1]
 
 
+def _input_key(input):
+    """Identity of the tensor the saved addresses were computed from: storage address, version counter (in-place edits
+    bump it) and shape.  A different tensor that the allocator hands the same address starts at another version or
+    shape only by luck, so the key also holds the tensor's id; any mismatch recomputes the addresses."""
+    return (input.data_ptr(), input._version, tuple(input.shape), id(input))
+
+
 def forward(input, mapping, luts):
     check_cuda_contiguous(input, mapping, luts)
     plan = plan_for(mapping, input.shape[1])
@@ -20,7 +27,7 @@ def forward(input, mapping, luts):
     ws = torch.empty(lib.dl_dwn_fwd_workspace_bytes(*dims), dtype=torch.uint8, device=input.device)
     nat.check(lib.dl_dwn_layer_fwd(input.data_ptr(), plan.idx32.data_ptr(), luts.data_ptr(), y.data_ptr(),
                                    saved.data_ptr(), ws.data_ptr(), ws.numel(), *dims, nat.stream()))
-    plan.last_saved = (input.data_ptr(), saved)  # reused by backward when it is called on the same input
+    plan.last_saved = (_input_key(input), saved)  # reused by backward when it is called on the same, unchanged input
     return y
 
 
@@ -30,7 +37,7 @@ def backward(input, mapping, luts, grad_output, alpha, beta):
     dims = _dims(input, mapping, luts)
     lib = nat.lib()
     cached = getattr(plan, "last_saved", None)
-    if cached is None or cached[0] != input.data_ptr():
+    if cached is None or cached[0] != _input_key(input):
         forward(input, mapping, luts)  # the legacy signature hands over x, not the saved addresses
         cached = plan.last_saved
     gx = torch.empty_like(input)

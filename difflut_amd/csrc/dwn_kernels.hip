@@ -834,6 +834,13 @@ static int dwn_check(int B, int I, int N, int k, int O) {
     if (k > DL_MAX_K) return DL_ERR_UNSUPPORTED;
     if (I > (1 << 28)) return DL_ERR_UNSUPPORTED;  // byte offsets into one batch tile's bit-planes are 32-bit
     if ((long long)N * O * ((long long)1 << k) > 0x7fffffffLL) return DL_ERR_UNSUPPORTED;
+    // batch tiles, padded row counts and the 1-D grids (column or input tiles x batch tiles rounded up to the 8 XCDs, plus
+    // the blocks that ride behind them) are 32-bit: refuse what would overflow them
+    if (B > 0x7fffffff - 64) return DL_ERR_UNSUPPORTED;
+    const long long bt8 = DL_XCDS * (((long long)B + 63) / 64 + DL_XCDS - 1) / DL_XCDS;
+    const long long lookup_blocks = (((long long)N * O + DWN_TC - 1) / DWN_TC) * bt8;
+    const long long gather_blocks = (((long long)I + 3) / 4) * bt8 + (((long long)N * O << k) + 1023) / 1024;
+    if (lookup_blocks > 0x7fffffffLL || gather_blocks > 0x7fffffffLL) return DL_ERR_UNSUPPORTED;
     return DL_OK;
 }
 // the fast kernels pack a node number into 23 bits of an entry record and address table rows and
@@ -1483,4 +1490,25 @@ extern "C" int dl_dwn_layer_bwd_tiled(const void *saved, const int32_t *inv_ptr,
     if (ws_bytes < dl_dwn_bwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
     return dwn_backward_fast(saved, inv_ptr, inv_pos, luts, gy, gy_tiled, alpha, beta, nullptr, gx, gx_tiled, gluts, ws, B, I, N, k, O,
                              (hipStream_t)stream);
+}
+
+// The chained backward with every node's own alpha and beta (device arrays [N]); beta_abs_max = max |beta_n| decides
+// which form of the coefficient table is safe for all nodes.  gy_form: 0 = gy row-major [B, N*O], 1 = tile-major
+// [B/64][N*O][64], 2 = the [B, groups] gradient of a GroupSum head's logits (groups, tau as in dl_dwn_layer_bwd_groups).
+extern "C" int dl_dwn_layer_bwd_chain_nodes(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos,
+                                            const float *luts, const float *gy, int gy_form, int groups, float tau,
+                                            const float *alpha_n, const float *beta_n, float beta_abs_max, float *gx,
+                                            int gx_tiled, float *gluts, void *ws, size_t ws_bytes, int B, int I, int N,
+                                            int k, int O, void *stream) {
+    if (!saved || !luts || !gy || !gluts || !ws || !alpha_n || !beta_n) return DL_ERR_NULL;
+    if (gx && (!inv_ptr || !inv_pos)) return DL_ERR_NULL;
+    if (gy_form < 0 || gy_form > 2) return DL_ERR_SHAPE;
+    int rc = dwn_check(B, I, N, k, O);
+    if (rc) return rc;
+    if (gy_form == 2 && (groups <= 0 || !(tau > 0.0f))) return DL_ERR_SHAPE;
+    if (!dwn_fast(N, k, O)) return DL_ERR_UNSUPPORTED;
+    if (ws_bytes < dl_dwn_bwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
+    const DwnGroupHead head = {groups, gy_form == 2 ? dwn_group_size(N * O, groups) : 1, gy_form == 2 ? 1.0f / tau : 1.0f};
+    return dwn_backward_fast(saved, inv_ptr, inv_pos, luts, gy, gy_form == 1, 0.0f, beta_abs_max, nullptr, gx, gx_tiled, gluts,
+                             ws, B, I, N, k, O, (hipStream_t)stream, gy_form == 2 ? &head : nullptr, alpha_n, beta_n);
 }

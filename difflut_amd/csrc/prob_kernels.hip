@@ -30,14 +30,25 @@ typedef float prob_f4 __attribute__((ext_vector_type(4)));
 //   reduce      : fixed-order sum of the chunk partials, times sigmoid'(w/T)/T
 //   gather_t    : gx[b,i] = sum over the CSR entries (n,j) of input i (and d) of gmT: a wavefront
 //                 owns 16 inputs, sums each in CSR order in a register, rows leave through LDS.
-__global__ __launch_bounds__(256) void prob_sig_table(const float *__restrict__ raw, float inv_t, float *__restrict__ sig,
+// The temperature of the layer: one value (inv = 1 / max(T, 1e-6)) or every node's own (t_n, a device array [N],
+// probabilistic_node.py:277-282 reads each node's buffer).
+struct ProbTemp {
+    float inv;
+    const float *t_n;
+};
+__device__ __forceinline__ float prob_inv_t_of(const ProbTemp &T, int n) {
+    if (!T.t_n) return T.inv;
+    const float t = T.t_n[n];
+    return 1.0f / (t > 1e-6f ? t : 1e-6f);
+}
+__global__ __launch_bounds__(256) void prob_sig_table(const float *__restrict__ raw, ProbTemp T, float *__restrict__ sig,
                                                        int N, int L, int O) {
     const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
     if (e >= (long long)N * L * O) return;
     const int a = (int)(e % L);
     const long long c = e / L;
     const int n = (int)(c / O), d = (int)(c % O);
-    sig[e] = dl_sigmoid(raw[((size_t)n * L + a) * O + d] * inv_t);
+    sig[e] = dl_sigmoid(raw[((size_t)n * L + a) * O + d] * prob_inv_t_of(T, n));
 }
 
 // grid (ceil(C / 64), B/64 rounded up), 256 threads.  With `sig` set the launch carries extra rows of blocks
@@ -45,8 +56,8 @@ __global__ __launch_bounds__(256) void prob_sig_table(const float *__restrict__ 
 // too short to fill the machine on its own.
 __global__ __launch_bounds__(256) void prob_to_tiles(const float *__restrict__ src, float *__restrict__ dst, int B, int C,
                                                       int tiles = 1 << 30, const float *__restrict__ raw = nullptr,
-                                                      float inv_t = 1.0f, float *__restrict__ sig = nullptr, int N = 0,
-                                                      int L = 1, int O = 1) {
+                                                      ProbTemp T = {1.0f, nullptr}, float *__restrict__ sig = nullptr,
+                                                      int N = 0, int L = 1, int O = 1) {
     __shared__ float tile[64][65];  // [column][row]
     if ((int)blockIdx.y >= tiles) {
         const long long e = ((long long)(blockIdx.y - tiles) * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
@@ -54,7 +65,7 @@ __global__ __launch_bounds__(256) void prob_to_tiles(const float *__restrict__ s
             const int a = (int)(e % L);
             const long long c = e / L;
             const int n = (int)(c / O), d = (int)(c % O);
-            sig[e] = dl_sigmoid(raw[((size_t)n * L + a) * O + d] * inv_t);
+            sig[e] = dl_sigmoid(raw[((size_t)n * L + a) * O + d] * prob_inv_t_of(T, n));
         }
         return;
     }
@@ -309,7 +320,7 @@ __global__ __launch_bounds__(64 * W) void prob_bwd_t(const float *__restrict__ x
 // sig == null (hybrid node): the plain sum, kept in the table's own layout [c][a]
 struct ProbReduce {  // the table-gradient reduction, also carried as extra blocks of the gather launch
     const float *gpart, *sig;
-    float inv_t;
+    ProbTemp T;
     float *graw;
     int N, L, O, chunks;
 };
@@ -319,7 +330,6 @@ __global__ __launch_bounds__(256) void prob_reduce_weights(ProbReduce R) {
 }
 __device__ __forceinline__ void prob_reduce_element(const ProbReduce &R, long long e) {
     const float *gpart = R.gpart, *sig = R.sig;
-    const float inv_t = R.inv_t;
     float *graw = R.graw;
     const int N = R.N, L = R.L, O = R.O, chunks = R.chunks;
     const long long total = (long long)N * L * O;
@@ -334,7 +344,7 @@ __device__ __forceinline__ void prob_reduce_element(const ProbReduce &R, long lo
     const long long c = e / L;
     const int n = (int)(c / O), d = (int)(c % O);
     const float s = sig[e];
-    graw[((size_t)n * L + a) * O + d] = acc * s * (1.0f - s) * inv_t;
+    graw[((size_t)n * L + a) * O + d] = acc * s * (1.0f - s) * prob_inv_t_of(R.T, n);
 }
 
 #define PROB_IS 64  // inputs per block of the gather
@@ -476,13 +486,14 @@ static void prob_launch_gather_and_reduce(const float *gmT, const int *inv_ptr, 
 // ---------------------------------------------------------------------------------
 // Generic kernels, any k up to DL_MAX_K.
 __global__ __launch_bounds__(256) void prob_generic_fwd(const float *__restrict__ x, const int *__restrict__ idx32,
-                                                         const float *__restrict__ raw, float inv_t, float *__restrict__ y,
+                                                         const float *__restrict__ raw, ProbTemp T, float *__restrict__ y,
                                                          int B, int I, int N, int K, int O) {
     const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
     const long long NO = (long long)N * O;
     if (gid >= (long long)B * NO) return;
     const int b = (int)(gid / NO);
     const int n = (int)((gid % NO) / O), d = (int)((gid % NO) % O);
+    const float inv_t = prob_inv_t_of(T, n);
     float xs[DL_MAX_K];
     for (int j = 0; j < K; ++j) xs[j] = x[(size_t)b * I + idx32[(size_t)n * K + j]];
     const int L = 1 << K;
@@ -497,13 +508,14 @@ __global__ __launch_bounds__(256) void prob_generic_fwd(const float *__restrict_
 
 // hybrid: `raw` is the table itself in the layout [n][d][a] and the input gradient carries q / (q + 1e-8)
 __global__ __launch_bounds__(256) void prob_generic_bwd(const float *__restrict__ x, const int *__restrict__ idx32,
-                                                         const float *__restrict__ raw, float inv_t,
+                                                         const float *__restrict__ raw, ProbTemp T,
                                                          const float *__restrict__ gy, float *__restrict__ gx,
                                                          float *__restrict__ graw, int B, int I, int N, int K, int O,
                                                          int hybrid) {
     const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
     if (gid >= (long long)B * N) return;
     const int b = (int)(gid / N), n = (int)(gid % N);
+    const float inv_t = prob_inv_t_of(T, n);
     float xs[DL_MAX_K], gxs[DL_MAX_K];
     for (int j = 0; j < K; ++j) { xs[j] = x[(size_t)b * I + idx32[(size_t)n * K + j]]; gxs[j] = 0.0f; }
     const int L = 1 << K;
@@ -533,13 +545,14 @@ __global__ __launch_bounds__(256) void prob_generic_bwd(const float *__restrict_
 }
 
 __global__ __launch_bounds__(256) void prob_eval_kernel(const float *__restrict__ x, const int *__restrict__ idx32,
-                                                         const float *__restrict__ raw, float inv_t, float *__restrict__ y,
+                                                         const float *__restrict__ raw, ProbTemp T, float *__restrict__ y,
                                                          int B, int I, int N, int K, int O) {
     const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
     const long long NO = (long long)N * O;
     if (gid >= (long long)B * NO) return;
     const int b = (int)(gid / NO);
     const int n = (int)((gid % NO) / O), d = (int)((gid % NO) % O);
+    const float inv_t = prob_inv_t_of(T, n);
     float s = 0.0f;
     for (int j = 0; j < K; ++j) s += x[(size_t)b * I + idx32[(size_t)n * K + j]] * (float)(1 << j);
     long long a = (long long)s;
@@ -564,7 +577,8 @@ static int prob_check(int B, int I, int N, int k, int O) {
 static inline bool prob_fast(int I, int N, int k, int O) {
     return k <= DL_MAX_FAST_K && I < (1 << 23) && (long long)N * O * k < (1 << 23);
 }
-static inline float prob_inv_t(float t) { return 1.0f / (t > 1e-6f ? t : 1e-6f); }  // temperature.clamp(min=1e-6)
+// temperature.clamp(min=1e-6); with a per-node array the kernels take every node's own value
+static inline ProbTemp prob_temp(float t, const float *t_n) { return ProbTemp{1.0f / (t > 1e-6f ? t : 1e-6f), t_n}; }
 static inline int prob_bt(int B) { return (B + 63) / 64; }
 // batch tiles per wavefront of prob_bwd_t: enough (column, chunk) wavefronts to fill the chip
 static inline int prob_tiles_per_chunk(int B, int N, int O) {
@@ -596,13 +610,12 @@ extern "C" size_t dl_prob_bwd_workspace_bytes(int B, int I, int N, int k, int O)
         case 4: CALL(4); break; case 5: CALL(5); break; default: CALL(6); break; \
     }
 
-extern "C" int dl_prob_layer_fwd(const float *x, const int32_t *idx32, const float *raw_w, float temperature, float *y,
-                                 void *saved, size_t saved_bytes, int B, int I, int N, int k, int O, void *stream) {
+static int prob_forward(const float *x, const int32_t *idx32, const float *raw_w, ProbTemp inv_t, float *y, void *saved,
+                        size_t saved_bytes, int B, int I, int N, int k, int O, void *stream) {
     if (!x || !idx32 || !raw_w || !y) return DL_ERR_NULL;
     int rc = prob_check(B, I, N, k, O);
     if (rc) return rc;
     hipStream_t s = (hipStream_t)stream;
-    const float inv_t = prob_inv_t(temperature);
     if (!prob_fast(I, N, k, O)) {
         DL_TIMED("prob_generic_fwd", s, (prob_generic_fwd<<<dl_ceil_div((long long)B * N * O, 256), 256, 0, s>>>(x, idx32, raw_w, inv_t, y, B, I, N, k, O)));
         return dl_launch_status();
@@ -625,16 +638,25 @@ extern "C" int dl_prob_layer_fwd(const float *x, const int32_t *idx32, const flo
     return dl_launch_status();
 }
 
-extern "C" int dl_prob_layer_bwd(const float *x, const void *saved, const int32_t *idx32, const int32_t *inv_ptr,
-                                 const int32_t *inv_pos,
-                                 const float *raw_w, float temperature, const float *gy, float *gx, float *graw,
-                                 void *ws, size_t ws_bytes, int B, int I, int N, int k, int O, void *stream) {
+extern "C" int dl_prob_layer_fwd(const float *x, const int32_t *idx32, const float *raw_w, float temperature, float *y,
+                                 void *saved, size_t saved_bytes, int B, int I, int N, int k, int O, void *stream) {
+    return prob_forward(x, idx32, raw_w, prob_temp(temperature, nullptr), y, saved, saved_bytes, B, I, N, k, O, stream);
+}
+extern "C" int dl_prob_layer_fwd_nodes(const float *x, const int32_t *idx32, const float *raw_w, const float *temperature_n,
+                                       float *y, void *saved, size_t saved_bytes, int B, int I, int N, int k, int O,
+                                       void *stream) {
+    if (!temperature_n) return DL_ERR_NULL;
+    return prob_forward(x, idx32, raw_w, prob_temp(1.0f, temperature_n), y, saved, saved_bytes, B, I, N, k, O, stream);
+}
+
+static int prob_backward(const float *x, const void *saved, const int32_t *idx32, const int32_t *inv_ptr,
+                         const int32_t *inv_pos, const float *raw_w, ProbTemp inv_t, const float *gy, float *gx, float *graw,
+                         void *ws, size_t ws_bytes, int B, int I, int N, int k, int O, void *stream) {
     if (!x || !idx32 || !raw_w || !gy || !graw) return DL_ERR_NULL;
     if (gx && (!inv_ptr || !inv_pos)) return DL_ERR_NULL;
     int rc = prob_check(B, I, N, k, O);
     if (rc) return rc;
     hipStream_t s = (hipStream_t)stream;
-    const float inv_t = prob_inv_t(temperature);
     const long long WT = (long long)N * ((long long)1 << k) * O;
     if (!prob_fast(I, N, k, O)) {
         DL_TIMED("prob_fill_zero", s, (prob_fill_zero<<<dl_ceil_div(WT, 256), 256, 0, s>>>(graw, WT)));
@@ -685,6 +707,22 @@ extern "C" int dl_prob_layer_bwd(const float *x, const void *saved, const int32_
     return dl_launch_status();
 }
 
+extern "C" int dl_prob_layer_bwd(const float *x, const void *saved, const int32_t *idx32, const int32_t *inv_ptr,
+                                 const int32_t *inv_pos,
+                                 const float *raw_w, float temperature, const float *gy, float *gx, float *graw,
+                                 void *ws, size_t ws_bytes, int B, int I, int N, int k, int O, void *stream) {
+    return prob_backward(x, saved, idx32, inv_ptr, inv_pos, raw_w, prob_temp(temperature, nullptr), gy, gx, graw, ws, ws_bytes,
+                         B, I, N, k, O, stream);
+}
+extern "C" int dl_prob_layer_bwd_nodes(const float *x, const void *saved, const int32_t *idx32, const int32_t *inv_ptr,
+                                       const int32_t *inv_pos, const float *raw_w, const float *temperature_n,
+                                       const float *gy, float *gx, float *graw, void *ws, size_t ws_bytes, int B, int I,
+                                       int N, int k, int O, void *stream) {
+    if (!temperature_n) return DL_ERR_NULL;
+    return prob_backward(x, saved, idx32, inv_ptr, inv_pos, raw_w, prob_temp(1.0f, temperature_n), gy, gx, graw, ws, ws_bytes,
+                         B, I, N, k, O, stream);
+}
+
 // Hybrid nodes: the forward is the DWN lookup; the backward is the probabilistic one on the table as given.
 extern "C" size_t dl_hybrid_bwd_workspace_bytes(int B, int I, int N, int k, int O) {
     if (B <= 0 || I <= 0 || N <= 0 || k <= 0 || O <= 0 || !prob_fast(I, N, k, O)) return 256;
@@ -704,7 +742,7 @@ extern "C" int dl_hybrid_layer_bwd(const float *x, const int32_t *idx32, const i
         DL_TIMED("prob_fill_zero", s, (prob_fill_zero<<<dl_ceil_div(WT, 256), 256, 0, s>>>(gluts, WT)));
         if (gx) prob_fill_zero<<<dl_ceil_div((long long)B * I, 256), 256, 0, s>>>(gx, (long long)B * I);
         DL_TIMED("prob_generic_bwd", s, (prob_generic_bwd<<<dl_ceil_div((long long)B * N, 256), 256, 0, s>>>(
-                                            x, idx32, luts, 1.0f, gy, gx, gluts, B, I, N, k, O, 1)));
+                                            x, idx32, luts, ProbTemp{1.0f, nullptr}, gy, gx, gluts, B, I, N, k, O, 1)));
         return dl_launch_status();
     }
     if (!ws) return DL_ERR_NULL;
@@ -725,7 +763,7 @@ extern "C" int dl_hybrid_layer_bwd(const float *x, const int32_t *idx32, const i
                                                                                  BT, tpc, gx != nullptr)))
     PROB_DISPATCH(k, CALL)
 #undef CALL
-    const ProbReduce R = {gpart, nullptr, 1.0f, gluts, N, L, O, chunks};
+    const ProbReduce R = {gpart, nullptr, ProbTemp{1.0f, nullptr}, gluts, N, L, O, chunks};
     prob_launch_gather_and_reduce(gmT, inv_ptr, inv_pos, gx, B, I, N, k, O, BT, R, WT, s);
     return dl_launch_status();
 }
@@ -740,15 +778,15 @@ extern "C" size_t dl_prob_eval_workspace_bytes(int B, int I, int N, int k, int O
     if (B <= 0 || I <= 0 || N <= 0 || k <= 0 || O <= 0 || k > DL_MAX_FAST_K) return 256;
     return prob_eval_table_bytes(N, k, O) + dl_dwn_eval_workspace_bytes(B, I, N, k, O);
 }
-extern "C" int dl_prob_layer_eval_ws(const float *x, const int32_t *idx32, const float *raw_w, float temperature, float *y,
-                                     void *ws, size_t ws_bytes, int B, int I, int N, int k, int O, void *stream) {
+static int prob_eval_ws(const float *x, const int32_t *idx32, const float *raw_w, ProbTemp T, float *y, void *ws,
+                        size_t ws_bytes, int B, int I, int N, int k, int O, void *stream) {
     if (!x || !idx32 || !raw_w || !y) return DL_ERR_NULL;
     int rc = prob_check(B, I, N, k, O);
     if (rc) return rc;
     hipStream_t s = (hipStream_t)stream;
     if (k > DL_MAX_FAST_K) {
         DL_TIMED("prob_eval_kernel", s, (prob_eval_kernel<<<dl_ceil_div((long long)B * N * O, 256), 256, 0, s>>>(
-                                            x, idx32, raw_w, prob_inv_t(temperature), y, B, I, N, k, O)));
+                                            x, idx32, raw_w, T, y, B, I, N, k, O)));
         return dl_launch_status();
     }
     if (!ws) return DL_ERR_NULL;
@@ -756,9 +794,19 @@ extern "C" int dl_prob_layer_eval_ws(const float *x, const int32_t *idx32, const
     float *sig = (float *)ws;
     const int L = 1 << k;
     DL_TIMED("prob_sig_table", s, (prob_sig_table<<<dl_ceil_div((long long)N * L * O, 256), 256, 0, s>>>(
-                                      raw_w, prob_inv_t(temperature), sig, N, L, O)));
+                                      raw_w, T, sig, N, L, O)));
     const size_t tb = prob_eval_table_bytes(N, k, O);
     return dl_dwn_layer_eval_ws(x, idx32, sig, y, (char *)ws + tb, ws_bytes - tb, B, I, N, k, O, stream);
+}
+extern "C" int dl_prob_layer_eval_ws(const float *x, const int32_t *idx32, const float *raw_w, float temperature, float *y,
+                                     void *ws, size_t ws_bytes, int B, int I, int N, int k, int O, void *stream) {
+    return prob_eval_ws(x, idx32, raw_w, prob_temp(temperature, nullptr), y, ws, ws_bytes, B, I, N, k, O, stream);
+}
+extern "C" int dl_prob_layer_eval_ws_nodes(const float *x, const int32_t *idx32, const float *raw_w,
+                                           const float *temperature_n, float *y, void *ws, size_t ws_bytes, int B, int I,
+                                           int N, int k, int O, void *stream) {
+    if (!temperature_n) return DL_ERR_NULL;
+    return prob_eval_ws(x, idx32, raw_w, prob_temp(1.0f, temperature_n), y, ws, ws_bytes, B, I, N, k, O, stream);
 }
 
 extern "C" int dl_prob_layer_eval(const float *x, const int32_t *idx32, const float *raw_w, float temperature, float *y,
@@ -767,6 +815,6 @@ extern "C" int dl_prob_layer_eval(const float *x, const int32_t *idx32, const fl
     int rc = prob_check(B, I, N, k, O);
     if (rc) return rc;
     DL_TIMED("prob_eval_kernel", (hipStream_t)stream, (prob_eval_kernel<<<dl_ceil_div((long long)B * N * O, 256), 256, 0, (hipStream_t)stream>>>(
-        x, idx32, raw_w, prob_inv_t(temperature), y, B, I, N, k, O)));
+        x, idx32, raw_w, prob_temp(temperature, nullptr), y, B, I, N, k, O)));
     return dl_launch_status();
 }

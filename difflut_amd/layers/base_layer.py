@@ -18,8 +18,8 @@ users, optimisers and state_dict see (`nodes.{i}.luts`, ...) are views into that
     a copy or a load keeps working).
 The per-node scalar buffers the fused kernels need (`alpha`, `beta`, `temperature`) are banked the same way
 (`ScalarBank`: one [N] tensor, each node's 0-dim buffer a view of it), so a state dict or an in-place edit that
-gives nodes different values is seen by the layer: DWN layers then hand the kernels the per-node arrays, the
-other fused paths refuse to run rather than use one node's value for all.
+gives nodes different values lands in the array the kernels are handed on every call: every fused path (single
+layers, chained stacks, convolutional levels) uses each node's own values, as the reference's node loop does.
 """
 import warnings
 from abc import ABC, abstractmethod
@@ -114,12 +114,17 @@ class ParameterBank:
 
 class ScalarBank:
     """The 0-dim buffer `name` of N nodes as one tensor [N]; each node's buffer is a view of its entry, so
-    `load_state_dict` and in-place edits land in the bank.  `summary()` is the host's view of it, read back
-    only when the bank's version changes: (all entries equal, first value, largest magnitude)."""
+    `load_state_dict` and in-place edits land in the bank and the kernels, which are handed the whole array on
+    every call, always see every node's current value.  The views keep the buffers' own dtype (`layer.double()`
+    leaves double buffers); `tensor()` is the float32 array the kernels read.  The only host-side knowledge is
+    `abs_max()` (the largest magnitude, which selects the form of the EFD coefficient table): read back when the
+    bank's version counter changes or after `invalidate()`."""
+
+    _PROBES = 16  # nodes checked per call beyond the first and the last when the layer is large
 
     def __init__(self, nodes, name):
         self.nodes, self.name = nodes, name
-        self.flat, self._stale, self._key, self._summary = None, False, None, None
+        self.flat, self._stale, self._key, self._abs_max, self._views, self._probe = None, False, None, None, [], 0
         self.tie()
 
     def tie(self):
@@ -128,34 +133,49 @@ class ScalarBank:
             other = getattr(b, "_scalar_bank", None)
             if other is not None and other is not self:
                 other._stale = True
-        self.flat = torch.stack([b.detach().reshape(()).to(torch.float32) for b in bufs]).contiguous()
+        self.flat = torch.stack([b.detach().reshape(()) for b in bufs]).contiguous()
+        self._views = []
         for row, node in enumerate(self.nodes):
             view = self.flat[row]
             view._scalar_bank = self
             node._buffers[self.name] = view
+            self._views.append(view)
         self._stale, self._key = False, None
 
+    def _is_view(self, row):
+        return self.nodes[row]._buffers[self.name] is self._views[row]
+
     def tied(self):
-        if self._stale:
+        """Every node's buffer is still the view handed out by tie().  All nodes are checked on small layers; on large
+        ones the first, the last and a window of nodes that moves on with every call (assignments through
+        `node.<name> = ...` set the stale flag themselves)."""
+        if self._stale or not self._views or self._views[0].device != self.flat.device:
             return False
-        first, last = self.nodes[0]._buffers[self.name], self.nodes[-1]._buffers[self.name]
-        base, step = self.flat.data_ptr(), self.flat.element_size()
-        return (first.device == self.flat.device and first.data_ptr() == base
-                and last.data_ptr() == base + step * (len(self.nodes) - 1))
+        n = len(self.nodes)
+        if n <= 4 * self._PROBES:
+            return all(self._is_view(row) for row in range(n))
+        rows = [0, n - 1] + [(self._probe + i) % n for i in range(self._PROBES)]
+        self._probe = (self._probe + self._PROBES) % n
+        return all(self._is_view(row) for row in rows)
 
     def tensor(self):
+        """The float32 device array [N] for the kernels (the bank itself when it is float32)."""
         if not self.tied():
             self.tie()
-        return self.flat
+        return self.flat if self.flat.dtype == torch.float32 else self.flat.float()
 
-    def summary(self):
+    def invalidate(self):
+        """Forget the host-side summary: needed after a write that bypasses the version counter (`buffer.data.fill_`,
+        an external kernel)."""
+        self._key = None
+
+    def abs_max(self):
         flat = self.tensor()
-        key = (flat._version, flat.data_ptr())
+        key = (self.flat._version, self.flat.data_ptr())
         if key != self._key:
-            host = flat.detach().cpu()
-            self._summary = (bool((host == host[0]).all()), float(host[0]), float(host.abs().max()))
+            self._abs_max = float(flat.detach().abs().max())
             self._key = key
-        return self._summary
+        return self._abs_max
 
 
 class LUTLayerMixin(nn.Module):
@@ -296,22 +316,22 @@ class BaseLUTLayer(ABC, LUTLayerMixin, nn.Module):
             bank.tie()
 
     def efd_scalars(self):
-        """(alpha, beta) of a DWN layer whose nodes all share them, as Python floats.  The paths that take one pair for
-        the whole layer (chained layers, convolutional levels) call this and refuse per-node values."""
-        (a_same, alpha, _), (b_same, beta, _) = self._scalars["alpha"].summary(), self._scalars["beta"].summary()
-        if not (a_same and b_same):
-            raise RuntimeError("the nodes of this layer carry different alpha / beta values; chained and convolutional "
-                               "execution takes one pair per layer - call the layer on its own (RandomLayer.forward "
-                               "passes every node's pair to the kernels)")
-        return alpha, beta
+        """(alpha [N], beta [N], max |beta|) of a DWN layer for the kernels: the nodes' own values as float32 device
+        arrays (every call reads the nodes' current values, dwn_node.py:450) and the host value that selects the form
+        of the coefficient table."""
+        return self._scalars["alpha"].tensor(), self._scalars["beta"].tensor(), self._scalars["beta"].abs_max()
 
-    def temperature_value(self):
-        """The temperature shared by the nodes of a probabilistic layer; per-node temperatures are refused."""
-        same, value, _ = self._scalars["temperature"].summary()
-        if not same:
-            raise RuntimeError("the nodes of this layer carry different temperatures; the fused probabilistic kernels "
-                               "take one temperature per layer")
-        return value
+    def temperatures(self):
+        """The nodes' temperatures [N] as a float32 device array (probabilistic_node.py:277-282 reads each node's)."""
+        return self._scalars["temperature"].tensor()
+
+    def invalidate_scalars(self):
+        """Call after writing a node's `alpha` / `beta` / `temperature` in a way autograd's version counter does not
+        see (`node.beta.data.fill_(...)`, an external kernel).  The kernels read the values themselves on every call;
+        what this refreshes is the host's max |beta|, which decides between the two forms of the EFD coefficient
+        table (the compact one divides by 1 - beta and is only used while every |beta| <= 1/2)."""
+        for bank in self._scalars.values():
+            bank.invalidate()
 
     def bank_parameters(self):
         """The layer's trainable tensors with every node parameter as ONE leaf [N, ...] (the storage the
@@ -333,32 +353,26 @@ class BaseLUTLayer(ABC, LUTLayerMixin, nn.Module):
 
             luts = self._banks["luts"].tensor()
             if self.training:
-                (a_same, alpha, _), (b_same, beta, b_max) = (self._scalars["alpha"].summary(),
-                                                             self._scalars["beta"].summary())
-                if a_same and b_same:
-                    return ops.DWNLayerFunction.apply(x, luts, plan, alpha, beta)
-                # every node's own pair (dwn_node.py:450 reads them per node)
-                return ops.DWNLayerFunction.apply(x, luts, plan, self._scalars["alpha"].tensor(),
-                                                  self._scalars["beta"].tensor(), b_max)
+                return ops.dwn_layer(x, luts, plan, *self.efd_scalars())
             return ops.dwn_layer_eval(x, luts.detach(), plan)
         if self._fused == "probabilistic":
             from .. import ops
 
             raw = self._banks["raw_weights"].tensor()
             if self.training:
-                return ops.ProbLayerFunction.apply(x, raw, plan, self.temperature_value())
-            return ops.prob_layer_eval(x, raw.detach(), plan, self.temperature_value())
+                return ops.prob_layer(x, raw, plan, self.temperatures())
+            return ops.prob_layer_eval(x, raw.detach(), plan, self.temperatures())
         if self._fused in ("dwn_stable", "hybrid"):
             from .. import ops
 
             raw = self._banks["raw_luts"].tensor()
             if not self.training:
                 with torch.no_grad():
-                    return ops.dwn_layer_eval(x, ops.TableSigmoidFunction.apply(raw), plan)
-            luts = ops.TableSigmoidFunction.apply(raw)
+                    return ops.dwn_layer_eval(x, ops.table_sigmoid(raw), plan)
+            luts = ops.table_sigmoid(raw)
             if self._fused == "hybrid":
-                return ops.HybridLayerFunction.apply(x, luts, plan)
-            return ops.DWNStableLayerFunction.apply(x, luts, self._banks["gradient_scale"].tensor().detach(), plan)
+                return ops.hybrid_layer(x, luts, plan)
+            return ops.dwn_stable_layer(x, luts, self._banks["gradient_scale"].tensor().detach(), plan)
         return None
 
     def _loop_nodes(self, mapped):

@@ -17,12 +17,14 @@ import torch.nn as nn
 from .. import _native, ops
 from ..nodes.node_config import NodeConfig
 from ..registry import register_convolutional_layer
-from .base_layer import LUTLayerMixin, ParameterBank
+from .base_layer import LUTLayerMixin, ParameterBank, ScalarBank
 from .layer_config import GroupedInputConfig
 from .random_layer import RandomLayer
 
 _BANKED = {"dwn": ("luts",), "probabilistic": ("raw_weights",), "dwn_stable": ("raw_luts", "gradient_scale"),
            "hybrid": ("raw_luts",)}
+# the per-node scalar buffers the kernels read, banked per depth level like the parameters
+_BANKED_SCALARS = {"dwn": ("alpha", "beta"), "probabilistic": ("temperature",), "dwn_stable": (), "hybrid": ()}
 
 
 class ConvolutionConfig:
@@ -87,7 +89,7 @@ class ConvolutionalLayer(LUTLayerMixin, nn.Module):
             self.trees.append(tree)
         self.unfold = nn.Unfold(kernel_size=self.receptive_field, padding=self.padding, stride=self.stride)
         self._kind = self._detect_kind()
-        self._level_banks, self._plans, self._plan_key = [], None, None
+        self._level_banks, self._level_scalar_banks, self._plans, self._plan_key = [], [], None, None
         if self._kind is not None:
             self._tie_levels()
 
@@ -112,10 +114,11 @@ class ConvolutionalLayer(LUTLayerMixin, nn.Module):
         return list(self.first_layer_chunks) if level == 0 else [tree[level - 1] for tree in self.trees]
 
     def _tie_levels(self):
-        self._level_banks = []
+        self._level_banks, self._level_scalar_banks = [], []
         for level in range(self.tree_depth + 1):
             nodes = [node for layer in self._level_layers(level) for node in layer.nodes]
             self._level_banks.append({name: ParameterBank(nodes, name) for name in _BANKED[self._kind]})
+            self._level_scalar_banks.append({name: ScalarBank(nodes, name) for name in _BANKED_SCALARS[self._kind]})
 
     def _apply(self, fn, *args, **kwargs):
         grads = [{name: bank.flat.grad for name, bank in banks.items()} for banks in self._level_banks]
@@ -126,24 +129,33 @@ class ConvolutionalLayer(LUTLayerMixin, nn.Module):
         for banks, kept in zip(self._level_banks, grads):
             for name, bank in banks.items():
                 bank.tie(keep_grad=None if kept[name] is None else fn(kept[name]))
+        for banks in self._level_scalar_banks:
+            for bank in banks.values():
+                bank.tie()
         self._plans = None
         return self
 
     def __setstate__(self, state):
         # after copy.deepcopy / unpickling the per-node Parameters are plain again: tie them to the level banks now
         super().__setstate__(state)
+        self.__dict__.setdefault("_level_scalar_banks", [])
         if self._kind is not None:
             self._tie_levels()
         self._plans = None
 
-    def _level_scalars(self, level, what):
-        """The value all sub-layers of a depth level share (`efd_scalars` or `temperature_value`): a level runs as one
-        layer call with one value, so differing nodes are refused rather than overridden."""
-        values = {getattr(layer, what)() for layer in self._level_layers(level)}
-        if len(values) != 1:
-            raise RuntimeError(f"the sub-layers of depth level {level} carry different {what.split('_')[0]} values; a level "
-                               "runs as one fused layer call and takes one value")
-        return values.pop()
+    def _level_scalars(self, level):
+        """What the kernels take for a depth level, every node's own values (a level runs as one fused layer call over
+        the nodes of all its sub-layers): DWN (alpha [nodes], beta [nodes], max |beta|), probabilistic temperature [nodes]."""
+        banks = self._level_scalar_banks[level]
+        if self._kind == "dwn":
+            return banks["alpha"].tensor(), banks["beta"].tensor(), banks["beta"].abs_max()
+        return banks["temperature"].tensor()
+
+    def invalidate_scalars(self):
+        """After a write to a node's alpha / beta / temperature that bypasses the version counter (`.data` edits)."""
+        for banks in self._level_scalar_banks:
+            for bank in banks.values():
+                bank.invalidate()
 
     def bank_parameters(self):
         """One leaf [nodes of the level, ...] per depth level and node parameter (what the fused calls
@@ -184,31 +196,31 @@ class ConvolutionalLayer(LUTLayerMixin, nn.Module):
         levels = range(self.tree_depth + 1)
         kind, h = self._kind, patches
         if image is not None:
-            scalars = [self._level_scalars(level, "efd_scalars") for level in levels]
+            scalars = [self._level_scalars(level) for level in levels]
             source = self._geometry() if flip is None else (*self._geometry(), flip)
             return ops.DWNStackFunction.apply(image, source, plans, scalars, None, *[b["luts"] for b in banks])
-        if kind == "dwn" and self.training and self.n_inputs_per_node <= ops.FAST_K:
-            scalars = [self._level_scalars(level, "efd_scalars") for level in levels]
+        if kind == "dwn" and self.training and self.n_inputs_per_node <= ops.FAST_K and h.is_cuda:
+            scalars = [self._level_scalars(level) for level in levels]
             return ops.DWNStackFunction.apply(h, None, plans, scalars, None, *[b["luts"] for b in banks])
         for level, plan, bank in zip(levels, plans, banks):
             if kind == "dwn":
                 if self.training:
-                    h = ops.DWNLayerFunction.apply(h, bank["luts"], plan, *self._level_scalars(level, "efd_scalars"))
+                    h = ops.dwn_layer(h, bank["luts"], plan, *self._level_scalars(level))
                 else:
                     h = ops.dwn_layer_eval(h, bank["luts"].detach(), plan)
             elif kind == "probabilistic":
-                temperature = self._level_scalars(level, "temperature_value")
+                temperature = self._level_scalars(level)
                 if self.training:
-                    h = ops.ProbLayerFunction.apply(h, bank["raw_weights"], plan, temperature)
+                    h = ops.prob_layer(h, bank["raw_weights"], plan, temperature)
                 else:
                     h = ops.prob_layer_eval(h, bank["raw_weights"].detach(), plan, temperature)
             elif not self.training:
                 with torch.no_grad():
-                    h = ops.dwn_layer_eval(h, ops.TableSigmoidFunction.apply(bank["raw_luts"]), plan)
+                    h = ops.dwn_layer_eval(h, ops.table_sigmoid(bank["raw_luts"]), plan)
             elif kind == "hybrid":
-                h = ops.HybridLayerFunction.apply(h, ops.TableSigmoidFunction.apply(bank["raw_luts"]), plan)
+                h = ops.hybrid_layer(h, ops.table_sigmoid(bank["raw_luts"]), plan)
             else:
-                h = ops.DWNStableLayerFunction.apply(h, ops.TableSigmoidFunction.apply(bank["raw_luts"]),
+                h = ops.dwn_stable_layer(h, ops.table_sigmoid(bank["raw_luts"]),
                                                      bank["gradient_scale"].detach(), plan)
         return h
 
@@ -230,7 +242,6 @@ class ConvolutionalLayer(LUTLayerMixin, nn.Module):
 
     # ------------------------------------------------------------------ interface
     def forward(self, x):
-        _native.require_device(x)
         if x.dim() != 4 or x.shape[1] != self.in_channels:
             raise ValueError(f"ConvolutionalLayer expects (batch, {self.in_channels}, height, width), got {tuple(x.shape)}")
         batch = x.shape[0]
@@ -240,10 +251,10 @@ class ConvolutionalLayer(LUTLayerMixin, nn.Module):
         # bit-flip augmentation of the patch matrix (convolutional.py:205-207): the mask is drawn here, the patch
         # extraction applies it on the way (also when the patches only ever exist as bit-planes)
         flip = self._flip_mask((batch * positions, self.input_size), x.device)
-        if self._kind is not None and self._chained():
+        if self._kind is not None and self._chained() and x.is_cuda:
             out = self._run_levels(None, image=x, flip=flip)
         else:
-            patches = ops.UnfoldFunction.apply(x, self._geometry(), flip)  # (batch * positions, channels * kh * kw)
+            patches = ops.unfold(x, self._geometry(), flip)  # (batch * positions, channels * kh * kw)
             out = self._run_levels(patches) if self._kind is not None else self._loop_trees(patches)
         out = out.view(batch, positions, self.out_channels).transpose(1, 2)
         out = out.reshape(batch, self.out_channels, out_h, out_w)

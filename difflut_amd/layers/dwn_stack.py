@@ -72,7 +72,7 @@ class DWNStack(nn.Module):
                 with torch.no_grad():
                     y = ops.dwn_stack_eval(x, thresholds, plans, luts, (self.head.k, self.head.tau) if fused_head else None)
                     return y if self.head is None or fused_head else self.head(y)
-        if not (self.training and self._chainable()):
+        if not (self.training and self._chainable() and torch.is_tensor(x) and x.is_cuda):
             if self.encoder is not None:
                 x = self.encoder.encode(x)
             for layer in self.layers:
@@ -89,7 +89,7 @@ class DWNStack(nn.Module):
         if thresholds is None:
             self.layers[0]._validate_input_dims(x)
         plans = [layer.mapping_plan() for layer in self.layers]
-        scalars = [layer.efd_scalars() for layer in self.layers]  # raises when a layer's nodes disagree
+        scalars = [layer.efd_scalars() for layer in self.layers]  # every node's own alpha and beta
         luts = [layer._banks["luts"].tensor() for layer in self.layers]
         if self.head is not None and self._fusable_head():
             return ops.DWNStackFunction.apply(x, thresholds, plans, scalars, (self.head.k, self.head.tau), *luts)

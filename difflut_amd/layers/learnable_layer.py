@@ -56,14 +56,13 @@ class LearnableMappingModule(nn.Module):
             self._hard_plan = ops.MappingPlan(self._cached_hard_indices.view(-1, 1), self.input_size)
 
     def forward(self, x):
-        _native.require_device(x, self.W)
         if self.training:
-            return ops.SoftMapFunction.apply(x, self.W, self.tau, self.precision)
+            return ops.soft_map(x, self.W, self.tau, self.precision)
         if (not self._cache_valid or self._cached_hard_indices is None or self._hard_plan is None
                 or self._hard_plan.device != x.device):
             self._compute_hard_selection()
             self._cache_valid = True
-        return ops.HardSelectFunction.apply(x, self._cached_hard_indices, self._hard_plan)
+        return ops.hard_select(x, self._cached_hard_indices, self._hard_plan)
 
 
 @register_layer("learnable")

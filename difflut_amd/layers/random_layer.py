@@ -4,7 +4,8 @@ Constructor, buffer name (`_mapping_indices`, int16 below 32768 inputs else int3
 rule and `get_mapping`/`get_mapping_matrix` follow difflut/layers/random_layer.py:123-356.
 forward() differs in how it gets there: for DWN / Probabilistic nodes the gather, all N nodes
 and (in backward) the scatter run as one fused device call and the [batch, N, n] tensor is
-never written; other node types take the gather kernel plus a per-node loop.
+never written; other node types take the gather kernel plus a per-node loop.  CPU tensors take
+the plain-torch branch of the same operators (the reference's rule: the extension iff `x.is_cuda`).
 """
 import torch
 
@@ -70,15 +71,13 @@ class RandomLayer(BaseLUTLayer):
         return self._plan
 
     def get_mapping(self, x):
-        _native.require_device(x)
-        return ops.GatherFunction.apply(x, self._mapping_indices, self.mapping_plan())
+        return ops.gather(x, self._mapping_indices, self.mapping_plan())
 
     def get_mapping_indices(self):
         return self._mapping_indices.long()
 
     def forward(self, x):
         self._validate_input_dims(x)
-        _native.require_device(x)
         out = self._run_nodes(x, self.mapping_plan())
         if out is None:
             out = self._loop_nodes(self.get_mapping(x))

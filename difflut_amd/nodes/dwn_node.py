@@ -41,7 +41,7 @@ def efd_forward(input, luts, alpha, beta):
     """(batch, k) inputs and (output_dim, 2^k) table -> (batch, output_dim); autograd-aware
     (dwn_node.py:319-338)."""
     plan = _identity_plan(input.shape[1], input.device)
-    return ops.DWNLayerFunction.apply(input, luts.unsqueeze(0), plan, alpha, beta)
+    return ops.dwn_layer(input, luts.unsqueeze(0), plan, alpha, beta)
 
 
 @register_node("dwn")
@@ -95,7 +95,7 @@ class DWNNode(BaseNode):
         luts = self.luts.unsqueeze(0).expand(layer_size, -1, -1)
         if self.training:
             alpha, beta = self.efd_scalars()
-            out = ops.DWNLayerFunction.apply(x, luts, plan, alpha, beta)
+            out = ops.dwn_layer(x, luts, plan, alpha, beta)
         else:
             out = ops.dwn_layer_eval(x, luts.detach(), plan)
         return out.view(x.shape[0], layer_size, self.num_outputs)

@@ -27,7 +27,7 @@ def dwn_stable_forward(input, luts, gradient_scale):
     if not torch.is_tensor(gradient_scale):
         gradient_scale = torch.full((1,), float(gradient_scale), device=input.device)
     plan = _identity_plan(input.shape[1], input.device)
-    return ops.DWNStableLayerFunction.apply(input, luts.unsqueeze(0), gradient_scale.reshape(1), plan)
+    return ops.dwn_stable_layer(input, luts.unsqueeze(0), gradient_scale.reshape(1), plan)
 
 
 @register_node("dwn_stable")
@@ -45,7 +45,7 @@ class DWNStableNode(BaseNode):
         self._apply_init_fn(self.raw_luts, name="raw_luts")
 
     def _get_luts(self):
-        return ops.TableSigmoidFunction.apply(self.raw_luts)
+        return ops.table_sigmoid(self.raw_luts)
 
     def forward_train(self, x):
         return dwn_stable_forward(x, self._get_luts(), self.gradient_scale.detach())

@@ -24,7 +24,7 @@ def hybrid_forward(input, luts, binary_combinations=None):
     (hybrid_node.py:229-249).  `binary_combinations` is accepted for signature compatibility: the
     kernels enumerate the corners themselves (input 0 = least significant bit)."""
     plan = _identity_plan(input.shape[1], input.device)
-    return ops.HybridLayerFunction.apply(input, luts.unsqueeze(0), plan)
+    return ops.hybrid_layer(input, luts.unsqueeze(0), plan)
 
 
 @register_node("hybrid")
@@ -44,7 +44,7 @@ class HybridNode(BaseNode):
         self.register_buffer("binary_combinations", bits.to(torch.float32))
 
     def _get_luts(self):
-        return ops.TableSigmoidFunction.apply(self.raw_luts)
+        return ops.table_sigmoid(self.raw_luts)
 
     def forward_train(self, x):
         return hybrid_forward(x, self._get_luts(), self.binary_combinations)

@@ -24,7 +24,7 @@ _CUDA_EXT_AVAILABLE = _native.is_built()
 def probabilistic_forward(input, raw_weights, temperature):
     """(batch, k), (2^k, output_dim) -> (batch, output_dim); autograd-aware."""
     plan = _identity_plan(input.shape[1], input.device)
-    return ops.ProbLayerFunction.apply(input, raw_weights.unsqueeze(0), plan, temperature)
+    return ops.prob_layer(input, raw_weights.unsqueeze(0), plan, temperature)
 
 
 @register_node("probabilistic")

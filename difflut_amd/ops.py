@@ -11,6 +11,7 @@ synchronises the device.
 import torch
 
 from . import _native as nat
+from . import cpu_ops
 
 FAST_K = 6
 
@@ -197,7 +198,8 @@ class DWNStackFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, source, plans, scalars, head, *luts):
-        """`head`: None, or (groups, tau) of a GroupSum that follows the last layer: the function then returns
+        """`scalars`: per layer (alpha, beta) as numbers, or (alpha [N], beta [N], max |beta|) with every node's own.
+        `head`: None, or (groups, tau) of a GroupSum that follows the last layer: the function then returns
         the [B, groups] sums and neither the last layer's [B, N] output nor its gradient is ever written.
         `source` says what the first layer reads:
         None                  x [B, I] itself;
@@ -280,7 +282,6 @@ class DWNStackFunction(torch.autograd.Function):
         for l in range(n - 1, -1, -1):
             B, I, N, k, O = dims = ctx.dims_all[l]
             plan = ctx.plans[l]
-            alpha, beta = ctx.scalars[l]
             if l > 0:
                 gx = torch.empty(lib.dl_dwn_tiled_bytes(B, I) // 4, dtype=torch.float32, device=g.device)
                 gx_tiled = 1
@@ -295,8 +296,21 @@ class DWNStackFunction(torch.autograd.Function):
                     gx = torch.empty((B, I), dtype=torch.float32, device=g.device)
             grads[l] = torch.empty_like(luts[l])
             ws = _bytes(lib.dl_dwn_bwd_workspace_bytes(*dims), g.device)
-            if l == n - 1 and ctx.head is not None:
-                groups, tau = ctx.head
+            headed = l == n - 1 and ctx.head is not None
+            groups, tau = ctx.head if headed else (1, 1.0)
+            if len(ctx.scalars[l]) == 3:  # every node's own alpha and beta
+                alpha_n, beta_n, beta_max = ctx.scalars[l]
+                alpha_n = _f32(alpha_n.detach()).reshape(-1).expand(N).contiguous()
+                beta_n = _f32(beta_n.detach()).reshape(-1).expand(N).contiguous()
+                nat.check(lib.dl_dwn_layer_bwd_chain_nodes(nat.ptr(saved[l]), nat.ptr(plan.inv_ptr), nat.ptr(plan.inv_pos),
+                                                           nat.ptr(luts[l]), nat.ptr(g), 2 if headed else tiled, int(groups),
+                                                           float(tau), nat.ptr(alpha_n), nat.ptr(beta_n), float(beta_max),
+                                                           nat.ptr(gx), gx_tiled, nat.ptr(grads[l]), nat.ptr(ws), ws.numel(),
+                                                           *dims, nat.stream()))
+                g, tiled = gx, gx_tiled
+                continue
+            alpha, beta = ctx.scalars[l]
+            if headed:
                 nat.check(lib.dl_dwn_layer_bwd_groups(nat.ptr(saved[l]), nat.ptr(plan.inv_ptr), nat.ptr(plan.inv_pos),
                                                       nat.ptr(luts[l]), nat.ptr(g), int(groups), float(tau), float(alpha),
                                                       float(beta), nat.ptr(gx), gx_tiled, nat.ptr(grads[l]), nat.ptr(ws),
@@ -363,6 +377,8 @@ def dwn_stack_eval(x, thresholds, plans, luts, head=None):
 
 
 def dwn_layer_eval(x, luts, plan):
+    if not x.is_cuda:
+        return cpu_ops.dwn_layer_eval(x, luts, plan)
     nat.require_device(x, luts)
     x, luts = _f32(x), _f32(luts)
     B, I = x.shape
@@ -480,8 +496,16 @@ class HybridLayerFunction(torch.autograd.Function):
 
 
 # ----------------------------------------------------------------------------- Probabilistic
+def _node_temperatures(temperature, N, device):
+    """None for one temperature (a number), else the nodes' own values as a float32 device array [N]."""
+    if not torch.is_tensor(temperature):
+        return None
+    return temperature.detach().to(device=device, dtype=torch.float32).reshape(-1).expand(N).contiguous()
+
+
 class ProbLayerFunction(torch.autograd.Function):
-    """y[b, n*O+d] = sum_a sigmoid(raw[n,a,d]/T) prod_j (x_j a_j + (1-x_j)(1-a_j))."""
+    """y[b, n*O+d] = sum_a sigmoid(raw[n,a,d]/T) prod_j (x_j a_j + (1-x_j)(1-a_j)); `temperature` is a number for the
+    whole layer or a tensor [N] with every node's own value."""
 
     @staticmethod
     def forward(ctx, x, raw, plan, temperature):
@@ -496,15 +520,20 @@ class ProbLayerFunction(torch.autograd.Function):
         y = torch.empty((B, N * O), dtype=torch.float32, device=x.device)
         dims = (B, I, N, k, O)
         saved = _bytes(nat.lib().dl_prob_saved_bytes(*dims), x.device)
-        nat.check(nat.lib().dl_prob_layer_fwd(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(raw), float(temperature),
-                                              nat.ptr(y), nat.ptr(saved), saved.numel(), *dims, nat.stream()))
-        ctx.save_for_backward(x, raw, saved)
-        ctx.plan, ctx.T, ctx.dims = plan, float(temperature), dims
+        T = _node_temperatures(temperature, N, x.device)
+        if T is None:
+            nat.check(nat.lib().dl_prob_layer_fwd(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(raw), float(temperature),
+                                                  nat.ptr(y), nat.ptr(saved), saved.numel(), *dims, nat.stream()))
+        else:
+            nat.check(nat.lib().dl_prob_layer_fwd_nodes(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(raw), nat.ptr(T),
+                                                        nat.ptr(y), nat.ptr(saved), saved.numel(), *dims, nat.stream()))
+        ctx.save_for_backward(x, raw, saved, T)
+        ctx.plan, ctx.T, ctx.dims = plan, None if T is not None else float(temperature), dims
         return y
 
     @staticmethod
     def backward(ctx, gy):
-        x, raw, saved = ctx.saved_tensors
+        x, raw, saved, T = ctx.saved_tensors
         plan = ctx.plan
         gy = _f32(gy)
         lib = nat.lib()
@@ -512,14 +541,21 @@ class ProbLayerFunction(torch.autograd.Function):
         gx = torch.empty((B, I), dtype=torch.float32, device=gy.device) if ctx.needs_input_grad[0] else None
         graw = torch.empty_like(raw)
         ws = _bytes(lib.dl_prob_bwd_workspace_bytes(*ctx.dims), gy.device)
-        nat.check(lib.dl_prob_layer_bwd(nat.ptr(x), nat.ptr(saved), nat.ptr(plan.idx32), nat.ptr(plan.inv_ptr),
-                                        nat.ptr(plan.inv_pos),
-                                        nat.ptr(raw), ctx.T, nat.ptr(gy), nat.ptr(gx), nat.ptr(graw), nat.ptr(ws),
-                                        ws.numel(), *ctx.dims, nat.stream()))
+        if T is None:
+            nat.check(lib.dl_prob_layer_bwd(nat.ptr(x), nat.ptr(saved), nat.ptr(plan.idx32), nat.ptr(plan.inv_ptr),
+                                            nat.ptr(plan.inv_pos),
+                                            nat.ptr(raw), ctx.T, nat.ptr(gy), nat.ptr(gx), nat.ptr(graw), nat.ptr(ws),
+                                            ws.numel(), *ctx.dims, nat.stream()))
+        else:
+            nat.check(lib.dl_prob_layer_bwd_nodes(nat.ptr(x), nat.ptr(saved), nat.ptr(plan.idx32), nat.ptr(plan.inv_ptr),
+                                                  nat.ptr(plan.inv_pos), nat.ptr(raw), nat.ptr(T), nat.ptr(gy), nat.ptr(gx),
+                                                  nat.ptr(graw), nat.ptr(ws), ws.numel(), *ctx.dims, nat.stream()))
         return gx, graw, None, None
 
 
 def prob_layer_eval(x, raw, plan, temperature):
+    if not x.is_cuda:
+        return cpu_ops.prob_layer_eval(x, raw, plan, temperature)
     nat.require_device(x, raw)
     x, raw = _f32(x), _f32(raw)
     B, I = x.shape
@@ -528,8 +564,13 @@ def prob_layer_eval(x, raw, plan, temperature):
     lib = nat.lib()
     dims = (B, I, N, plan.k, O)
     ws = _bytes(lib.dl_prob_eval_workspace_bytes(*dims), x.device)
-    nat.check(lib.dl_prob_layer_eval_ws(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(raw), float(temperature), nat.ptr(y),
-                                        nat.ptr(ws), ws.numel(), *dims, nat.stream()))
+    T = _node_temperatures(temperature, N, x.device)
+    if T is None:
+        nat.check(lib.dl_prob_layer_eval_ws(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(raw), float(temperature), nat.ptr(y),
+                                            nat.ptr(ws), ws.numel(), *dims, nat.stream()))
+    else:
+        nat.check(lib.dl_prob_layer_eval_ws_nodes(nat.ptr(x), nat.ptr(plan.idx32), nat.ptr(raw), nat.ptr(T), nat.ptr(y),
+                                                  nat.ptr(ws), ws.numel(), *dims, nat.stream()))
     return y
 
 
@@ -572,6 +613,8 @@ class SoftMapFunction(torch.autograd.Function):
 
 
 def row_argmax(W):
+    if not W.is_cuda:
+        return cpu_ops.row_argmax(W)
     nat.require_device(W)
     W = _f32(W)
     sel = torch.empty((W.shape[0],), dtype=torch.int32, device=W.device)
@@ -607,6 +650,8 @@ class HardSelectFunction(torch.autograd.Function):
 
 # ----------------------------------------------------------------------------- encoder / head
 def thermometer_encode(x, thresholds):
+    if not x.is_cuda:
+        return cpu_ops.thermometer_encode(x, thresholds)
     nat.require_device(x, thresholds)
     x, thr = _f32(x), _f32(thresholds)
     B, F = x.shape
@@ -661,3 +706,63 @@ class GroupSumFunction(torch.autograd.Function):
         gx = torch.empty((B, F), dtype=torch.float32, device=gy.device)
         nat.check(nat.lib().dl_group_sum_bwd(nat.ptr(gy), nat.ptr(gx), B, F, groups, tau, nat.stream()))
         return gx, None, None
+
+
+# ----------------------------------------------------------------------------- dispatch
+# The reference's rule (random_layer.py:272, dwn_node.py:334, probabilistic_node.py:277): the extension runs iff the
+# input is a device tensor, otherwise the CPU code does.  Layers, nodes, the encoder and the head call these.
+def gather(x, idx, plan):
+    return GatherFunction.apply(x, idx, plan) if x.is_cuda else cpu_ops.gather(x, idx)
+
+
+def dwn_layer(x, luts, plan, alpha, beta, beta_abs_max=None):
+    if x.is_cuda:
+        return DWNLayerFunction.apply(x, luts, plan, alpha, beta, beta_abs_max)
+    return cpu_ops.dwn_layer(x, luts, plan, alpha, beta)
+
+
+def dwn_stable_layer(x, luts, scale, plan):
+    return DWNStableLayerFunction.apply(x, luts, scale, plan) if x.is_cuda else cpu_ops.dwn_stable_layer(x, luts, scale, plan)
+
+
+def hybrid_layer(x, luts, plan):
+    return HybridLayerFunction.apply(x, luts, plan) if x.is_cuda else cpu_ops.hybrid_layer(x, luts, plan)
+
+
+def table_sigmoid(raw):
+    return TableSigmoidFunction.apply(raw) if raw.is_cuda else torch.sigmoid(raw.float())
+
+
+def prob_layer(x, raw, plan, temperature):
+    return ProbLayerFunction.apply(x, raw, plan, temperature) if x.is_cuda else cpu_ops.prob_layer(x, raw, plan, temperature)
+
+
+def soft_map(x, W, tau, precision=0):
+    return SoftMapFunction.apply(x, W, tau, precision) if x.is_cuda else cpu_ops.soft_map(x, W, tau, precision)
+
+
+def hard_select(x, sel, plan):
+    return HardSelectFunction.apply(x, sel, plan) if x.is_cuda else cpu_ops.hard_select(x, sel)
+
+
+def unfold(x, geom, flip=None):
+    """Patch matrix [B*OH*OW, C*KH*KW] of an image batch; on the CPU nn.functional.unfold, transposed and flattened
+    as convolutional.py:199-205 does, with the flip applied to the patches."""
+    if x.is_cuda:
+        return UnfoldFunction.apply(x, geom, flip)
+    kh, kw, sh, sw, ph, pw = geom
+    cols = torch.nn.functional.unfold(x.float(), (kh, kw), padding=(ph, pw), stride=(sh, sw))
+    patches = cols.transpose(1, 2).reshape(-1, cols.shape[1])
+    if flip is not None:
+        patches = patches + torch.where(flip.bool(), 1.0 - 2.0 * patches.detach(), torch.zeros_like(patches))
+    return patches
+
+
+def group_sum(x, groups, tau):
+    return GroupSumFunction.apply(x, groups, tau) if x.is_cuda else cpu_ops.group_sum(x, groups, tau)
+
+
+def cross_entropy(logits, labels):
+    if logits.is_cuda:
+        return CrossEntropyFunction.apply(logits, labels)
+    return torch.nn.functional.cross_entropy(logits.float(), labels.long())

@@ -48,12 +48,12 @@ class GroupSum(nn.Module):
         if features % self.k != 0:
             warnings.warn(f"GroupSum: Input has {features} features which is not divisible by k={self.k}. Adding "
                           f"{self.k - features % self.k} zero-padded features.", UserWarning, stacklevel=2)
-        return ops.GroupSumFunction.apply(x, self.k, self.tau)
+        return ops.group_sum(x, self.k, self.tau)
 
 
 def cross_entropy(logits, labels):
     """Mean cross-entropy of [batch, classes] logits (e.g. what GroupSum returns) against int64 class labels, loss and
     gradient from one pass on the device: a drop-in for `torch.nn.functional.cross_entropy(logits, labels)` with
     its default mean reduction (no class weights, no label smoothing, no ignore_index)."""
-    return ops.CrossEntropyFunction.apply(logits, labels)
+    return ops.cross_entropy(logits, labels)
 

@@ -3,7 +3,8 @@
  * One shared library, libdifflut_hip.so, built from difflut_amd/csrc/ by hipcc.
  * Plain pointers and sizes only; every pointer is DEVICE memory unless it says
  * host.  `stream` is a hipStream_t passed as void*.  Nothing here allocates or
- * frees device memory and nothing synchronises the device: outputs and
+ * frees device memory and nothing synchronises the device (except
+ * dl_profile_read, which waits for the kernels it reports on): outputs and
  * workspaces come from the caller, kernels are enqueued on `stream`.
  *
  * Return value of every int function: 0 = ok, negative = argument error
@@ -22,8 +23,9 @@
  * Size limits (DL_ERR_UNSUPPORTED beyond them, checked on the host before anything is launched):
  * k <= DL_MAX_K; N * O * 2^k < 2^31 table entries per layer; I <= 2^28 for the k <= 6 DWN kernels;
  * B <= 4 000 000 rows for the probabilistic entry points and dl_thermometer_planes (their batch tiles are a
- * grid dimension); C * KH * KW <= 4096 patch columns for dl_unfold / dl_fold.  The gathers, the bit-plane
- * packing and the DWN layers take any B that fits an int.
+ * grid dimension); C * KH * KW <= 4096 patch columns for dl_unfold / dl_fold.  The DWN layers take
+ * B <= 2^31 - 65 rows as long as their 1-D grids fit 31 bits: ceil(N*O/128) * T and ceil(I/4) * T + N*O*2^k/1024
+ * blocks, T = ceil(B/64) rounded up to a multiple of 8.  The gathers and the bit-plane packing take any B that fits an int.
  */
 #ifndef DIFFLUT_HIP_H
 #define DIFFLUT_HIP_H
@@ -95,7 +97,10 @@ int dl_dwn_layer_fwd(const float *x, const int32_t *idx32, const float *luts, fl
  * allocates and frees nothing.  Limit: ceil(B/64) * I * 8 <= DL_DWN_STATIC_SCRATCH_BYTES when
  * k <= DL_MAX_FAST_K (e.g. B = 4096 with I = 16384), otherwise DL_ERR_SCRATCH; larger k uses no scratch.
  * All calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams, two threads)
- * race on it and must be serialised by the caller.  Nothing in it has to survive between calls. */
+ * race on it and must be serialised by the caller.  Nothing in it has to survive between calls.
+ * The first call on each device also looks up the device address of the array (hipGetSymbolAddress, which may
+ * load the code object): make that call before any stream capture begins; every later call on the device only
+ * enqueues kernels and can be captured. */
 #define DL_DWN_STATIC_SCRATCH_BYTES (8u << 20)
 int dl_dwn_layer_fwd_static(const float *x, const int32_t *idx32, const float *luts, float *y,
                             void *saved, int B, int I, int N, int k, int O, void *stream);
@@ -153,6 +158,14 @@ int dl_dwn_layer_bwd_groups(const void *saved, const int32_t *inv_ptr, const int
                             const float *glogits, int groups, float tau, float alpha, float beta,
                             float *gx, int gx_tiled, float *gluts, void *ws, size_t ws_bytes,
                             int B, int I, int N, int k, int O, void *stream);
+/* The chained backward with every node's own alpha and beta (device arrays [N]; the reference reads each node's
+ * buffers, difflut/nodes/dwn_node.py:417-418,450).  beta_abs_max = max |beta_n| (a host value) selects the form of
+ * the coefficient table.  gy_form: 0 = gy row-major [B, N*O], 1 = tile-major [B/64][N*O][64], 2 = the [B, groups]
+ * gradient of a GroupSum head's logits (groups, tau as in dl_dwn_layer_bwd_groups; ignored otherwise). */
+int dl_dwn_layer_bwd_chain_nodes(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos, const float *luts,
+                                 const float *gy, int gy_form, int groups, float tau, const float *alpha_n,
+                                 const float *beta_n, float beta_abs_max, float *gx, int gx_tiled, float *gluts,
+                                 void *ws, size_t ws_bytes, int B, int I, int N, int k, int O, void *stream);
 /* The eval forward below with a workspace (dl_dwn_eval_workspace_bytes): the same result for any input, and
  * the bit-plane kernels' speed when every input value is exactly 0 or 1 (checked on the device while packing;
  * no host synchronisation - both kernels are launched and one returns at once). */
@@ -246,6 +259,14 @@ int dl_prob_layer_bwd(const float *x, const void *saved, const int32_t *idx32,
                       const float *raw_w, float temperature, const float *gy,
                       float *gx, float *graw, void *ws, size_t ws_bytes,
                       int B, int I, int N, int k, int O, void *stream);
+/* The same forward and backward with every node's own temperature (device array [N]; the reference reads each
+ * node's `temperature` buffer, difflut/nodes/probabilistic_node.py:277-282, 224-239). */
+int dl_prob_layer_fwd_nodes(const float *x, const int32_t *idx32, const float *raw_w, const float *temperature_n,
+                            float *y, void *saved, size_t saved_bytes, int B, int I, int N, int k, int O, void *stream);
+int dl_prob_layer_bwd_nodes(const float *x, const void *saved, const int32_t *idx32, const int32_t *inv_ptr,
+                            const int32_t *inv_pos, const float *raw_w, const float *temperature_n, const float *gy,
+                            float *gx, float *graw, void *ws, size_t ws_bytes, int B, int I, int N, int k, int O,
+                            void *stream);
 /* Eval forward (probabilistic_node.py:302-328): y = (sigmoid(raw_w[n,addr,d]/T) >= 0.5). */
 int dl_prob_layer_eval(const float *x, const int32_t *idx32, const float *raw_w, float temperature,
                        float *y, int B, int I, int N, int k, int O, void *stream);
@@ -255,6 +276,8 @@ int dl_prob_layer_eval(const float *x, const int32_t *idx32, const float *raw_w,
 size_t dl_prob_eval_workspace_bytes(int B, int I, int N, int k, int O);
 int dl_prob_layer_eval_ws(const float *x, const int32_t *idx32, const float *raw_w, float temperature, float *y,
                           void *ws, size_t ws_bytes, int B, int I, int N, int k, int O, void *stream);
+int dl_prob_layer_eval_ws_nodes(const float *x, const int32_t *idx32, const float *raw_w, const float *temperature_n,
+                                float *y, void *ws, size_t ws_bytes, int B, int I, int N, int k, int O, void *stream);
 
 /* ------------------------------------------------------------------------
  * LearnableLayer soft connectivity (training) and hard selection (eval).

@@ -141,8 +141,7 @@ def test_constructor_validation_and_cpu_refusal():
         layer(torch.zeros(8))
     with pytest.raises(ValueError, match="expected input with 8 features"):
         layer(torch.zeros(2, 9))
-    with pytest.raises(RuntimeError, match="ROCm devices only"):
-        layer(torch.zeros(2, 8))  # no CPU fallback
+    assert layer(torch.zeros(2, 8)).shape == (2, 4)  # CPU tensors take the plain-torch branch
     assert DWNNode(input_dim=6, output_dim=1).alpha.item() == pytest.approx(0.5 * 0.75 ** 5)
 
 
@@ -224,8 +223,7 @@ def test_convolutional_layer_construction_matches_reference(golden_next):
     assert layer.hidden_layers == [4, 2, 1] and len(layer.first_layer_chunks) == 2 and len(layer.trees) == 3
     assert [tuple(t.shape) for t in layer.bank_parameters()] == [(12, 1, 4), (6, 1, 4), (3, 1, 4)]
     assert np.array_equal(torch.rand(4, 2, 4, 4)[:2].numpy(), g["conv_x"])  # generator position after construction
-    with pytest.raises(RuntimeError):
-        layer(torch.rand(2, 2, 4, 4))  # CPU tensors are refused
+    assert layer(torch.rand(2, 2, 4, 4)).shape == (2, 3, 3, 3)  # CPU tensors take the plain-torch branch
     torch.manual_seed(32)
     gcfg = ConvolutionConfig(tree_depth=1, in_channels=4, out_channels=5, receptive_field=3, stride=1, padding=0,
                              chunk_size=2, seed=43)
@@ -321,39 +319,59 @@ def test_bank_notices_nodes_taken_over_or_replaced():
 def test_scalar_buffers_are_banked_and_differences_are_seen():
     layer = _small_dwn_layer()
     alpha, beta = layer._scalars["alpha"], layer._scalars["beta"]
-    same, value, _ = alpha.summary()
-    assert same and value == pytest.approx(0.5 * 0.75 ** 2)
-    assert layer.efd_scalars() == (pytest.approx(0.5 * 0.75 ** 2), pytest.approx(1 / 3))
+    alpha_n, beta_n, beta_max = layer.efd_scalars()
+    assert alpha_n.shape == beta_n.shape == (12,) and alpha_n.dtype == torch.float32
+    assert float(alpha_n[3]) == pytest.approx(0.5 * 0.75 ** 2) and beta_max == pytest.approx(1 / 3)
     assert set(layer.state_dict()) >= {"nodes.0.alpha", "nodes.11.beta"} and layer.state_dict()["nodes.0.alpha"].shape == ()
-    # a state dict with another value for one node in the middle lands in the bank
+    # a state dict with another value for one node in the middle lands in the array the kernels are handed
     state = layer.state_dict()
     state["nodes.7.alpha"] = torch.tensor(0.25)
     layer.load_state_dict(state)
-    assert alpha.tied() and float(alpha.flat[7]) == 0.25
-    assert alpha.summary()[0] is False
-    with pytest.raises(RuntimeError, match="different alpha"):
-        layer.efd_scalars()
-    # in-place edits too; making all equal again is seen as well
+    assert alpha.tied() and float(layer.efd_scalars()[0][7]) == 0.25 and float(layer.efd_scalars()[0][6]) != 0.25
+    # in-place edits too
     with torch.no_grad():
-        for node in layer.nodes:
-            node.alpha.fill_(0.25)
-    assert alpha.summary()[:2] == (True, 0.25)
+        layer.nodes[4].beta.fill_(0.75)
+    assert float(layer.efd_scalars()[1][4]) == 0.75 and layer.efd_scalars()[2] == pytest.approx(0.75)
     # replacing a node's buffer object re-ties on the next use
     layer.nodes[2].beta = torch.tensor(0.9)
     assert not beta.tied()
-    assert beta.summary() == (False, pytest.approx(1 / 3), pytest.approx(0.9))
+    assert layer.efd_scalars()[2] == pytest.approx(0.9)
     assert layer.nodes[2].beta.data_ptr() == beta.flat[2].data_ptr()
+    # a buffer entry swapped behind the module's back (no __setattr__) is noticed as well
+    layer.nodes[5]._buffers["alpha"] = torch.tensor(0.5)
+    assert not alpha.tied()
+    assert float(layer.efd_scalars()[0][5]) == 0.5 and alpha.tied()
 
 
-def test_probabilistic_layer_refuses_per_node_temperatures():
+def test_writes_that_bypass_the_version_counter():
+    """`buffer.data.fill_` does not bump the version the host-side summary is keyed on: the kernels still get the
+    value (they are handed the array itself), and `invalidate_scalars()` refreshes max |beta|, which selects the
+    form of the coefficient table."""
+    layer = _small_dwn_layer()
+    assert layer.efd_scalars()[2] == pytest.approx(1 / 3)
+    layer.nodes[1].beta.data.fill_(0.9)
+    assert float(layer.efd_scalars()[1][1]) == pytest.approx(0.9)  # the value itself is never stale
+    assert layer.efd_scalars()[2] == pytest.approx(1 / 3)          # the cached maximum is
+    layer.invalidate_scalars()
+    assert layer.efd_scalars()[2] == pytest.approx(0.9)
+
+
+def test_scalar_banks_keep_the_buffers_dtype():
+    layer = _small_dwn_layer().double()
+    assert layer.nodes[3].alpha.dtype == torch.float64 and layer.nodes[3].luts.dtype == torch.float64
+    alpha_n, beta_n, _ = layer.efd_scalars()
+    assert alpha_n.dtype == beta_n.dtype == torch.float32  # the kernels' view
+    assert layer.state_dict()["nodes.3.beta"].dtype == torch.float64
+
+
+def test_probabilistic_layer_hands_over_per_node_temperatures():
     from difflut_amd.layers import RandomLayer
     from difflut_amd.nodes import NodeConfig, ProbabilisticNode
     layer = RandomLayer(16, 8, ProbabilisticNode, NodeConfig(input_dim=2, output_dim=1), seed=1)
-    assert layer.temperature_value() == 1.0
+    assert torch.equal(layer.temperatures(), torch.ones(8))
     with torch.no_grad():
         layer.nodes[5].temperature.fill_(2.0)
-    with pytest.raises(RuntimeError, match="different temperatures"):
-        layer.temperature_value()
+    assert float(layer.temperatures()[5]) == 2.0 and float(layer.temperatures()[4]) == 1.0
 
 
 def test_size_limits_and_argument_errors_are_reported_before_any_launch():

@@ -62,3 +62,44 @@ def test_static_scratch_forward_at_its_limit_and_beyond():
     rc = lib.dl_dwn_layer_fwd_static(x.data_ptr(), one.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(),
                                      B + 1, I, 1, 6, 1, nat.stream())
     assert rc == -6 and b"scratch" in lib.dl_error_string(rc)
+
+
+def test_static_scratch_forward_allocates_nothing_and_can_be_captured():
+    """After the first call on the device (which looks up the array's address) a call neither changes the device's
+    free memory nor needs anything a stream capture forbids: the same call replayed from a HIP graph, with eager
+    work and synchronisations in between, gives the eager result every time."""
+    from difflut_amd import _native as nat
+    lib = nat.lib()
+    B, I, N, k, O = 300, 200, 260, 6, 1
+    dims = (B, I, N, k, O)
+    rng = np.random.default_rng(21)
+    idx = orc.random_mapping(I, N, k, seed=22).to(torch.int32).to(DEV).contiguous()
+    luts = torch.as_tensor(rng.uniform(-1, 1, (N, O, 1 << k)).astype(np.float32)).to(DEV)
+    x = torch.as_tensor(rng.random((B, I)).astype(np.float32)).to(DEV)
+    y = torch.empty((B, N * O), device=DEV)
+    saved = torch.zeros(lib.dl_dwn_saved_bytes(*dims), dtype=torch.uint8, device=DEV)
+
+    def call():
+        nat.check(lib.dl_dwn_layer_fwd_static(x.data_ptr(), idx.data_ptr(), luts.data_ptr(), y.data_ptr(), saved.data_ptr(),
+                                              *dims, nat.stream()))
+
+    call()  # the first call on this device, outside any capture
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    call()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            call()
+    for rep in range(3):
+        x.copy_(torch.as_tensor(rng.random((B, I)).astype(np.float32)))
+        y.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        want = orc.dwn_layer_forward(x.cpu().numpy(), idx.cpu().numpy().astype(np.int64), luts.cpu().numpy())
+        assert np.array_equal(y.cpu().numpy(), want.reshape(B, N * O)), rep
+        assert float((y * 2).sum()) == float((y * 2).sum())  # eager work between the replays
