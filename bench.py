@@ -141,16 +141,34 @@ def steady_state(step, ms=PRERUN_MS, max_ms=PRERUN_MAX_MS, chunk=8):
     return chunk * len(times)
 
 
+WINDOWS = 5
+
+
+def timed_windows(step, steps, windows=WINDOWS):
+    """`windows` back-to-back timed regions of exactly `steps` steps, each bracketed by a device synchronisation on both
+    sides: milliseconds per step of every window.  The reported figure is the median window; minimum and maximum go
+    into the line as well, so that the spread of one run is visible (boxes of the pool differ by several per cent)."""
+    out = []
+    for _ in range(windows):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        out.append((time.perf_counter() - t0) * 1e3 / steps)
+    return out
+
+
+def window_summary(per_window):
+    return {"count": len(per_window), "steps_each": None, "median_ms": float(np.median(per_window)),
+            "min_ms": float(min(per_window)), "max_ms": float(max(per_window))}
+
+
 def time_steps(step, steps, warmup):
     steady_state(step)
     for _ in range(warmup):
         step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) * 1e3 / steps
+    return float(np.median(timed_windows(step, steps)))
 
 
 def kernel_times(step, reps):
@@ -187,7 +205,8 @@ def run_stack(args):
         width = n * O
     head = GroupSum(k=10, tau=1.0, use_randperm=False)
     params = [p for layer in layers for p in layer.bank_parameters()]
-    opt = torch.optim.Adam(params, lr=1e-3, fused=True)  # one kernel for the four table banks instead of eight
+    from difflut_amd.utils import BankAdam
+    opt = BankAdam(params, lr=1e-3)  # torch.optim.Adam's arithmetic, one launch of the library for the four table banks
     from difflut_amd.layers import DWNStack
     # same layers; thermometer code and activations as bit-planes, tile-major gradients between layers
     stack = DWNStack(layers, encoder=enc, head=head).train()
@@ -591,13 +610,8 @@ def main():
     prerun_steps = steady_state(step)  # untimed: sustained clocks (see steady_state)
     for _ in range(args.warmup):
         step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
+    per_window = timed_windows(step, args.steps)  # WINDOWS regions of exactly --steps steps, each between two syncs
+    ms_per_step = float(np.median(per_window))
     evals = B * N
 
     # per-kernel durations: HIP events recorded by the library around each launch, same stream
@@ -628,6 +642,9 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
+        "timed_windows": dict(window_summary(per_window), steps_each=args.steps,
+                              note="ms_per_step is the median window; every window is exactly --steps steps between two "
+                                   "device synchronisations"),
         "steady_state_prerun": {"min_ms": PRERUN_MS, "max_ms": PRERUN_MAX_MS, "steps": prerun_steps,
                                 "why": "untimed steps before the warm-up, until chunks of 8 steps agree within 1 %: "
                                        "device clocks settle about 20 ms after idle"},

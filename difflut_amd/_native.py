@@ -75,6 +75,7 @@ SIGNATURES = {
     "dl_cross_entropy_workspace_bytes": (_Z, [_I]),
     "dl_cross_entropy": (_I, [_P, _P, _P, _P, _P, _Z, _I, _I, _P]),
     "dl_group_sum_bwd": (_I, [_P, _P, _I, _I, _I, _F, _P]),
+    "dl_adam_step": (_I, [_P, _P, _P, _P, _P, _I, _F, _F, _F, _F, _F, _I, _I, _P]),
     "dl_profile_enable": (_I, [_I]),
     "dl_profile_read": (_I, [ctypes.c_char_p, _Z, ctypes.POINTER(_F), _I]),
 }

@@ -338,6 +338,18 @@ int dl_cross_entropy(const float *logits, const long long *labels, float *loss, 
 int dl_group_sum_bwd(const float *gy, float *gx, int B, int F, int groups, float tau, void *stream);
 
 /* ------------------------------------------------------------------------
+ * Adam update of parameter banks (the [N, O, 2^k] tensors the layers keep their nodes' tables in): the arithmetic
+ * of torch.optim.Adam without amsgrad - what the reference's training scripts apply to the per-node parameters
+ * (experiments and examples construct torch.optim.Adam(model.parameters(), lr=...)) - for `count` tensors in one
+ * launch.  params / grads / exp_avg / exp_avg_sq and numel are HOST arrays of `count` device pointers / element
+ * counts; `step` is the 1-based step number (bias corrections 1 - beta^step are computed on the host in double).
+ * In place: params, exp_avg, exp_avg_sq. */
+#define DL_ADAM_MAX_TENSORS 8 /* tensors per launch; more are taken in several launches */
+int dl_adam_step(void *const *params, const void *const *grads, void *const *exp_avg, void *const *exp_avg_sq,
+                 const long long *numel, int count, float lr, float beta1, float beta2, float eps, float weight_decay,
+                 int step, int maximize, void *stream);
+
+/* ------------------------------------------------------------------------
  * Convolutional LUT layer: patch extraction and its adjoint.
  * Replaces nn.Unfold + transpose + contiguous + view in ConvolutionalLayer.forward
  * (difflut/layers/convolutional.py:199-205) and what autograd does for them in the backward.

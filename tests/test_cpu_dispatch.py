@@ -237,3 +237,20 @@ def test_single_nodes_on_cpu(golden):
     xp = torch.rand(7, 3)
     np.testing.assert_allclose(pnode(xp).detach().numpy(),
                                orc.prob_forward(xp.numpy(), pnode.raw_weights.detach().numpy(), 1.0), rtol=1e-5, atol=1e-6)
+
+
+def test_bank_adam_matches_torch_adam_on_cpu():
+    from difflut_amd.utils import BankAdam
+
+    torch.manual_seed(2)
+    a = [torch.randn(7, 1, 16, requires_grad=True), torch.randn(33, requires_grad=True)]
+    b = [t.detach().clone().requires_grad_() for t in a]
+    ours, ref = BankAdam(a, lr=0.01, weight_decay=0.1), torch.optim.Adam(b, lr=0.01, weight_decay=0.1)
+    for _ in range(4):
+        for x, y in zip(a, b):
+            g = torch.randn_like(x)
+            x.grad, y.grad = g.clone(), g.clone()
+        ours.step()
+        ref.step()
+    for x, y in zip(a, b):
+        np.testing.assert_allclose(x.detach().numpy(), y.detach().numpy(), rtol=1e-6, atol=1e-7)

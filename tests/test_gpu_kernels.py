@@ -487,3 +487,29 @@ def test_row_counts_beyond_one_grid_dimension():
     bits[:R] = (v >= 0.5).long()
     want_planes = (bits.view(BT, 64, C) << torch.arange(64, device=DEV).view(1, 64, 1)).sum(1)  # wraps into the sign bit
     assert torch.equal(planes[:BT * C].view(BT, C), want_planes)
+
+
+@pytest.mark.parametrize("opts", [dict(lr=0.01), dict(lr=0.003, betas=(0.8, 0.95), eps=1e-6, weight_decay=0.05),
+                                  dict(lr=0.01, maximize=True)])
+def test_bank_adam_against_torch_adam(opts):
+    """`dl_adam_step`: several tensors of ragged sizes (one of them not 16-byte aligned) in one launch, five steps,
+    against torch.optim.Adam on the same gradients."""
+    from difflut_amd.utils import BankAdam
+
+    torch.manual_seed(11)
+    base = torch.randn(5000 + 1, device=DEV)
+    ours = [torch.randn(300, 1, 64, device=DEV).requires_grad_(), torch.randn(2049, device=DEV).requires_grad_(),
+            None, torch.randn(3, device=DEV).requires_grad_()]
+    ours[2] = base[1:].detach().requires_grad_()  # a view that starts 4 bytes into its allocation
+    ref = [t.detach().clone().requires_grad_() for t in ours]
+    opt, ropt = BankAdam(ours, **opts), torch.optim.Adam(ref, **opts)
+    for _ in range(5):
+        for x, y in zip(ours, ref):
+            g = torch.randn_like(x)
+            x.grad, y.grad = g.clone(), g.clone()
+        opt.step()
+        ropt.step()
+    for x, y in zip(ours, ref):
+        np.testing.assert_allclose(x.detach().cpu().numpy(), y.detach().cpu().numpy(), rtol=2e-6, atol=1e-7)
+    from difflut_amd import _native
+    assert _native.lib().dl_adam_step(None, None, None, None, None, 1, 0.1, 0.9, 0.999, 1e-8, 0.0, 1, 0, None) == -1
