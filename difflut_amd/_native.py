@@ -76,6 +76,8 @@ SIGNATURES = {
     "dl_cross_entropy": (_I, [_P, _P, _P, _P, _P, _Z, _I, _I, _P]),
     "dl_group_sum_bwd": (_I, [_P, _P, _I, _I, _I, _F, _P]),
     "dl_adam_step": (_I, [_P, _P, _P, _P, _P, _I, _F, _F, _F, _F, _F, _I, _I, _P]),
+    "dl_grad_stabilize_workspace_bytes": (_Z, [ctypes.c_longlong, ctypes.c_longlong, _I]),
+    "dl_grad_stabilize": (_I, [_P, _P, ctypes.c_longlong, ctypes.c_longlong, _I, _F, _I, _F, _P, _Z, _P]),
     "dl_profile_enable": (_I, [_I]),
     "dl_profile_read": (_I, [ctypes.c_char_p, _Z, ctypes.POINTER(_F), _I]),
 }

@@ -91,3 +91,92 @@ extern "C" int dl_adam_step(void *const *params, const void *const *grads, void 
     }
     return dl_launch_status();
 }
+
+// ---------------------------------------------------------------------------------
+// Gradient stabilisation of the layers (base_layer.py:266-339 of the reference): out = (g - mean) * sqrt(target /
+// (mean((g - mean)^2) + eps)), the mean taken over the whole tensor ("layerwise") or per row ("batchwise"), the mean
+// subtracted only when asked.  Sums are kept in double and added in a fixed order.
+//   per row:   one block per row, one launch.
+//   layerwise: grad_stab_partials leaves (sum, sum of squares) per block; grad_stab_apply lets every block add the
+//              partials in block order and rescale its own piece - two launches instead of torch's seven kernels.
+#define GS_THREADS 256
+#define GS_PER_BLOCK 4096  // elements per block of the layerwise form
+
+__device__ __forceinline__ void gs_block_sums(double &s, double &q, double *red) {
+    // sum over the block in a fixed order: lanes by butterfly, wavefronts in order
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        s += __shfl_xor(s, o);
+        q += __shfl_xor(q, o);
+    }
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) { red[2 * wave] = s; red[2 * wave + 1] = q; }
+    __syncthreads();
+    s = 0.0; q = 0.0;
+    for (int w = 0; w < GS_THREADS / 64; ++w) { s += red[2 * w]; q += red[2 * w + 1]; }
+    __syncthreads();
+}
+
+__global__ __launch_bounds__(GS_THREADS) void grad_stab_rows(const float *__restrict__ g, float *__restrict__ out, long long cols,
+                                                              float target, int subtract_mean, float eps) {
+    __shared__ double red[2 * GS_THREADS / 64];
+    const float *row = g + (size_t)blockIdx.x * cols;
+    float *dst = out + (size_t)blockIdx.x * cols;
+    double s = 0.0, q = 0.0;
+    for (long long c = threadIdx.x; c < cols; c += GS_THREADS) { const double v = row[c]; s += v; q += v * v; }
+    gs_block_sums(s, q, red);
+    const double mean = subtract_mean ? s / (double)cols : 0.0;
+    const double var = q / (double)cols - (subtract_mean ? mean * mean : 0.0);  // mean((g - mean)^2)
+    const float scale = (float)sqrt((double)target / ((var > 0.0 ? var : 0.0) + (double)eps)), m = (float)mean;
+    for (long long c = threadIdx.x; c < cols; c += GS_THREADS) dst[c] = (row[c] - m) * scale;
+}
+
+__global__ __launch_bounds__(GS_THREADS) void grad_stab_partials(const float *__restrict__ g, double *__restrict__ part, long long n) {
+    __shared__ double red[2 * GS_THREADS / 64];
+    const long long base = (long long)blockIdx.x * GS_PER_BLOCK;
+    double s = 0.0, q = 0.0;
+    for (int u = threadIdx.x; u < GS_PER_BLOCK; u += GS_THREADS)
+        if (base + u < n) { const double v = g[base + u]; s += v; q += v * v; }
+    gs_block_sums(s, q, red);
+    if (threadIdx.x == 0) { part[2 * (size_t)blockIdx.x] = s; part[2 * (size_t)blockIdx.x + 1] = q; }
+}
+
+__global__ __launch_bounds__(GS_THREADS) void grad_stab_apply(const float *__restrict__ g, float *__restrict__ out,
+                                                               const double *__restrict__ part, long long n, int blocks,
+                                                               float target, int subtract_mean, float eps) {
+    __shared__ double red[2 * GS_THREADS / 64];
+    double s = 0.0, q = 0.0;
+    for (int b = threadIdx.x; b < blocks; b += GS_THREADS) { s += part[2 * (size_t)b]; q += part[2 * (size_t)b + 1]; }
+    gs_block_sums(s, q, red);  // every block adds the partials in the same order: one value for the whole tensor
+    const double mean = subtract_mean ? s / (double)n : 0.0;
+    const double var = q / (double)n - (subtract_mean ? mean * mean : 0.0);
+    const float scale = (float)sqrt((double)target / ((var > 0.0 ? var : 0.0) + (double)eps)), m = (float)mean;
+    const long long base = (long long)blockIdx.x * GS_PER_BLOCK;
+    for (int u = threadIdx.x; u < GS_PER_BLOCK; u += GS_THREADS)
+        if (base + u < n) out[base + u] = (g[base + u] - m) * scale;
+}
+
+extern "C" size_t dl_grad_stabilize_workspace_bytes(long long rows, long long cols, int per_row) {
+    if (rows <= 0 || cols <= 0 || per_row) return 256;
+    return dl_align256((size_t)((rows * cols + GS_PER_BLOCK - 1) / GS_PER_BLOCK) * 2 * sizeof(double));
+}
+
+extern "C" int dl_grad_stabilize(const float *g, float *out, long long rows, long long cols, int per_row, float target_std,
+                                 int subtract_mean, float eps, void *ws, size_t ws_bytes, void *stream) {
+    if (!g || !out) return DL_ERR_NULL;
+    if (rows <= 0 || cols <= 0) return DL_ERR_SHAPE;
+    hipStream_t s = (hipStream_t)stream;
+    if (per_row) {
+        if (rows > 0x7fffffffLL) return DL_ERR_UNSUPPORTED;
+        DL_TIMED("grad_stab_rows", s, (grad_stab_rows<<<(int)rows, GS_THREADS, 0, s>>>(g, out, cols, target_std, subtract_mean, eps)));
+        return dl_launch_status();
+    }
+    const long long n = rows * cols, blocks = (n + GS_PER_BLOCK - 1) / GS_PER_BLOCK;
+    if (blocks > 0x7fffffffLL) return DL_ERR_UNSUPPORTED;
+    if (!ws) return DL_ERR_NULL;
+    if (ws_bytes < dl_grad_stabilize_workspace_bytes(rows, cols, 0)) return DL_ERR_WORKSPACE;
+    DL_TIMED("grad_stab_partials", s, (grad_stab_partials<<<(int)blocks, GS_THREADS, 0, s>>>(g, (double *)ws, n)));
+    DL_TIMED("grad_stab_apply", s, (grad_stab_apply<<<(int)blocks, GS_THREADS, 0, s>>>(g, out, (const double *)ws, n, (int)blocks,
+                                                                                    target_std, subtract_mean, eps)));
+    return dl_launch_status();
+}

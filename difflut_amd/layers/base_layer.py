@@ -237,6 +237,10 @@ class LUTLayerMixin(nn.Module):
         if self.grad_stabilization == "none" or not self.training or grad is None:
             return grad
         dims = None if self.grad_stabilization == "layerwise" else 1
+        if grad.is_cuda and grad.dim() == 2 and grad.dtype == torch.float32:
+            from .. import ops  # one or two library launches instead of seven torch kernels
+
+            return ops.grad_stabilize(grad, dims == 1, self.grad_target_std, self.grad_subtract_mean, self.grad_epsilon)
         g = grad.clone()
         if self.grad_subtract_mean:
             g -= g.mean() if dims is None else g.mean(dim=1, keepdim=True)

@@ -758,6 +758,20 @@ def unfold(x, geom, flip=None):
     return patches
 
 
+def grad_stabilize(grad, per_row, target_std, subtract_mean, eps):
+    """(grad - mean) * sqrt(target_std / (mean((grad - mean)^2) + eps)) for a [rows, cols] gradient on the device, over
+    the whole tensor or per row (base_layer.py:266-339); a new tensor."""
+    nat.require_device(grad)
+    g = _f32(grad)
+    rows, cols = g.shape
+    out = torch.empty_like(g)
+    lib = nat.lib()
+    ws = _bytes(lib.dl_grad_stabilize_workspace_bytes(rows, cols, int(per_row)), g.device)
+    nat.check(lib.dl_grad_stabilize(nat.ptr(g), nat.ptr(out), rows, cols, int(per_row), float(target_std),
+                                    int(bool(subtract_mean)), float(eps), nat.ptr(ws), ws.numel(), nat.stream()))
+    return out
+
+
 def group_sum(x, groups, tau):
     return GroupSumFunction.apply(x, groups, tau) if x.is_cuda else cpu_ops.group_sum(x, groups, tau)
 

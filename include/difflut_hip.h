@@ -344,6 +344,14 @@ int dl_group_sum_bwd(const float *gy, float *gx, int B, int F, int groups, float
  * launch.  params / grads / exp_avg / exp_avg_sq and numel are HOST arrays of `count` device pointers / element
  * counts; `step` is the 1-based step number (bias corrections 1 - beta^step are computed on the host in double).
  * In place: params, exp_avg, exp_avg_sq. */
+/* Gradient stabilisation of a layer's output gradient (LUTLayerMixin._apply_gradient_stabilization,
+ * difflut/layers/base_layer.py:266-339): out = (g - mean) * sqrt(target_std / (mean((g - mean)^2) + eps)) over the
+ * whole [rows, cols] tensor (per_row = 0, "layerwise") or per row (per_row = 1, "batchwise"); the mean is subtracted
+ * only when subtract_mean is set.  Sums in double, fixed order.  out may equal g only for per_row = 1.  The layerwise
+ * form needs dl_grad_stabilize_workspace_bytes(rows, cols, 0) bytes. */
+size_t dl_grad_stabilize_workspace_bytes(long long rows, long long cols, int per_row);
+int dl_grad_stabilize(const float *g, float *out, long long rows, long long cols, int per_row, float target_std,
+                      int subtract_mean, float eps, void *ws, size_t ws_bytes, void *stream);
 #define DL_ADAM_MAX_TENSORS 8 /* tensors per launch; more are taken in several launches */
 int dl_adam_step(void *const *params, const void *const *grads, void *const *exp_avg, void *const *exp_avg_sq,
                  const long long *numel, int count, float lr, float beta1, float beta2, float eps, float weight_decay,

@@ -513,3 +513,21 @@ def test_bank_adam_against_torch_adam(opts):
         np.testing.assert_allclose(x.detach().cpu().numpy(), y.detach().cpu().numpy(), rtol=2e-6, atol=1e-7)
     from difflut_amd import _native
     assert _native.lib().dl_adam_step(None, None, None, None, None, 1, 0.1, 0.9, 0.999, 1e-8, 0.0, 1, 0, None) == -1
+
+
+@pytest.mark.parametrize("per_row", [False, True])
+@pytest.mark.parametrize("subtract_mean", [False, True])
+def test_grad_stabilize_against_the_reference_formula(per_row, subtract_mean):
+    """`dl_grad_stabilize` against the torch operations of base_layer.py:266-339 evaluated in float64."""
+    torch.manual_seed(3)
+    rows, cols = 37, 5003
+    g = (torch.randn(rows, cols, device=DEV) * 0.3 + 0.05)
+    out = _ops().grad_stabilize(g, per_row, 0.7, subtract_mean, 1e-8)
+    w = g.double()
+    if subtract_mean:
+        w = w - (w.mean(dim=1, keepdim=True) if per_row else w.mean())
+    var = w.pow(2).mean(dim=1, keepdim=True) if per_row else w.pow(2).mean()
+    want = w * torch.sqrt(0.7 / (var + 1e-8))
+    np.testing.assert_allclose(out.cpu().numpy(), want.cpu().numpy(), rtol=1e-5, atol=1e-6)
+    again = _ops().grad_stabilize(g, per_row, 0.7, subtract_mean, 1e-8)
+    assert torch.equal(out, again)  # fixed order of additions
