@@ -43,6 +43,10 @@ SIGNATURES = {
     "dl_dwn_layer_fwd_planes_groups": (_I, [_P, _P, _P, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _I, _F, _P]),
     "dl_dwn_layer_bwd_groups": (_I, [_P, _P, _P, _P, _P, _I, _F, _F, _F, _P, _I, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
     "dl_dwn_layer_bwd_chain_nodes": (_I, [_P, _P, _P, _P, _P, _I, _I, _F, _P, _P, _F, _P, _I, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
+    "dl_dwn_chain_fusable": (_I, [_I, _I, _I, _I, _I, _I, _F]),
+    "dl_dwn_bwd_fused_workspace_bytes": (_Z, [_I, _I, _I, _I, _I, _I]),
+    "dl_dwn_layer_bwd_chain_fused": (_I, [_P, _P, _P, _P, _P, _I, _I, _F, _P, _P, _F, _P, _I, _P, _P, _I, _P, _P, _Z,
+                                          _I, _I, _I, _I, _I, _P]),
     "dl_dwn_stable_layer_bwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _I, _I, _I, _I, _I, _P]),
     "dl_table_sigmoid_fwd": (_I, [_P, _P, ctypes.c_longlong, _P]),
     "dl_table_sigmoid_bwd": (_I, [_P, _P, _P, ctypes.c_longlong, _P]),

@@ -427,6 +427,9 @@ __device__ __forceinline__ int dwn_quad_xor(int v) {
 // the order of additions), and the function says whether this lane is the one that adds `sum` to the bin - the
 // lowest-ranked lane of its group.  Partner hr ^ 1 ranks lower when hr is odd, partners hr ^ 2 and hr ^ 3 when hr >= 2;
 // written on booleans so that the comparisons stay lane masks in scalar registers.
+// One lane's addition into its LDS bin: read, add, write.  (The LDS float add instruction, which needs no wait in between,
+// measured three times slower here: 196 us instead of 60 for the 4096 x 8192 histogram.)
+__device__ __forceinline__ void dwn_bin_add(float *bin, float v) { *bin += v; }
 __device__ __forceinline__ bool dwn_quad_merge(unsigned a, float v, int hr, float &sum) {
     const unsigned a1 = (unsigned)dwn_quad_xor<1>((int)a), a2 = (unsigned)dwn_quad_xor<2>((int)a),
                    a3 = (unsigned)dwn_quad_xor<3>((int)a);
@@ -530,7 +533,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_transpose_hist(const float *__res
                 const float v = tile[r0 + hr][hc];  // rows past B carry 0
                 const unsigned a = atile[hc][r0 + hr];
                 float sum;
-                if (dwn_quad_merge(a, v, hr, sum)) hist[hc][a] += sum;
+                if (dwn_quad_merge(a, v, hr, sum)) dwn_bin_add(&hist[hc][a], sum);
             }
         }
     }
@@ -599,7 +602,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_hist_tiled(const float *__restric
                     const float v = vs[e];
                     const unsigned a = (aw[m] >> (8 * e)) & 0xffu;
                     float sum;
-                    if (dwn_quad_merge(a, v, hr, sum)) hist[hc][a] += sum;
+                    if (dwn_quad_merge(a, v, hr, sum)) dwn_bin_add(&hist[hc][a], sum);
                 }
             }
 #pragma unroll
@@ -799,6 +802,190 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT,
         const int b = t * 64 + r;
         if (b < B && ii < iend) __builtin_nontemporal_store(tile[ii][r], &gx[(size_t)b * I + i0 + ii]);
     }
+}
+
+// ---------------------------------------------------------------------------------
+// bwd_gx_hist: the input gradient of a chained layer, written tile-major, with the table-gradient histogram of the
+// layer IN FRONT folded in.  In a chain the input gradient of layer l + 1 is the output gradient of layer l: column i of
+// it, together with the addresses layer l saved, is all layer l's histogram needs - and here it sits in the LDS the
+// moment it is complete.  So the wavefront that has just summed its inputs' rows of a batch tile adds them into the
+// bins of those columns (the quad merge of hist_tiled) before it moves on, and the separate pass that re-reads the
+// [B, I] fp32 gradient for layer l's histogram is gone.  Bins have to live across batch tiles, so a block keeps its
+// slab and walks `tiles_per_block` tiles of its XCD (t = xcd + 8 i); it ends with its bins as one partial set
+// ([set][column][bin]), the sets are added in set order afterwards (dwn_reduce_partials): fixed order, no atomics.
+// The gather itself is dwn_bwd_gx's (O == 1, S form): the unrolled path for sixteen inputs of three entries, the
+// general loop otherwise; same order of additions.
+template <int K, int WI>
+__global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__ gyT, const uint8_t *__restrict__ addrT,
+                                                        const float *__restrict__ S, const int *__restrict__ inv_ptr,
+                                                        const int *__restrict__ inv_pos, float *__restrict__ gx,
+                                                        const uint8_t *__restrict__ prev_addrT, float *__restrict__ prev_partial,
+                                                        int I, int N, int BT, int slabs, int tiles_per_block, int Lp) {
+    constexpr int IS = 4 * WI;  // inputs per block
+    constexpr int L = 1 << K;
+    __shared__ float tile[IS][65];  // [input][row]
+    __shared__ float hist[IS][65];  // [input = column of the layer in front][bin]
+    const int xcd = blockIdx.x % DL_XCDS, q = blockIdx.x / DL_XCDS;
+    const int slab = q % slabs, grp = q / slabs;
+    const int i0 = slab * IS;
+    const int lane = threadIdx.x & 63;
+    const int wave = dl_uniform(threadIdx.x >> 6);
+    const int iend = min(IS, I - i0);
+    const int wbeg = wave * WI;
+    const int myptr = inv_ptr[min(i0 + wbeg + min(lane, WI), I)];
+    const int ebeg = __builtin_amdgcn_readlane(myptr, 0);
+    const int eend = __builtin_amdgcn_readlane(myptr, WI);
+#pragma unroll
+    for (int r = 0; r < WI; ++r) hist[wbeg + r][lane] = 0.0f;  // my columns' bins (wave-local rows of the array)
+    // histogram role of this lane: column (of my wavefront's WI) and the sixteen rows 16 hr .. 16 hr + 15 of a tile
+    const int hcl = lane >> 2, hr = lane & 3;
+    const bool hlive = hcl < WI && wbeg + hcl < iend;  // whole quads share the column
+    const int hc = wbeg + min(hcl, WI - 1);
+    const size_t hcol = (size_t)min(i0 + hc, I - 1) * 64 + hr * 16;  // my sixteen address bytes within a tile of prev_addrT
+    // step h of a tile's histogram: row 16 hr + h of my column, the quad's equal addresses merged into one addition
+    auto hist_step = [&](const float (&hv)[16], const uint4 &haw, int h) {
+        const unsigned w = h < 4 ? haw.x : h < 8 ? haw.y : h < 12 ? haw.z : haw.w;
+        const unsigned a = (w >> (8 * (h & 3))) & 0xffu;
+        float sum;
+        if (dwn_quad_merge(a, hv[h], hr, sum)) dwn_bin_add(&hist[hc][a], sum);
+    };
+    constexpr int FAN = 3;
+    bool uniform3 = false;
+    int rec3 = 0;
+    if (WI == 16) {
+        const int len = __shfl_down(myptr, 1) - myptr;  // lanes 0..15: entries of my input
+        uniform3 = __ballot(lane >= WI || len == FAN) == ~0ull;
+        if (uniform3) {
+            const int p = lane < WI * FAN ? inv_pos[ebeg + lane] : 0;
+            const int n = p / K;
+            rec3 = (n << 3) | (p - n * K);
+        }
+    }
+    const int tiles_xcd = (BT - xcd + DL_XCDS - 1) / DL_XCDS;  // tiles t = xcd + 8 i < BT
+    const int i_begin = grp * tiles_per_block, i_end = min(tiles_xcd, i_begin + tiles_per_block);
+    if (WI == 16 && uniform3) {
+        // Sixteen inputs of three entries (then every input of the wavefront exists): unrolled.  (Running a tile's
+        // histogram one tile late, from registers, between the requests of a group of entries and their use, measured
+        // slower: 247 against 238 us per launch over the deep stack - the steps cost issue slots, not latency.)
+        for (int ti = i_begin; ti < i_end; ++ti) {
+            const int t = xcd + DL_XCDS * ti;
+            const uint8_t *addr_t = addrT + (size_t)t * N * 64 + lane;
+            const float *gy_t = gyT + (size_t)t * N * 64 + lane;
+            float *gx_t = gx + ((size_t)t * I + i0 + wbeg) * 64 + lane;
+            const uint4 haw = *reinterpret_cast<const uint4 *>(prev_addrT + (size_t)t * I * 64 + hcol);
+            float acc = 0.0f;
+#pragma unroll
+            for (int s0 = 0; s0 < WI * FAN; s0 += DWN_EG) {
+                int rj[DWN_EG];
+                unsigned a[DWN_EG];
+                float g[DWN_EG], coef[DWN_EG];
+#pragma unroll
+                for (int qq = 0; qq < DWN_EG; ++qq) {
+                    const int r = __builtin_amdgcn_readlane(rec3, s0 + qq);
+                    const int rn = r >> 3;
+                    rj[qq] = r & 7;
+                    a[qq] = addr_t[(size_t)rn * 64];
+                    g[qq] = gy_t[(size_t)rn * 64];
+                    coef[qq] = S[(size_t)rn * L + (lane & (L - 1))];
+                }
+#pragma unroll
+                for (int qq = 0; qq < DWN_EG; ++qq) {
+                    const float hi = dl_lane_read(coef[qq], (int)(a[qq] | (1u << rj[qq])));
+                    const float lo = dl_lane_read(coef[qq], (int)(a[qq] & ~(1u << rj[qq])));
+                    const float term = g[qq] * (hi - lo);
+                    const int sidx = s0 + qq;  // compile-time after unrolling
+                    acc = (sidx % FAN == 0) ? 0.0f + term : acc + term;
+                    if (sidx % FAN == FAN - 1) {
+                        tile[wbeg + sidx / FAN][lane] = acc;
+                        // gx as [B/64][I][64], streamed past the L2 (which holds the rows the gather re-reads)
+                        __builtin_nontemporal_store(acc, gx_t + (size_t)(sidx / FAN) * 64);
+                    }
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            float hv[16];
+#pragma unroll
+            for (int h = 0; h < 16; ++h) hv[h] = tile[hc][hr * 16 + h];
+#pragma unroll
+            for (int h = 0; h < 16; ++h) hist_step(hv, haw, h);
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();  // the next tile overwrites the rows just read
+        }
+    } else {
+        for (int ti = i_begin; ti < i_end; ++ti) {
+            const int t = xcd + DL_XCDS * ti;
+            const uint8_t *addr_t = addrT + (size_t)t * N * 64 + lane;
+            const float *gy_t = gyT + (size_t)t * N * 64 + lane;
+            // the addresses of the layer in front for my column and rows: asked for now, used after the gather
+            const uint4 haw = *reinterpret_cast<const uint4 *>(prev_addrT + (size_t)t * I * 64 + hcol);
+#pragma unroll
+            for (int r = 0; r < WI; ++r) tile[wbeg + r][lane] = 0.0f;  // inputs nobody reads keep 0
+            float acc = 0.0f;
+            int cur = -1;
+            for (int base = ebeg; base < eend; base += 64) {
+                const int e = base + lane;
+                const bool valid = e < eend;
+                const int p = valid ? inv_pos[e] : 0;
+                int ii = 0;  // local input of entry e = number of my inputs that end at or before e
+#pragma unroll
+                for (int l = 1; l <= WI; ++l) ii += (__builtin_amdgcn_readlane(myptr, l) <= e) ? 1 : 0;
+                const int n = p / K, j = p - n * K;
+                const int rec = (n << 8) | (j << 5) | ii;
+                const int cnt = min(64, eend - base);
+                for (int s0 = 0; s0 < cnt; s0 += DWN_EG) {
+                    int rj[DWN_EG], ri[DWN_EG];
+                    unsigned a[DWN_EG];
+                    float g[DWN_EG], coef[DWN_EG];
+#pragma unroll
+                    for (int qq = 0; qq < DWN_EG; ++qq) {
+                        const int r = __builtin_amdgcn_readlane(rec, min(s0 + qq, cnt - 1));
+                        const int rn = r >> 8;
+                        rj[qq] = (r >> 5) & 7;
+                        ri[qq] = r & 31;
+                        a[qq] = addr_t[(size_t)rn * 64];
+                        g[qq] = gy_t[(size_t)rn * 64];
+                        coef[qq] = S[(size_t)rn * L + (lane & (L - 1))];
+                    }
+#pragma unroll
+                    for (int qq = 0; qq < DWN_EG; ++qq) {
+                        if (s0 + qq >= cnt) break;  // wave-uniform
+                        const float hi = dl_lane_read(coef[qq], (int)(a[qq] | (1u << rj[qq])));
+                        const float lo = dl_lane_read(coef[qq], (int)(a[qq] & ~(1u << rj[qq])));
+                        if (ri[qq] != cur) {
+                            if (cur >= 0) tile[wbeg + cur][lane] = acc;
+                            acc = 0.0f;
+                            cur = ri[qq];
+                        }
+                        acc += g[qq] * (hi - lo);
+                    }
+                }
+            }
+            if (cur >= 0) tile[wbeg + cur][lane] = acc;
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            // gx as [B/64][I][64]: my inputs, 256 B each, streamed past the L2 (which holds the rows the gather re-reads)
+#pragma unroll
+            for (int r = 0; r < WI; ++r)
+                if (wbeg + r < iend)
+                    __builtin_nontemporal_store(tile[wbeg + r][lane], &gx[((size_t)t * I + i0 + wbeg + r) * 64 + lane]);
+            // the same rows into the bins of the layer in front (rows past the batch carry 0 and add nothing)
+            if (hlive) {
+                float hv[16];
+#pragma unroll
+                for (int h = 0; h < 16; ++h) hv[h] = tile[hc][hr * 16 + h];
+#pragma unroll
+                for (int h = 0; h < 16; ++h) hist_step(hv, haw, h);
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();  // the next tile clears the rows just read
+        }
+    }
+    // my columns' bins as one partial set
+    const int set = grp * DL_XCDS + xcd;
+    float *out = prev_partial + ((size_t)set * I + i0 + wbeg) * Lp;
+    const int ncols = max(0, min(WI, iend - wbeg));
+    for (int e = lane; e < ncols * Lp; e += 64) out[e] = hist[wbeg + e / Lp][e % Lp];
 }
 
 // ---------------------------------------------------------------------------------
@@ -1016,11 +1203,50 @@ struct DwnGroupHead {
     int groups, gsize;
     float inv_tau;
 };
+// The layer in front of this one in a chain (its N_prev * 1 outputs are this layer's I inputs): with its saved addresses
+// the gather can fill that layer's table-gradient bins from the input gradient it has just summed (dwn_bwd_gx_hist).
+struct DwnFusedPrev {
+    const uint8_t *addrT;  // [B/64][I][64], what that layer's forward saved
+    float *gluts;          // [I][2^k_prev] out
+    int k;
+    float *partial;        // [sets][I][2^k_prev] scratch
+};
+__global__ __launch_bounds__(256) void dwn_build_tables(DwnTables tb) { dwn_table_block(tb, blockIdx.x); }
+// How the tiles of an XCD are shared out over the blocks of a slab.  Every group of blocks ends with a partial set of
+// bins that has to be written and summed again, so few groups: two (measured best on the deep stack: one leaves a long
+// tail of 16-tile blocks, three and more pay for their sets), more only where two would not give the chip one round of
+// blocks; at most 128 MB of partial sets.
+static inline void dwn_fused_split(int BT, int I, int k_prev, int IS, int &slabs, int &groups, int &tpb) {
+    slabs = dl_ceil_div(I, IS);
+    const int tiles_xcd = dl_ceil_div(BT, DL_XCDS);
+    const long long set_bytes = (long long)DL_XCDS * I * ((long long)4 << k_prev);
+    int by_memory = (int)((128LL << 20) / (set_bytes > 0 ? set_bytes : 1));
+    if (by_memory < 1) by_memory = 1;
+    groups = (1024 + 4 * slabs) / (DL_XCDS * slabs);  // 1024 blocks / (8 slabs), rounded
+    if (groups < 2) groups = 2;
+    if (groups > by_memory) groups = by_memory;
+    if (groups > tiles_xcd) groups = tiles_xcd;
+    if (groups < 1) groups = 1;
+    tpb = dl_ceil_div(tiles_xcd, groups);
+    groups = dl_ceil_div(tiles_xcd, tpb);
+}
+// inputs per wavefront of the fused gather: the rule of dwn_launch_gx; 0 = lists too long for it (not fused)
+static inline int dwn_fused_wi(int I, int N, int K) {
+    if ((long long)N * K >= 32LL * I) return 0;
+    return (long long)N * K >= 6LL * I ? DWN_WI_SMALL : DWN_WI;
+}
+static inline size_t dwn_fused_partial_bytes(int B, int I, int N, int k, int k_prev) {
+    const int wi = dwn_fused_wi(I, N, k);
+    if (!wi) return 0;
+    int slabs, groups, tpb;
+    dwn_fused_split(dwn_bt(B), I, k_prev, 4 * wi, slabs, groups, tpb);
+    return dl_align256((size_t)groups * DL_XCDS * I * ((size_t)4 << k_prev));
+}
 static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos, const float *luts,
                              const float *gy, int gy_tiled, float alpha, float beta, const float *scale, float *gx,
                              int gx_tiled, float *gluts, void *ws, int B, int I, int N, int k, int O, hipStream_t s,
                              const DwnGroupHead *head = nullptr, const float *alpha_n = nullptr,
-                             const float *beta_n = nullptr) {
+                             const float *beta_n = nullptr, const DwnFusedPrev *prev = nullptr) {
     const long long NO = (long long)N * O;
     const int L = 1 << k;
     const uint8_t *addrT = (const uint8_t *)saved;
@@ -1036,7 +1262,11 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
     // fixed-order sum of the histogram partials rides in the gather's launch the same way.
     DwnTables tb = {gx ? luts : nullptr, D, scale, alpha_n, beta_n, alpha, beta, (int)NO, k, O, sform ? 1 : 0};
     const dim3 hgrid(col_tiles, chunks + dl_ceil_div(dwn_table_blocks(tb), col_tiles));
-    if (head)
+    if (!gluts) {
+        // the table gradient of this layer is already there (the gather of the layer behind filled its bins): only the
+        // coefficient tables remain to be built.  gy is tile-major in that case.
+        if (dwn_table_blocks(tb)) DL_TIMED("dwn_build_tables", s, (dwn_build_tables<<<dwn_table_blocks(tb), 256, 0, s>>>(tb)));
+    } else if (head)
         DL_TIMED("dwn_bwd_hist_groups", s, (dwn_bwd_hist_tiled<true><<<hgrid, 256, 0, s>>>(
                                                gy, addrT, gluts, (int)NO, O, L, BT, tpc, partial, chunks, tb, gx ? gyT : nullptr, B,
                                                head->groups, head->gsize, head->inv_tau)));
@@ -1050,10 +1280,35 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
         DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<false><<<hgrid, 256, 0, s>>>(
                                                   gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc, partial, scale, chunks, tb)));
     // (the row-major histogram's scale is applied in the sum; the tile-major ones scale afterwards)
-    DwnReduce red = {chunks > 1 ? partial : nullptr, gluts, NO * L, chunks, (head || gy_tiled) ? nullptr : scale, L, O};
-    if (!gx && dwn_reduce_blocks(red))
+    DwnReduce red = {gluts && chunks > 1 ? partial : nullptr, gluts, NO * L, chunks, (head || gy_tiled) ? nullptr : scale, L, O};
+    const int fused_wi = prev && gx && gx_tiled && O == 1 && sform ? dwn_fused_wi(I, N, k) : 0;
+    if ((!gx || fused_wi) && dwn_reduce_blocks(red))
         DL_TIMED("dwn_reduce_partials", s, (dwn_reduce_partials<<<dwn_reduce_blocks(red), 256, 0, s>>>(red)));
-    if (gx) {
+    if (fused_wi) {
+        // the gather that also fills the bins of the layer in front
+        const float *src = gy_tiled ? gy : gyT;
+        int slabs, groups, tpb;
+        dwn_fused_split(BT, I, prev->k, 4 * fused_wi, slabs, groups, tpb);
+        const int grid = DL_XCDS * slabs * groups, Lp = 1 << prev->k;
+#define DWN_GXH(K_, WI_)                                                                                                   \
+    DL_TIMED("dwn_bwd_gx_hist", s, (dwn_bwd_gx_hist<K_, WI_><<<grid, 256, 0, s>>>(src, addrT, D, inv_ptr, inv_pos, gx, prev->addrT, \
+                                                                                  prev->partial, I, N, BT, slabs, tpb, Lp)))
+#define DWN_GXH_K(K_)                                  \
+    if (fused_wi == DWN_WI) DWN_GXH(K_, DWN_WI);       \
+    else DWN_GXH(K_, DWN_WI_SMALL)
+        switch (k) {
+            case 1: DWN_GXH_K(1); break;
+            case 2: DWN_GXH_K(2); break;
+            case 3: DWN_GXH_K(3); break;
+            case 4: DWN_GXH_K(4); break;
+            case 5: DWN_GXH_K(5); break;
+            default: DWN_GXH_K(6); break;
+        }
+#undef DWN_GXH_K
+#undef DWN_GXH
+        const DwnReduce pred = {prev->partial, prev->gluts, (long long)I * Lp, groups * DL_XCDS, nullptr, Lp, 1};
+        DL_TIMED("dwn_reduce_partials", s, (dwn_reduce_partials<<<dwn_reduce_blocks(pred), 256, 0, s>>>(pred)));
+    } else if (gx) {
         const float *src = gy_tiled ? gy : gyT;
         switch (k) {
             case 1: dwn_launch_gx<1>(src, addrT, D, inv_ptr, inv_pos, gx, B, I, N, O, sform, gx_tiled, red, s); break;
@@ -1165,6 +1420,8 @@ __global__ __launch_bounds__(256) void dwn_eval_bitsliced(const u64 *__restrict_
                                                            int B, int I, int N, int O, int BT, int tiles_per_block,
                                                            uint8_t *__restrict__ addrT = nullptr) {
     constexpr int L = 1 << K;
+    typedef unsigned u4v __attribute__((ext_vector_type(4)));
+    __shared__ u4v stage[SAVE ? 4 : 1][SAVE ? 64 * 5 : 1];  // per wavefront: 64 nodes x 64 address bytes, rows padded to 80
     const int NO = N * O;
     const int lane = threadIdx.x & 63;
     const int wave = dl_uniform(threadIdx.x >> 6);
@@ -1173,11 +1430,15 @@ __global__ __launch_bounds__(256) void dwn_eval_bitsliced(const u64 *__restrict_
     const int c = min(wc0 + lane, NO - 1);
     // truth tables of the wavefront's 64 columns: row u of the tables is read with lane = entry and voted on
     unsigned t_lo = 0u, t_hi = 0u;
-    for (int u = 0; u < 64; ++u) {
-        const int cu = min(wc0 + u, NO - 1);
-        const float v = lane < L ? luts[(size_t)cu * L + lane] : 0.0f;
-        const u64 bits = __ballot(v >= 0.5f);
-        if (lane == u) { t_lo = (unsigned)bits; t_hi = (unsigned)(bits >> 32); }
+    {
+        float tv[64];  // all 64 rows asked for at once: one trip to memory, not one per handful of rows
+#pragma unroll
+        for (int u = 0; u < 64; ++u) tv[u] = lane < L ? luts[(size_t)min(wc0 + u, NO - 1) * L + lane] : 0.0f;
+#pragma unroll
+        for (int u = 0; u < 64; ++u) {
+            const u64 bits = __ballot(tv[u] >= 0.5f);
+            if (lane == u) { t_lo = (unsigned)bits; t_hi = (unsigned)(bits >> 32); }
+        }
     }
     int off[K];  // word offsets of my inputs inside a tile's planes
 #pragma unroll
@@ -1216,26 +1477,54 @@ __global__ __launch_bounds__(256) void dwn_eval_bitsliced(const u64 *__restrict_
         const u64 valid = rows == 64 ? ~0ull : ((1ull << rows) - 1ull);
         if (wc0 + lane < NO) planes_out[(size_t)t * NO + wc0 + lane] = (((u64)vhi[0] << 32) | vlo[0]) & valid;
         if (SAVE && wc0 + lane < NO && c % O == 0) {
-            typedef unsigned u4v __attribute__((ext_vector_type(4)));
             u4v *dst = reinterpret_cast<u4v *>(addrT + ((size_t)t * N + c / O) * 64);
+            // word q = the address bytes of rows 4q .. 4q + 3.  Bit j of those four bytes: nibble q of plane j times
+            // 0x204081 has the nibble's bit r at bit 8r (no two partial products meet, so nothing carries), times 2^j
+            // puts it at bit j of byte r.  The nibbles are taken as bytes of two masked copies of the plane word (even
+            // and odd nibbles); from j = 3 on the copies carry the nibble at bits 3..6 and the constant 2^(j-3), which
+            // keeps both factors inside 24 bits.
+            unsigned word[16];
+#pragma unroll
+            for (int q = 0; q < 16; ++q) word[q] = 0u;
+#pragma unroll
+            for (int j = 0; j < K; ++j) {
+                constexpr unsigned SPREAD = 0x204081u;
+                const int sh = j >= 3 ? 3 : 0;
+                const unsigned factor = SPREAD << (j - sh), keep = 0x01010101u << j, nibbles = 0x0F0F0F0Fu << sh;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const unsigned half = h ? (unsigned)(w[j] >> 32) : (unsigned)w[j];
+                    const unsigned even = (half << sh) & nibbles, odd = ((half >> 4) << sh) & nibbles;
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) {
+                        const unsigned nib = (((q & 1) ? odd : even) >> (8 * (q >> 1))) & 0xFFu;
+                        word[h * 8 + q] |= __umul24(nib, factor) & keep;
+                    }
+                }
+            }
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
-                unsigned word[4];
-#pragma unroll
-                for (int qq = 0; qq < 4; ++qq) {
-                    const int q = q4 * 4 + qq;  // rows 4q .. 4q + 3
-                    unsigned acc = 0u;
-#pragma unroll
-                    for (int j = 0; j < K; ++j) {
-                        const unsigned half = q < 8 ? (unsigned)w[j] : (unsigned)(w[j] >> 32);
-                        const unsigned nib = (half >> (4 * (q & 7))) & 0xFu;
-                        acc |= ((nib * 0x204081u) & 0x01010101u) << j;
-                    }
-                    word[qq] = acc;
-                }
-                const u4v v = {word[0], word[1], word[2], word[3]};
-                dst[q4] = v;
+                const u4v v = {word[4 * q4], word[4 * q4 + 1], word[4 * q4 + 2], word[4 * q4 + 3]};
+                if (O == 1)
+                    stage[wave][lane * 5 + q4] = v;
+                else
+                    dst[q4] = v;
             }
+        }
+        if (SAVE && O == 1) {
+            // one output per node: the wavefront's 64 nodes own 4 KB in a row.  Through the LDS, so that every store
+            // instruction writes 1 KB of whole lines instead of a quarter of 64 lines.
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const int node = q4 * 16 + (lane >> 2);
+                const u4v v = stage[wave][node * 5 + (lane & 3)];
+                if (wc0 + node < NO)
+                    *reinterpret_cast<u4v *>(addrT + ((size_t)t * N + wc0) * 64 + (size_t)q4 * 1024 + lane * 16) = v;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
         }
 #pragma unroll
         for (int j = 0; j < K; ++j) w[j] = wn[j];
@@ -1247,7 +1536,9 @@ static void dwn_launch_eval_bitsliced(const u64 *planes, const int *idx32, const
                                       int N, int O, hipStream_t s, uint8_t *addrT = nullptr) {
     const int BT = dwn_bt(B);
     const int col_blocks = dl_ceil_div((long long)N * O, 256);
-    int chunks = col_blocks >= 2048 ? 1 : 2048 / col_blocks;  // about 2048 blocks, each long enough to repay its tables
+    // about 1024 blocks, one resident round: each repays its tables over more tiles (2048: 45 us per launch of the deep
+    // stack's training forward, 1024: 41, 4096: 53)
+    int chunks = col_blocks >= 1024 ? 1 : 1024 / col_blocks;
     if (chunks > BT) chunks = BT;
     const int tpb = dl_ceil_div(BT, chunks);
     if (addrT)
@@ -1511,4 +1802,52 @@ extern "C" int dl_dwn_layer_bwd_chain_nodes(const void *saved, const int32_t *in
     const DwnGroupHead head = {groups, gy_form == 2 ? dwn_group_size(N * O, groups) : 1, gy_form == 2 ? 1.0f / tau : 1.0f};
     return dwn_backward_fast(saved, inv_ptr, inv_pos, luts, gy, gy_form == 1, 0.0f, beta_abs_max, nullptr, gx, gx_tiled, gluts,
                              ws, B, I, N, k, O, (hipStream_t)stream, gy_form == 2 ? &head : nullptr, alpha_n, beta_n);
+}
+
+// ---- chained backward with the histogram of the layer in front folded into the gather
+// 1 when dl_dwn_layer_bwd_chain_fused can fill the table gradient of the layer in front (k_prev inputs per node, one
+// output per node) from this layer's tile-major input gradient: k <= 6 on both sides, one output per node, the compact
+// coefficient table (every |beta| <= 1/2), CSR lists short enough for the multi-input gather.
+extern "C" int dl_dwn_chain_fusable(int B, int I, int N, int k, int O, int k_prev, float beta_abs_max) {
+    if (dwn_check(B, I, N, k, O) || !dwn_fast(N, k, O) || O != 1) return 0;
+    if (k_prev <= 0 || k_prev > DL_MAX_FAST_K || !dwn_fast(I, k_prev, 1)) return 0;
+    if (!(beta_abs_max <= 0.5f)) return 0;
+    return dwn_fused_wi(I, N, k) != 0;
+}
+extern "C" size_t dl_dwn_bwd_fused_workspace_bytes(int B, int I, int N, int k, int O, int k_prev) {
+    if (!dwn_fast(N, k, O) || k_prev <= 0 || k_prev > DL_MAX_FAST_K) return 256;
+    return dl_dwn_bwd_workspace_bytes(B, I, N, k, O) + dwn_fused_partial_bytes(B, I, N, k, k_prev);
+}
+// dl_dwn_layer_bwd_chain_nodes with two options.  gluts == NULL: this layer's table gradient has already been computed
+// (by the call for the layer behind it); gy must then be tile-major (gy_form 1).  prev_saved != NULL: the layer in front
+// (I nodes of k_prev inputs, one output each; prev_saved = what its forward saved) gets its table gradient prev_gluts
+// [I, 2^k_prev] from this call; requires gx tile-major and dl_dwn_chain_fusable(...) == 1.
+extern "C" int dl_dwn_layer_bwd_chain_fused(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos,
+                                            const float *luts, const float *gy, int gy_form, int groups, float tau,
+                                            const float *alpha_n, const float *beta_n, float beta_abs_max, float *gx,
+                                            int gx_tiled, float *gluts, const void *prev_saved, int k_prev,
+                                            float *prev_gluts, void *ws, size_t ws_bytes, int B, int I, int N, int k, int O,
+                                            void *stream) {
+    if (!saved || !luts || !gy || !ws || !alpha_n || !beta_n) return DL_ERR_NULL;
+    if (gx && (!inv_ptr || !inv_pos)) return DL_ERR_NULL;
+    if (gy_form < 0 || gy_form > 2) return DL_ERR_SHAPE;
+    if (!gluts && gy_form != 1) return DL_ERR_SHAPE;
+    if (!gluts && !gx) return DL_ERR_NULL;  // nothing to do
+    int rc = dwn_check(B, I, N, k, O);
+    if (rc) return rc;
+    if (gy_form == 2 && (groups <= 0 || !(tau > 0.0f))) return DL_ERR_SHAPE;
+    if (!dwn_fast(N, k, O)) return DL_ERR_UNSUPPORTED;
+    DwnFusedPrev prev = {nullptr, nullptr, 0, nullptr};
+    size_t need = dl_dwn_bwd_workspace_bytes(B, I, N, k, O);
+    if (prev_saved) {
+        if (!prev_gluts || !gx || !gx_tiled) return DL_ERR_NULL;
+        if (!dl_dwn_chain_fusable(B, I, N, k, O, k_prev, beta_abs_max)) return DL_ERR_UNSUPPORTED;
+        prev = DwnFusedPrev{(const uint8_t *)prev_saved, prev_gluts, k_prev, (float *)((char *)ws + need)};
+        need = dl_dwn_bwd_fused_workspace_bytes(B, I, N, k, O, k_prev);
+    }
+    if (ws_bytes < need) return DL_ERR_WORKSPACE;
+    const DwnGroupHead head = {groups, gy_form == 2 ? dwn_group_size(N * O, groups) : 1, gy_form == 2 ? 1.0f / tau : 1.0f};
+    return dwn_backward_fast(saved, inv_ptr, inv_pos, luts, gy, gy_form == 1, 0.0f, beta_abs_max, nullptr, gx, gx_tiled, gluts,
+                             ws, B, I, N, k, O, (hipStream_t)stream, gy_form == 2 ? &head : nullptr, alpha_n, beta_n,
+                             prev_saved ? &prev : nullptr);
 }

@@ -279,6 +279,7 @@ class DWNStackFunction(torch.autograd.Function):
         lib = nat.lib()
         g, tiled = _f32(gy), 0
         grads = [None] * n
+        have_tables = [False] * n  # table gradient already produced by the call for the layer behind
         for l in range(n - 1, -1, -1):
             B, I, N, k, O = dims = ctx.dims_all[l]
             plan = ctx.plans[l]
@@ -294,7 +295,8 @@ class DWNStackFunction(torch.autograd.Function):
                     gx = torch.empty(lib.dl_dwn_tiled_bytes(B, I) // 4, dtype=torch.float32, device=g.device)
                 else:
                     gx = torch.empty((B, I), dtype=torch.float32, device=g.device)
-            grads[l] = torch.empty_like(luts[l])
+            if not have_tables[l]:
+                grads[l] = torch.empty_like(luts[l])
             ws = _bytes(lib.dl_dwn_bwd_workspace_bytes(*dims), g.device)
             headed = l == n - 1 and ctx.head is not None
             groups, tau = ctx.head if headed else (1, 1.0)
@@ -302,11 +304,24 @@ class DWNStackFunction(torch.autograd.Function):
                 alpha_n, beta_n, beta_max = ctx.scalars[l]
                 alpha_n = _f32(alpha_n.detach()).reshape(-1).expand(N).contiguous()
                 beta_n = _f32(beta_n.detach()).reshape(-1).expand(N).contiguous()
-                nat.check(lib.dl_dwn_layer_bwd_chain_nodes(nat.ptr(saved[l]), nat.ptr(plan.inv_ptr), nat.ptr(plan.inv_pos),
-                                                           nat.ptr(luts[l]), nat.ptr(g), 2 if headed else tiled, int(groups),
-                                                           float(tau), nat.ptr(alpha_n), nat.ptr(beta_n), float(beta_max),
-                                                           nat.ptr(gx), gx_tiled, nat.ptr(grads[l]), nat.ptr(ws), ws.numel(),
-                                                           *dims, nat.stream()))
+                # the gather of this layer can fill the table gradient of the layer in front as it goes: that layer's
+                # own pass over its [B, N] output gradient is then left out
+                k_prev = ctx.dims_all[l - 1][3] if l > 0 else 0
+                fuse = (l > 0 and gx_tiled == 1 and ctx.dims_all[l - 1][4] == 1
+                        and lib.dl_dwn_chain_fusable(*dims, k_prev, float(beta_max)) == 1)
+                if have_tables[l] and gx is None:  # nothing left to compute for this layer
+                    g = None
+                    continue
+                if fuse:
+                    grads[l - 1] = torch.empty_like(luts[l - 1])
+                    have_tables[l - 1] = True
+                    ws = _bytes(lib.dl_dwn_bwd_fused_workspace_bytes(*dims, k_prev), g.device)
+                nat.check(lib.dl_dwn_layer_bwd_chain_fused(
+                    nat.ptr(saved[l]), nat.ptr(plan.inv_ptr), nat.ptr(plan.inv_pos), nat.ptr(luts[l]), nat.ptr(g),
+                    2 if headed else tiled, int(groups), float(tau), nat.ptr(alpha_n), nat.ptr(beta_n), float(beta_max),
+                    nat.ptr(gx), gx_tiled, None if have_tables[l] else nat.ptr(grads[l]),
+                    nat.ptr(saved[l - 1]) if fuse else None, k_prev, nat.ptr(grads[l - 1]) if fuse else None,
+                    nat.ptr(ws), ws.numel(), *dims, nat.stream()))
                 g, tiled = gx, gx_tiled
                 continue
             alpha, beta = ctx.scalars[l]

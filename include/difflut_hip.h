@@ -166,6 +166,24 @@ int dl_dwn_layer_bwd_chain_nodes(const void *saved, const int32_t *inv_ptr, cons
                                  const float *gy, int gy_form, int groups, float tau, const float *alpha_n,
                                  const float *beta_n, float beta_abs_max, float *gx, int gx_tiled, float *gluts,
                                  void *ws, size_t ws_bytes, int B, int I, int N, int k, int O, void *stream);
+/* dl_dwn_layer_bwd_chain_nodes that can also produce the table gradient of the layer IN FRONT.  In a chain this layer's
+ * input gradient is that layer's output gradient (random_layer.py:306-340 run layer by layer), so the gather adds every
+ * batch tile it has just summed into that layer's bins, and that layer's own pass over its [B, N] output gradient is
+ * left out.  No counterpart in the reference, which runs each node's backward on its own (efd_cuda_kernel.cu:195-331).
+ *   prev_saved (nullable): what the forward of the layer in front saved (I nodes of k_prev inputs, ONE output each);
+ *     prev_gluts [I, 2^k_prev] then receives its table gradient.  Needs gx tile-major (gx_tiled = 1) and
+ *     dl_dwn_chain_fusable(...) == 1 (k, k_prev <= DL_MAX_FAST_K, O == 1, beta_abs_max <= 1/2, N k < 32 I);
+ *     workspace dl_dwn_bwd_fused_workspace_bytes.  Bins are summed per block and then in block order: reproducible,
+ *     but a different order of additions than dl_dwn_layer_bwd_tiled's for the same table.
+ *   gluts (nullable): NULL when this layer's own table gradient has already been produced by the call for the layer
+ *     behind it; gy must then be tile-major (gy_form 1) and gx non-NULL. */
+int dl_dwn_chain_fusable(int B, int I, int N, int k, int O, int k_prev, float beta_abs_max);
+size_t dl_dwn_bwd_fused_workspace_bytes(int B, int I, int N, int k, int O, int k_prev);
+int dl_dwn_layer_bwd_chain_fused(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos, const float *luts,
+                                 const float *gy, int gy_form, int groups, float tau, const float *alpha_n,
+                                 const float *beta_n, float beta_abs_max, float *gx, int gx_tiled, float *gluts,
+                                 const void *prev_saved, int k_prev, float *prev_gluts, void *ws, size_t ws_bytes,
+                                 int B, int I, int N, int k, int O, void *stream);
 /* The eval forward below with a workspace (dl_dwn_eval_workspace_bytes): the same result for any input, and
  * the bit-plane kernels' speed when every input value is exactly 0 or 1 (checked on the device while packing;
  * no host synchronisation - both kernels are launched and one returns at once). */

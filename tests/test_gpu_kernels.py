@@ -126,6 +126,114 @@ def test_dwn_backward_tile_major_output_all_list_lengths(shape):
     np.testing.assert_allclose(results[1][1].cpu().numpy(), wl, rtol=1e-5, atol=2e-4)
 
 
+FUSED_CHAIN_SHAPES = [  # (B, I0, k_front, I = nodes of the front layer, N, k)
+    (200, 40, 6, 128, 64, 6),    # every input read three times: the unrolled path; fewer batch tiles than XCDs
+    (1100, 64, 4, 256, 128, 6),  # 18 batch tiles: XCDs with three and with two; 16 bins per column
+    (333, 30, 5, 100, 45, 5),    # lists of two and three entries, a last slab of 36 inputs
+    (130, 16, 3, 20, 40, 6),     # twelve entries per input: four inputs per wavefront
+    (64, 12, 6, 70, 35, 2),
+]
+
+
+@pytest.mark.parametrize("shape", FUSED_CHAIN_SHAPES)
+def test_dwn_chained_backward_fills_the_table_gradient_of_the_layer_in_front(shape):
+    """dl_dwn_layer_bwd_chain_fused against the two calls it replaces (the layer's own backward with a tile-major
+    input gradient, then the front layer's histogram over that gradient) and against the oracle.  The input
+    gradient and the layer's own table gradient keep their order of additions: bit-equal.  The front layer's
+    bins are summed per block and then over blocks: rtol 1e-5 with a floor of 2e-5 of the largest bin."""
+    from difflut_amd import _native as nat
+    B, I0, kf, I, N, k = shape
+    ops = _ops()
+    lib = nat.lib()
+    x0, idx_f, luts_f, _ = make_case(sum(shape) % 991, B, I0, I, kf, 1, lo=0.0)
+    _, idx, luts, gy = make_case(sum(shape) % 983, B, I, N, k, 1)
+    plan_f = ops.MappingPlan(dev(idx_f, torch.int32), I0)
+    plan = ops.MappingPlan(dev(idx, torch.int32), I)
+    front, dims = (B, I0, I, kf, 1), (B, I, N, k, 1)
+    rng = np.random.default_rng(7)
+    alpha_n = dev(rng.uniform(0.1, 0.6, N).astype(np.float32))
+    beta_n = dev(rng.uniform(-0.4, 0.45, N).astype(np.float32))
+    beta_max = float(beta_n.abs().max())
+
+    def forward(xin, pl, tab, d):
+        y = torch.empty(d[0], d[2], device=DEV)
+        saved = torch.empty(lib.dl_dwn_saved_bytes(*d), dtype=torch.uint8, device=DEV)
+        ws = torch.empty(lib.dl_dwn_fwd_workspace_bytes(*d), dtype=torch.uint8, device=DEV)
+        nat.check(lib.dl_dwn_layer_fwd(xin.data_ptr(), pl.idx32.data_ptr(), tab.data_ptr(), y.data_ptr(), saved.data_ptr(),
+                                       ws.data_ptr(), ws.numel(), *d, nat.stream()))
+        return y, saved
+
+    lf, ld, gd = dev(luts_f), dev(luts), dev(gy.reshape(B, N))
+    h, saved_f = forward(dev(x0), plan_f, lf, front)
+    _, saved = forward(h, plan, ld, dims)
+    BT = (B + 63) // 64
+    assert lib.dl_dwn_chain_fusable(*dims, kf, beta_max) == 1
+    # the two calls
+    ws = torch.empty(lib.dl_dwn_bwd_workspace_bytes(*dims), dtype=torch.uint8, device=DEV)
+    gx_ref = torch.zeros(BT * I * 64, device=DEV)
+    gl_ref = torch.empty_like(ld)
+    nat.check(lib.dl_dwn_layer_bwd_chain_nodes(saved.data_ptr(), plan.inv_ptr.data_ptr(), plan.inv_pos.data_ptr(), ld.data_ptr(),
+                                               gd.data_ptr(), 0, 1, 1.0, alpha_n.data_ptr(), beta_n.data_ptr(), beta_max,
+                                               gx_ref.data_ptr(), 1, gl_ref.data_ptr(), ws.data_ptr(), ws.numel(), *dims,
+                                               nat.stream()))
+    wsf = torch.empty(lib.dl_dwn_bwd_workspace_bytes(*front), dtype=torch.uint8, device=DEV)
+    glf_ref = torch.empty_like(lf)
+    nat.check(lib.dl_dwn_layer_bwd_tiled(saved_f.data_ptr(), None, None, lf.data_ptr(), gx_ref.data_ptr(), 1, 0.3, 0.3, None, 0,
+                                         glf_ref.data_ptr(), wsf.data_ptr(), wsf.numel(), *front, nat.stream()))
+    # the one call
+    wsx = torch.empty(lib.dl_dwn_bwd_fused_workspace_bytes(*dims, kf), dtype=torch.uint8, device=DEV)
+    gx = torch.zeros(BT * I * 64, device=DEV)
+    gl = torch.empty_like(ld)
+    glf = torch.full_like(lf, 7.0)
+    nat.check(lib.dl_dwn_layer_bwd_chain_fused(saved.data_ptr(), plan.inv_ptr.data_ptr(), plan.inv_pos.data_ptr(), ld.data_ptr(),
+                                               gd.data_ptr(), 0, 1, 1.0, alpha_n.data_ptr(), beta_n.data_ptr(), beta_max,
+                                               gx.data_ptr(), 1, gl.data_ptr(), saved_f.data_ptr(), kf, glf.data_ptr(),
+                                               wsx.data_ptr(), wsx.numel(), *dims, nat.stream()))
+    assert torch.equal(gx, gx_ref)
+    assert torch.equal(gl, gl_ref)
+    floor = 2e-5 * float(glf_ref.abs().max())
+    np.testing.assert_allclose(glf.cpu().numpy(), glf_ref.cpu().numpy(), rtol=1e-5, atol=floor)
+    # the oracle on the front layer, fed with the input gradient just computed (rows past B carry zeros)
+    rows = gx.view(BT, I, 64).permute(0, 2, 1).reshape(BT * 64, I)[:B].cpu().numpy()
+    _, want = orc.dwn_layer_backward(x0, idx_f, luts_f, rows.reshape(B, I, 1), np.float32(0.3), np.float32(0.3))
+    np.testing.assert_allclose(glf.cpu().numpy(), want, rtol=1e-5, atol=floor)
+    # the layer's own table gradient already there: gy tile-major, no gluts
+    gyT = torch.zeros(BT * 64, N, device=DEV)
+    gyT[:B] = gd
+    gyT = gyT.view(BT, 64, N).permute(0, 2, 1).contiguous()
+    gx2 = torch.zeros_like(gx)
+    glf2 = torch.empty_like(lf)
+    nat.check(lib.dl_dwn_layer_bwd_chain_fused(saved.data_ptr(), plan.inv_ptr.data_ptr(), plan.inv_pos.data_ptr(), ld.data_ptr(),
+                                               gyT.data_ptr(), 1, 1, 1.0, alpha_n.data_ptr(), beta_n.data_ptr(), beta_max,
+                                               gx2.data_ptr(), 1, None, saved_f.data_ptr(), kf, glf2.data_ptr(),
+                                               wsx.data_ptr(), wsx.numel(), *dims, nat.stream()))
+    assert torch.equal(gx2, gx_ref)
+    assert torch.equal(glf2, glf)  # fixed order of additions: the same bits on every call
+    # and without a front layer it is the plain chained backward
+    gx3 = torch.zeros_like(gx)
+    nat.check(lib.dl_dwn_layer_bwd_chain_fused(saved.data_ptr(), plan.inv_ptr.data_ptr(), plan.inv_pos.data_ptr(), ld.data_ptr(),
+                                               gyT.data_ptr(), 1, 1, 1.0, alpha_n.data_ptr(), beta_n.data_ptr(), beta_max,
+                                               gx3.data_ptr(), 1, None, None, 0, None, ws.data_ptr(), ws.numel(), *dims,
+                                               nat.stream()))
+    assert torch.equal(gx3, gx_ref)
+
+
+def test_dwn_chained_backward_refuses_what_it_cannot_fuse():
+    from difflut_amd import _native as nat
+    lib = nat.lib()
+    assert lib.dl_dwn_chain_fusable(64, 9, 64, 6, 1, 6, 0.3) == 0    # 42 entries per input: the one-input gather
+    assert lib.dl_dwn_chain_fusable(64, 128, 64, 6, 1, 6, 0.75) == 0  # |beta| > 1/2: the other coefficient form
+    assert lib.dl_dwn_chain_fusable(64, 128, 64, 6, 2, 6, 0.3) == 0   # two outputs per node
+    assert lib.dl_dwn_chain_fusable(64, 128, 64, 6, 1, 7, 0.3) == 0   # front layer on the generic path
+    assert lib.dl_dwn_chain_fusable(64, 128, 64, 6, 1, 4, 0.3) == 1
+    buf = torch.zeros(1 << 16, device=DEV)
+    rc = lib.dl_dwn_layer_bwd_chain_fused(buf.data_ptr(), buf.data_ptr(), buf.data_ptr(), buf.data_ptr(), buf.data_ptr(), 0, 1,
+                                          1.0, buf.data_ptr(), buf.data_ptr(), 0.75, buf.data_ptr(), 1, buf.data_ptr(),
+                                          buf.data_ptr(), 6, buf.data_ptr(), buf.data_ptr(), buf.numel() * 4, 64, 128, 64, 6, 1,
+                                          nat.stream())
+    assert rc == -3  # DL_ERR_UNSUPPORTED
+
+
 def test_dwn_threshold_is_inclusive_and_exact_at_half():
     ops = _ops()
     x = np.array([[0.5, 0.49999997, 0.50000006, 0.0, 1.0, -3.0]], dtype=np.float32)
