@@ -867,6 +867,13 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
         // Sixteen inputs of three entries (then every input of the wavefront exists): unrolled.  (Running a tile's
         // histogram one tile late, from registers, between the requests of a group of entries and their use, measured
         // slower: 247 against 238 us per launch over the deep stack - the steps cost issue slots, not latency.)
+        // The block keeps its entries over all its tiles, so the coefficient rows of the wavefront's 48 entries stay in
+        // registers: one load per entry and block instead of one per entry and tile, and the 256 B x N of coefficient
+        // rows no longer share the L2 with the rows of the tiles.
+        float coef[WI * FAN];
+#pragma unroll
+        for (int e = 0; e < WI * FAN; ++e)
+            coef[e] = S[(size_t)(__builtin_amdgcn_readlane(rec3, e) >> 3) * L + (lane & (L - 1))];
         for (int ti = i_begin; ti < i_end; ++ti) {
             const int t = xcd + DL_XCDS * ti;
             const uint8_t *addr_t = addrT + (size_t)t * N * 64 + lane;
@@ -878,7 +885,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
             for (int s0 = 0; s0 < WI * FAN; s0 += DWN_EG) {
                 int rj[DWN_EG];
                 unsigned a[DWN_EG];
-                float g[DWN_EG], coef[DWN_EG];
+                float g[DWN_EG];
 #pragma unroll
                 for (int qq = 0; qq < DWN_EG; ++qq) {
                     const int r = __builtin_amdgcn_readlane(rec3, s0 + qq);
@@ -886,12 +893,11 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
                     rj[qq] = r & 7;
                     a[qq] = addr_t[(size_t)rn * 64];
                     g[qq] = gy_t[(size_t)rn * 64];
-                    coef[qq] = S[(size_t)rn * L + (lane & (L - 1))];
                 }
 #pragma unroll
                 for (int qq = 0; qq < DWN_EG; ++qq) {
-                    const float hi = dl_lane_read(coef[qq], (int)(a[qq] | (1u << rj[qq])));
-                    const float lo = dl_lane_read(coef[qq], (int)(a[qq] & ~(1u << rj[qq])));
+                    const float hi = dl_lane_read(coef[s0 + qq], (int)(a[qq] | (1u << rj[qq])));
+                    const float lo = dl_lane_read(coef[s0 + qq], (int)(a[qq] & ~(1u << rj[qq])));
                     const float term = g[qq] * (hi - lo);
                     const int sidx = s0 + qq;  // compile-time after unrolling
                     acc = (sidx % FAN == 0) ? 0.0f + term : acc + term;
