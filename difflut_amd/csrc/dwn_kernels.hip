@@ -811,7 +811,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT,
 // moment it is complete.  So the wavefront that has just summed its inputs' rows of a batch tile adds them into the
 // bins of those columns (the quad merge of hist_tiled) before it moves on, and the separate pass that re-reads the
 // [B, I] fp32 gradient for layer l's histogram is gone.  Bins have to live across batch tiles, so a block keeps its
-// slab and walks `tiles_per_block` tiles of its XCD (t = xcd + 8 i); it ends with its bins as one partial set
+// slab and walks `tiles_per_block` tiles of its class (t = cls + ncls i); it ends with its bins as one partial set
 // ([set][column][bin]), the sets are added in set order afterwards (dwn_reduce_partials): fixed order, no atomics.
 // The gather itself is dwn_bwd_gx's (O == 1, S form): the unrolled path for sixteen inputs of three entries, the
 // general loop otherwise; same order of additions.
@@ -820,13 +820,18 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
                                                         const float *__restrict__ S, const int *__restrict__ inv_ptr,
                                                         const int *__restrict__ inv_pos, float *__restrict__ gx,
                                                         const uint8_t *__restrict__ prev_addrT, float *__restrict__ prev_partial,
-                                                        int I, int N, int BT, int slabs, int tiles_per_block, int Lp) {
+                                                        int I, int N, int BT, int slabs, int split, int part,
+                                                        int tiles_per_block, int Lp) {
     constexpr int IS = 4 * WI;  // inputs per block
     constexpr int L = 1 << K;
     __shared__ float tile[IS][65];  // [input][row]
     __shared__ float hist[IS][65];  // [input = column of the layer in front][bin]
+    // `split` XCDs share a class of tiles, each with its own part of the slabs (at most as many as stay resident on an
+    // XCD): the blocks that read a tile on one XCD then all run at once, and a tile's rows pass through that L2 once.
     const int xcd = blockIdx.x % DL_XCDS, q = blockIdx.x / DL_XCDS;
-    const int slab = q % slabs, grp = q / slabs;
+    const int sub = xcd % split, cls = xcd / split, ncls = DL_XCDS / split;
+    const int slab = sub * part + q % part, grp = q / part;
+    if (slab >= slabs) return;
     const int i0 = slab * IS;
     const int lane = threadIdx.x & 63;
     const int wave = dl_uniform(threadIdx.x >> 6);
@@ -861,8 +866,8 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
             rec3 = (n << 3) | (p - n * K);
         }
     }
-    const int tiles_xcd = (BT - xcd + DL_XCDS - 1) / DL_XCDS;  // tiles t = xcd + 8 i < BT
-    const int i_begin = grp * tiles_per_block, i_end = min(tiles_xcd, i_begin + tiles_per_block);
+    const int tiles_cls = (BT - cls + ncls - 1) / ncls;  // tiles t = cls + ncls i < BT
+    const int i_begin = grp * tiles_per_block, i_end = min(tiles_cls, i_begin + tiles_per_block);
     if (WI == 16 && uniform3) {
         // Sixteen inputs of three entries (then every input of the wavefront exists): unrolled.  (Running a tile's
         // histogram one tile late, from registers, between the requests of a group of entries and their use, measured
@@ -875,7 +880,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
         for (int e = 0; e < WI * FAN; ++e)
             coef[e] = S[(size_t)(__builtin_amdgcn_readlane(rec3, e) >> 3) * L + (lane & (L - 1))];
         for (int ti = i_begin; ti < i_end; ++ti) {
-            const int t = xcd + DL_XCDS * ti;
+            const int t = cls + ncls * ti;
             const uint8_t *addr_t = addrT + (size_t)t * N * 64 + lane;
             const float *gy_t = gyT + (size_t)t * N * 64 + lane;
             float *gx_t = gx + ((size_t)t * I + i0 + wbeg) * 64 + lane;
@@ -920,7 +925,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
         }
     } else {
         for (int ti = i_begin; ti < i_end; ++ti) {
-            const int t = xcd + DL_XCDS * ti;
+            const int t = cls + ncls * ti;
             const uint8_t *addr_t = addrT + (size_t)t * N * 64 + lane;
             const float *gy_t = gyT + (size_t)t * N * 64 + lane;
             // the addresses of the layer in front for my column and rows: asked for now, used after the gather
@@ -988,7 +993,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
         }
     }
     // my columns' bins as one partial set
-    const int set = grp * DL_XCDS + xcd;
+    const int set = grp * ncls + cls;
     float *out = prev_partial + ((size_t)set * I + i0 + wbeg) * Lp;
     const int ncols = max(0, min(WI, iend - wbeg));
     for (int e = lane; e < ncols * Lp; e += 64) out[e] = hist[wbeg + e / Lp][e % Lp];
@@ -1218,23 +1223,32 @@ struct DwnFusedPrev {
     float *partial;        // [sets][I][2^k_prev] scratch
 };
 __global__ __launch_bounds__(256) void dwn_build_tables(DwnTables tb) { dwn_table_block(tb, blockIdx.x); }
-// How the tiles of an XCD are shared out over the blocks of a slab.  Every group of blocks ends with a partial set of
-// bins that has to be written and summed again, so few groups: two (measured best on the deep stack: one leaves a long
-// tail of 16-tile blocks, three and more pay for their sets), more only where two would not give the chip one round of
-// blocks; at most 128 MB of partial sets.
-static inline void dwn_fused_split(int BT, int I, int k_prev, int IS, int &slabs, int &groups, int &tpb) {
-    slabs = dl_ceil_div(I, IS);
-    const int tiles_xcd = dl_ceil_div(BT, DL_XCDS);
-    const long long set_bytes = (long long)DL_XCDS * I * ((long long)4 << k_prev);
-    int by_memory = (int)((128LL << 20) / (set_bytes > 0 ? set_bytes : 1));
-    if (by_memory < 1) by_memory = 1;
-    groups = (1024 + 4 * slabs) / (DL_XCDS * slabs);  // 1024 blocks / (8 slabs), rounded
-    if (groups < 2) groups = 2;
-    if (groups > by_memory) groups = by_memory;
-    if (groups > tiles_xcd) groups = tiles_xcd;
-    if (groups < 1) groups = 1;
-    tpb = dl_ceil_div(tiles_xcd, groups);
-    groups = dl_ceil_div(tiles_xcd, tpb);
+// How the fused gather is laid over the chip.  An XCD keeps DWN_RESIDENT of its blocks at a time; blocks that read the
+// same tile through the same L2 should all be among them, or the tile's rows are fetched once per round of blocks.  So
+// `split` XCDs (1, 2, 4 or 8) share a class of tiles, each taking `part` <= DWN_RESIDENT of the slabs, and where a part
+// is smaller than that, `groups` blocks per slab share the class's tiles (each ends with a partial set of bins that has
+// to be written and summed again; at most 128 MB of them).  One round of blocks, every block the same number of tiles.
+#define DWN_RESIDENT 128  // 32 CUs x 4 blocks (33 KB of LDS each)
+struct DwnFusedSplit {
+    int slabs, split, part, groups, tpb, sets;
+};
+static inline DwnFusedSplit dwn_fused_split(int BT, int I, int k_prev, int IS) {
+    DwnFusedSplit f;
+    f.slabs = dl_ceil_div(I, IS);
+    f.split = 1;
+    while (f.split < DL_XCDS && dl_ceil_div(f.slabs, f.split) > DWN_RESIDENT) f.split *= 2;
+    f.part = dl_ceil_div(f.slabs, f.split);
+    const int ncls = DL_XCDS / f.split, tiles_cls = dl_ceil_div(BT, ncls);
+    const long long set_bytes = (long long)I * ((long long)4 << k_prev);
+    int by_memory = (int)((128LL << 20) / (set_bytes * ncls > 0 ? set_bytes * ncls : 1));
+    f.groups = DWN_RESIDENT / f.part;
+    if (f.groups > by_memory) f.groups = by_memory;
+    if (f.groups > tiles_cls) f.groups = tiles_cls;
+    if (f.groups < 1) f.groups = 1;
+    f.tpb = dl_ceil_div(tiles_cls, f.groups);
+    f.groups = dl_ceil_div(tiles_cls, f.tpb);
+    f.sets = f.groups * ncls;
+    return f;
 }
 // inputs per wavefront of the fused gather: the rule of dwn_launch_gx; 0 = lists too long for it (not fused)
 static inline int dwn_fused_wi(int I, int N, int K) {
@@ -1244,9 +1258,8 @@ static inline int dwn_fused_wi(int I, int N, int K) {
 static inline size_t dwn_fused_partial_bytes(int B, int I, int N, int k, int k_prev) {
     const int wi = dwn_fused_wi(I, N, k);
     if (!wi) return 0;
-    int slabs, groups, tpb;
-    dwn_fused_split(dwn_bt(B), I, k_prev, 4 * wi, slabs, groups, tpb);
-    return dl_align256((size_t)groups * DL_XCDS * I * ((size_t)4 << k_prev));
+    const DwnFusedSplit f = dwn_fused_split(dwn_bt(B), I, k_prev, 4 * wi);
+    return dl_align256((size_t)f.sets * I * ((size_t)4 << k_prev));
 }
 static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos, const float *luts,
                              const float *gy, int gy_tiled, float alpha, float beta, const float *scale, float *gx,
@@ -1293,12 +1306,11 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
     if (fused_wi) {
         // the gather that also fills the bins of the layer in front
         const float *src = gy_tiled ? gy : gyT;
-        int slabs, groups, tpb;
-        dwn_fused_split(BT, I, prev->k, 4 * fused_wi, slabs, groups, tpb);
-        const int grid = DL_XCDS * slabs * groups, Lp = 1 << prev->k;
+        const DwnFusedSplit f = dwn_fused_split(BT, I, prev->k, 4 * fused_wi);
+        const int grid = DL_XCDS * f.part * f.groups, Lp = 1 << prev->k;
 #define DWN_GXH(K_, WI_)                                                                                                   \
     DL_TIMED("dwn_bwd_gx_hist", s, (dwn_bwd_gx_hist<K_, WI_><<<grid, 256, 0, s>>>(src, addrT, D, inv_ptr, inv_pos, gx, prev->addrT, \
-                                                                                  prev->partial, I, N, BT, slabs, tpb, Lp)))
+                                                                                  prev->partial, I, N, BT, f.slabs, f.split, f.part, f.tpb, Lp)))
 #define DWN_GXH_K(K_)                                  \
     if (fused_wi == DWN_WI) DWN_GXH(K_, DWN_WI);       \
     else DWN_GXH(K_, DWN_WI_SMALL)
@@ -1312,7 +1324,7 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
         }
 #undef DWN_GXH_K
 #undef DWN_GXH
-        const DwnReduce pred = {prev->partial, prev->gluts, (long long)I * Lp, groups * DL_XCDS, nullptr, Lp, 1};
+        const DwnReduce pred = {prev->partial, prev->gluts, (long long)I * Lp, f.sets, nullptr, Lp, 1};
         DL_TIMED("dwn_reduce_partials", s, (dwn_reduce_partials<<<dwn_reduce_blocks(pred), 256, 0, s>>>(pred)));
     } else if (gx) {
         const float *src = gy_tiled ? gy : gyT;
