@@ -3,7 +3,9 @@
 Same registry names, constructors and autograd behaviour as the `difflut` package for
 RandomLayer, LearnableLayer, DWNNode, ProbabilisticNode, ThermometerEncoder and GroupSum;
 the arithmetic runs in hand-written HIP kernels (difflut_amd/lib/libdifflut_hip.so, C ABI
-in include/difflut_hip.h).  Tensors must live on a ROCm device; there is no CPU path.
+in include/difflut_hip.h) for tensors on a ROCm device.  Tensors on the CPU take plain-torch
+operators of the same arithmetic (difflut_amd/cpu_ops.py), as the reference's operators do
+when `x.is_cuda` is false.
 """
 from .encoder.base_encoder import BaseEncoder
 from .layers.base_layer import BaseLUTLayer

@@ -1,7 +1,8 @@
 """ctypes binding of libdifflut_hip.so (the C ABI declared in include/difflut_hip.h).
 
-There is no CPU fallback: if the library is missing or the tensors are not on a
-ROCm device the calls raise.  Tensors are passed as raw device pointers together
+The library never falls back: if it is missing, or a tensor handed to it is not on a
+ROCm device, the calls raise (CPU tensors are dispatched to plain-torch operators before
+they get here, difflut_amd/ops.py).  Tensors are passed as raw device pointers together
 with torch's current HIP stream; outputs and workspaces are allocated by the
 caller with torch's caching allocator.
 """
@@ -100,7 +101,7 @@ def lib():
         if not is_built():
             raise RuntimeError(
                 f"HIP extension not available: {LIB_PATH} is missing. Build it with "
-                "`python -m difflut_amd.build` (needs hipcc); there is no CPU fallback.")
+                "`python -m difflut_amd.build` (needs hipcc); device tensors have no other path.")
         handle = ctypes.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(handle, name)
@@ -127,7 +128,7 @@ def require_device(*tensors):
         if t is not None and not t.is_cuda:
             raise RuntimeError(
                 "difflut_amd kernels run on ROCm devices only; got a tensor on "
-                f"'{t.device}'. Move the module and its inputs to 'cuda' (there is no CPU path).")
+                f"'{t.device}'. All tensors of one call must be on the same ROCm device (or all on the CPU).")
 
 
 def profile_enable(on=True):

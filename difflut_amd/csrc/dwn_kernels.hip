@@ -1859,6 +1859,7 @@ extern "C" int dl_dwn_layer_bwd_chain_fused(const void *saved, const int32_t *in
     size_t need = dl_dwn_bwd_workspace_bytes(B, I, N, k, O);
     if (prev_saved) {
         if (!prev_gluts || !gx || !gx_tiled) return DL_ERR_NULL;
+        if ((uintptr_t)prev_saved & 15) return DL_ERR_UNSUPPORTED;  // its addresses are read sixteen at a time
         if (!dl_dwn_chain_fusable(B, I, N, k, O, k_prev, beta_abs_max)) return DL_ERR_UNSUPPORTED;
         prev = DwnFusedPrev{(const uint8_t *)prev_saved, prev_gluts, k_prev, (float *)((char *)ws + need)};
         need = dl_dwn_bwd_fused_workspace_bytes(B, I, N, k, O, k_prev);

@@ -170,7 +170,8 @@ int dl_dwn_layer_bwd_chain_nodes(const void *saved, const int32_t *inv_ptr, cons
  * input gradient is that layer's output gradient (random_layer.py:306-340 run layer by layer), so the gather adds every
  * batch tile it has just summed into that layer's bins, and that layer's own pass over its [B, N] output gradient is
  * left out.  No counterpart in the reference, which runs each node's backward on its own (efd_cuda_kernel.cu:195-331).
- *   prev_saved (nullable): what the forward of the layer in front saved (I nodes of k_prev inputs, ONE output each);
+ *   prev_saved (nullable, 16-byte aligned): what the forward of the layer in front saved (I nodes of k_prev inputs, ONE
+ *     output each);
  *     prev_gluts [I, 2^k_prev] then receives its table gradient.  Needs gx tile-major (gx_tiled = 1) and
  *     dl_dwn_chain_fusable(...) == 1 (k, k_prev <= DL_MAX_FAST_K, O == 1, beta_abs_max <= 1/2, N k < 32 I);
  *     workspace dl_dwn_bwd_fused_workspace_bytes.  Bins are summed per block and then in block order: reproducible,
