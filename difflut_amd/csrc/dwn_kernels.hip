@@ -269,7 +269,36 @@ struct DwnReduce {
     const float *scale;
     int L, O;
 };
+// From DWN_SLICED_CHUNKS chunks on (few columns, many batch tiles: a convolutional level, a narrow last layer) a thread
+// that added all chunks of its four elements would run alone for tens of microseconds.  Then sixteen lanes share four
+// elements: lane slice s adds chunks s, s + 16, ... in order, and the sixteen sums are joined by a butterfly over the
+// lanes - another fixed order.
+#define DWN_SLICED_CHUNKS 64
+__device__ __forceinline__ bool dwn_reduce_sliced(const DwnReduce &r) { return r.chunks >= DWN_SLICED_CHUNKS && r.NOL % 4 == 0; }
 __device__ __forceinline__ void dwn_reduce_block(const DwnReduce &r, int block) {
+    if (dwn_reduce_sliced(r)) {
+        const int lane = threadIdx.x & 63, col = lane & 3, slice = lane >> 2;
+        const long long e4 = (((long long)block * 4 + (threadIdx.x >> 6)) * 4 + col) * 4;  // a wavefront: 16 elements
+        const bool live = e4 < r.NOL;
+        float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (live)
+            for (int ch = slice; ch < r.chunks; ch += 16) {
+                const float4 v = *reinterpret_cast<const float4 *>(r.partial + (size_t)ch * r.NOL + e4);
+                sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+            }
+#pragma unroll
+        for (int off = 4; off < 64; off <<= 1) {
+            sum.x += __shfl_xor(sum.x, off); sum.y += __shfl_xor(sum.y, off);
+            sum.z += __shfl_xor(sum.z, off); sum.w += __shfl_xor(sum.w, off);
+        }
+        if (live && slice == 0) {
+            const float sc[4] = {r.scale ? r.scale[((e4 + 0) / r.L) / r.O] : 1.0f, r.scale ? r.scale[((e4 + 1) / r.L) / r.O] : 1.0f,
+                                 r.scale ? r.scale[((e4 + 2) / r.L) / r.O] : 1.0f, r.scale ? r.scale[((e4 + 3) / r.L) / r.O] : 1.0f};
+            r.gluts[e4] = sum.x * sc[0], r.gluts[e4 + 1] = sum.y * sc[1];  // the caller's array: no alignment assumed
+            r.gluts[e4 + 2] = sum.z * sc[2], r.gluts[e4 + 3] = sum.w * sc[3];
+        }
+        return;
+    }
     const long long e4 = ((long long)block * 256 + threadIdx.x) * 4;
     if (e4 >= r.NOL) return;
     float sum[4] = {0.f, 0.f, 0.f, 0.f};
@@ -291,7 +320,10 @@ __device__ __forceinline__ void dwn_reduce_block(const DwnReduce &r, int block) 
     for (int q = 0; q < 4; ++q)
         if (e4 + q < r.NOL) r.gluts[e4 + q] = sum[q] * (r.scale ? r.scale[((e4 + q) / r.L) / r.O] : 1.0f);
 }
-static inline int dwn_reduce_blocks(const DwnReduce &r) { return r.partial ? dl_ceil_div(r.NOL, 1024) : 0; }
+static inline int dwn_reduce_blocks(const DwnReduce &r) {
+    if (!r.partial) return 0;
+    return r.chunks >= DWN_SLICED_CHUNKS && r.NOL % 4 == 0 ? dl_ceil_div(r.NOL, 64) : dl_ceil_div(r.NOL, 1024);
+}
 __global__ __launch_bounds__(256) void dwn_reduce_partials(DwnReduce r) { dwn_reduce_block(r, blockIdx.x); }
 
 // ---------------------------------------------------------------------------------
@@ -821,7 +853,9 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
                                                         const int *__restrict__ inv_pos, float *__restrict__ gx,
                                                         const uint8_t *__restrict__ prev_addrT, float *__restrict__ prev_partial,
                                                         int I, int N, int BT, int slabs, int split, int part,
-                                                        int tiles_per_block, int Lp) {
+                                                        int tiles_per_block, int Lp, int gather_blocks, DwnReduce red) {
+    // the fixed-order sum of this layer's own histogram partials rides behind the gather's blocks
+    if ((int)blockIdx.x >= gather_blocks) return dwn_reduce_block(red, (int)blockIdx.x - gather_blocks);
     constexpr int IS = 4 * WI;  // inputs per block
     constexpr int L = 1 << K;
     __shared__ float tile[IS][65];  // [input][row]
@@ -1301,16 +1335,16 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
     // (the row-major histogram's scale is applied in the sum; the tile-major ones scale afterwards)
     DwnReduce red = {gluts && chunks > 1 ? partial : nullptr, gluts, NO * L, chunks, (head || gy_tiled) ? nullptr : scale, L, O};
     const int fused_wi = prev && gx && gx_tiled && O == 1 && sform ? dwn_fused_wi(I, N, k) : 0;
-    if ((!gx || fused_wi) && dwn_reduce_blocks(red))
+    if (!gx && dwn_reduce_blocks(red))
         DL_TIMED("dwn_reduce_partials", s, (dwn_reduce_partials<<<dwn_reduce_blocks(red), 256, 0, s>>>(red)));
     if (fused_wi) {
         // the gather that also fills the bins of the layer in front
         const float *src = gy_tiled ? gy : gyT;
         const DwnFusedSplit f = dwn_fused_split(BT, I, prev->k, 4 * fused_wi);
-        const int grid = DL_XCDS * f.part * f.groups, Lp = 1 << prev->k;
+        const int gather_blocks = DL_XCDS * f.part * f.groups, grid = gather_blocks + dwn_reduce_blocks(red), Lp = 1 << prev->k;
 #define DWN_GXH(K_, WI_)                                                                                                   \
     DL_TIMED("dwn_bwd_gx_hist", s, (dwn_bwd_gx_hist<K_, WI_><<<grid, 256, 0, s>>>(src, addrT, D, inv_ptr, inv_pos, gx, prev->addrT, \
-                                                                                  prev->partial, I, N, BT, f.slabs, f.split, f.part, f.tpb, Lp)))
+                                                                                  prev->partial, I, N, BT, f.slabs, f.split, f.part, f.tpb, Lp, gather_blocks, red)))
 #define DWN_GXH_K(K_)                                  \
     if (fused_wi == DWN_WI) DWN_GXH(K_, DWN_WI);       \
     else DWN_GXH(K_, DWN_WI_SMALL)
