@@ -60,10 +60,10 @@ __global__ __launch_bounds__(256) void dwn_pack_planes(const float *__restrict__
         const int rows = min(DWN_PACK_ROWS, B - r0);  // <= 0 for pieces past the batch
         const float *base = x + (size_t)r0 * I + i0;
         unsigned acc[VEC];
-    #pragma unroll
+#pragma unroll
         for (int v = 0; v < VEC; ++v) acc[v] = 0u;
         if (rows == DWN_PACK_ROWS) {
-    #pragma unroll
+#pragma unroll
             for (int r = 0; r < DWN_PACK_ROWS; ++r) {
                 const float *src = base + (size_t)r * I;
                 if constexpr (VEC == 4) {
@@ -84,7 +84,7 @@ __global__ __launch_bounds__(256) void dwn_pack_planes(const float *__restrict__
             }
         } else {
             for (int r = 0; r < rows; ++r) {
-    #pragma unroll
+#pragma unroll
                 for (int v = 0; v < VEC; ++v) {
                     const float val = base[(size_t)r * I + v];
                     acc[v] |= (val >= 0.5f ? 1u : 0u) << r;
@@ -93,7 +93,7 @@ __global__ __launch_bounds__(256) void dwn_pack_planes(const float *__restrict__
             }
         }
         unsigned short *out = reinterpret_cast<unsigned short *>(planes + (size_t)t * I + i0) + piece;
-    #pragma unroll
+#pragma unroll
         for (int v = 0; v < VEC; ++v) out[v * PIECES] = (unsigned short)acc[v];
     }
     if (CHECK && odd) *all_binary = 0;  // every writer stores the same value
@@ -847,7 +847,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT,
 // ([set][column][bin]), the sets are added in set order afterwards (dwn_reduce_partials): fixed order, no atomics.
 // The gather itself is dwn_bwd_gx's (O == 1, S form): the unrolled path for sixteen inputs of three entries, the
 // general loop otherwise; same order of additions.
-template <int K, int WI>
+template <int K, int WI, int FAN>
 __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__ gyT, const uint8_t *__restrict__ addrT,
                                                         const float *__restrict__ S, const int *__restrict__ inv_ptr,
                                                         const int *__restrict__ inv_pos, float *__restrict__ gx,
@@ -888,10 +888,11 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
         float sum;
         if (dwn_quad_merge(a, hv[h], hr, sum)) dwn_bin_add(&hist[hc][a], sum);
     };
-    constexpr int FAN = 3;
+    // FAN > 0: the host found N K = FAN I, which is what a mapping built from whole permutations of the inputs gives -
+    // every input read exactly FAN times; checked per wavefront, anything else takes the general loop.
     bool uniform3 = false;
     int rec3 = 0;
-    if (WI == 16) {
+    if constexpr (FAN > 0) {
         const int len = __shfl_down(myptr, 1) - myptr;  // lanes 0..15: entries of my input
         uniform3 = __ballot(lane >= WI || len == FAN) == ~0ull;
         if (uniform3) {
@@ -902,62 +903,65 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
     }
     const int tiles_cls = (BT - cls + ncls - 1) / ncls;  // tiles t = cls + ncls i < BT
     const int i_begin = grp * tiles_per_block, i_end = min(tiles_cls, i_begin + tiles_per_block);
-    if (WI == 16 && uniform3) {
-        // Sixteen inputs of three entries (then every input of the wavefront exists): unrolled.  (Running a tile's
-        // histogram one tile late, from registers, between the requests of a group of entries and their use, measured
-        // slower: 247 against 238 us per launch over the deep stack - the steps cost issue slots, not latency.)
-        // The block keeps its entries over all its tiles, so the coefficient rows of the wavefront's 48 entries stay in
-        // registers: one load per entry and block instead of one per entry and tile, and the 256 B x N of coefficient
-        // rows no longer share the L2 with the rows of the tiles.
-        float coef[WI * FAN];
+    if constexpr (FAN > 0) {
+        if (uniform3) {
+            // Sixteen inputs of FAN entries each (then every input of the wavefront exists): unrolled.  (Running a tile's
+            // histogram one tile late, from registers, between the requests of a group of entries and their use, measured
+            // slower: 247 against 238 us per launch over the deep stack - the steps cost issue slots, not latency.)
+            // The block keeps its entries over all its tiles, so the coefficient rows of the wavefront's 16 FAN entries
+            // stay in registers: one load per entry and block instead of one per entry and tile, and the 256 B x N of
+            // coefficient rows no longer share the L2 with the rows of the tiles.
+            float coef[FAN > 0 ? WI * FAN : 1];
 #pragma unroll
-        for (int e = 0; e < WI * FAN; ++e)
-            coef[e] = S[(size_t)(__builtin_amdgcn_readlane(rec3, e) >> 3) * L + (lane & (L - 1))];
-        for (int ti = i_begin; ti < i_end; ++ti) {
-            const int t = cls + ncls * ti;
-            const uint8_t *addr_t = addrT + (size_t)t * N * 64 + lane;
-            const float *gy_t = gyT + (size_t)t * N * 64 + lane;
-            float *gx_t = gx + ((size_t)t * I + i0 + wbeg) * 64 + lane;
-            const uint4 haw = *reinterpret_cast<const uint4 *>(prev_addrT + (size_t)t * I * 64 + hcol);
-            float acc = 0.0f;
+            for (int e = 0; e < WI * FAN; ++e)
+                coef[e] = S[(size_t)(__builtin_amdgcn_readlane(rec3, e) >> 3) * L + (lane & (L - 1))];
+            for (int ti = i_begin; ti < i_end; ++ti) {
+                const int t = cls + ncls * ti;
+                const uint8_t *addr_t = addrT + (size_t)t * N * 64 + lane;
+                const float *gy_t = gyT + (size_t)t * N * 64 + lane;
+                float *gx_t = gx + ((size_t)t * I + i0 + wbeg) * 64 + lane;
+                const uint4 haw = *reinterpret_cast<const uint4 *>(prev_addrT + (size_t)t * I * 64 + hcol);
+                float acc = 0.0f;
 #pragma unroll
-            for (int s0 = 0; s0 < WI * FAN; s0 += DWN_EG) {
-                int rj[DWN_EG];
-                unsigned a[DWN_EG];
-                float g[DWN_EG];
+                for (int s0 = 0; s0 < WI * FAN; s0 += DWN_EG) {
+                    int rj[DWN_EG];
+                    unsigned a[DWN_EG];
+                    float g[DWN_EG];
 #pragma unroll
-                for (int qq = 0; qq < DWN_EG; ++qq) {
-                    const int r = __builtin_amdgcn_readlane(rec3, s0 + qq);
-                    const int rn = r >> 3;
-                    rj[qq] = r & 7;
-                    a[qq] = addr_t[(size_t)rn * 64];
-                    g[qq] = gy_t[(size_t)rn * 64];
-                }
+                    for (int qq = 0; qq < DWN_EG; ++qq) {
+                        const int r = __builtin_amdgcn_readlane(rec3, s0 + qq);
+                        const int rn = r >> 3;
+                        rj[qq] = r & 7;
+                        a[qq] = addr_t[(size_t)rn * 64];
+                        g[qq] = gy_t[(size_t)rn * 64];
+                    }
 #pragma unroll
-                for (int qq = 0; qq < DWN_EG; ++qq) {
-                    const float hi = dl_lane_read(coef[s0 + qq], (int)(a[qq] | (1u << rj[qq])));
-                    const float lo = dl_lane_read(coef[s0 + qq], (int)(a[qq] & ~(1u << rj[qq])));
-                    const float term = g[qq] * (hi - lo);
-                    const int sidx = s0 + qq;  // compile-time after unrolling
-                    acc = (sidx % FAN == 0) ? 0.0f + term : acc + term;
-                    if (sidx % FAN == FAN - 1) {
-                        tile[wbeg + sidx / FAN][lane] = acc;
-                        // gx as [B/64][I][64], streamed past the L2 (which holds the rows the gather re-reads)
-                        __builtin_nontemporal_store(acc, gx_t + (size_t)(sidx / FAN) * 64);
+                    for (int qq = 0; qq < DWN_EG; ++qq) {
+                        const float hi = dl_lane_read(coef[s0 + qq], (int)(a[qq] | (1u << rj[qq])));
+                        const float lo = dl_lane_read(coef[s0 + qq], (int)(a[qq] & ~(1u << rj[qq])));
+                        const float term = g[qq] * (hi - lo);
+                        const int sidx = s0 + qq;  // compile-time after unrolling
+                        acc = (sidx % FAN == 0) ? 0.0f + term : acc + term;
+                        if (sidx % FAN == FAN - 1) {
+                            tile[wbeg + sidx / FAN][lane] = acc;
+                            // gx as [B/64][I][64], streamed past the L2 (which holds the rows the gather re-reads)
+                            __builtin_nontemporal_store(acc, gx_t + (size_t)(sidx / FAN) * 64);
+                        }
                     }
                 }
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                float hv[16];
+#pragma unroll
+                for (int h = 0; h < 16; ++h) hv[h] = tile[hc][hr * 16 + h];
+#pragma unroll
+                for (int h = 0; h < 16; ++h) hist_step(hv, haw, h);
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                __builtin_amdgcn_wave_barrier();  // the next tile overwrites the rows just read
             }
-            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            float hv[16];
-#pragma unroll
-            for (int h = 0; h < 16; ++h) hv[h] = tile[hc][hr * 16 + h];
-#pragma unroll
-            for (int h = 0; h < 16; ++h) hist_step(hv, haw, h);
-            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-            __builtin_amdgcn_wave_barrier();  // the next tile overwrites the rows just read
-        }
-    } else {
+    }
+    }
+    if (!(FAN > 0 && uniform3)) {
         for (int ti = i_begin; ti < i_end; ++ti) {
             const int t = cls + ncls * ti;
             const uint8_t *addr_t = addrT + (size_t)t * N * 64 + lane;
@@ -1025,6 +1029,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
             __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
             __builtin_amdgcn_wave_barrier();  // the next tile clears the rows just read
         }
+    
     }
     // my columns' bins as one partial set
     const int set = grp * ncls + cls;
@@ -1341,13 +1346,17 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
         // the gather that also fills the bins of the layer in front
         const float *src = gy_tiled ? gy : gyT;
         const DwnFusedSplit f = dwn_fused_split(BT, I, prev->k, 4 * fused_wi);
+        const int fan = (long long)N * k % I == 0 ? (int)((long long)N * k / I) : 0;  // every input read `fan` times?
         const int gather_blocks = DL_XCDS * f.part * f.groups, grid = gather_blocks + dwn_reduce_blocks(red), Lp = 1 << prev->k;
-#define DWN_GXH(K_, WI_)                                                                                                   \
-    DL_TIMED("dwn_bwd_gx_hist", s, (dwn_bwd_gx_hist<K_, WI_><<<grid, 256, 0, s>>>(src, addrT, D, inv_ptr, inv_pos, gx, prev->addrT, \
+#define DWN_GXH(K_, WI_, FAN_)                                                                                                \
+    DL_TIMED("dwn_bwd_gx_hist", s, (dwn_bwd_gx_hist<K_, WI_, FAN_><<<grid, 256, 0, s>>>(src, addrT, D, inv_ptr, inv_pos, gx, prev->addrT, \
                                                                                   prev->partial, I, N, BT, f.slabs, f.split, f.part, f.tpb, Lp, gather_blocks, red)))
-#define DWN_GXH_K(K_)                                  \
-    if (fused_wi == DWN_WI) DWN_GXH(K_, DWN_WI);       \
-    else DWN_GXH(K_, DWN_WI_SMALL)
+#define DWN_GXH_K(K_)                                                \
+    if (fused_wi != DWN_WI) DWN_GXH(K_, DWN_WI_SMALL, 0);            \
+    else if (fan == 1) DWN_GXH(K_, DWN_WI, 1);                       \
+    else if (fan == 2) DWN_GXH(K_, DWN_WI, 2);                       \
+    else if (fan == 3) DWN_GXH(K_, DWN_WI, 3);                       \
+    else DWN_GXH(K_, DWN_WI, 0)
         switch (k) {
             case 1: DWN_GXH_K(1); break;
             case 2: DWN_GXH_K(2); break;

@@ -131,7 +131,8 @@ FUSED_CHAIN_SHAPES = [  # (B, I0, k_front, I = nodes of the front layer, N, k)
     (1100, 64, 4, 256, 128, 6),  # 18 batch tiles: XCDs with three and with two; 16 bins per column
     (333, 30, 5, 100, 45, 5),    # lists of two and three entries, a last slab of 36 inputs
     (130, 16, 3, 20, 40, 6),     # twelve entries per input: four inputs per wavefront
-    (64, 12, 6, 70, 35, 2),
+    (64, 12, 6, 70, 35, 2),      # every input read once
+    (150, 20, 4, 96, 32, 6),     # every input read twice
 ]
 
 
