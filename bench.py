@@ -96,15 +96,16 @@ def stack_bytes(B, F, nbits, widths, k, train):
     fraction of the roofline cannot exceed 1): raw features in; every layer's input once written and once read as
     bit-planes (1 bit per value); tables read; logits.  Training adds: the saved address of every (node, row), one
     byte, written forward and read by the histogram and by the gather; the fp32 gradient with respect to every hidden
-    activation, written once and read twice (histogram, gather) in tile-major form; the gradient of the logits; and
-    nine passes over the tables in all (forward, backward, gradient, Adam read p/g/m/v, write p/m/v)."""
+    activation, written once in tile-major form and read once (the gather that reads it also fills the histogram of the
+    layer in front); the gradient of the logits; and nine passes over the tables in all (forward, backward, gradient,
+    Adam read p/g/m/v, write p/m/v)."""
     ins = [F * nbits] + widths[:-1]
     tables = sum(widths) * (1 << k) * 4
     planes = sum(ins) * B // 8
     nbytes = B * F * 4 + 2 * planes + tables + B * 10 * 4
     if train:
         nbytes += 3 * B * sum(widths)                   # saved addresses: written, read twice
-        nbytes += 3 * 4 * B * sum(widths[:-1])          # hidden-activation gradients: written, read twice
+        nbytes += 2 * 4 * B * sum(widths[:-1])          # hidden-activation gradients: written, read once
         nbytes += 2 * B * 10 * 4 + 8 * tables
     return nbytes
 
@@ -269,7 +270,7 @@ def run_stack(args):
            "value": evals / (ms * 1e-3), "unit": "node-evals/s", "ms_per_step": ms, "dtype": "f32",
            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
            "vs_baseline": None, "data": "synthetic",
-           "config": {"workload": args.workload, "batch": B, "features": F, "layers": widths, "k": k, "optimizer": "torch.optim.Adam(fused=True)",
+           "config": {"workload": args.workload, "batch": B, "features": F, "layers": widths, "k": k, "optimizer": "difflut_amd.utils.BankAdam (Adam, one launch over the table banks)",
                       "execution": "layer by layer" if args.layer_by_layer else "chained (DWNStack)"},
            "roofline_step": {"bound": "hbm", "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                              "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes_per_step": nbytes},
