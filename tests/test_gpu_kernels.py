@@ -235,6 +235,50 @@ def test_dwn_chained_backward_refuses_what_it_cannot_fuse():
     assert rc == -3  # DL_ERR_UNSUPPORTED
 
 
+@pytest.mark.parametrize("shape", [(300, 12, 128, 6, 1), (1300, 7, 80, 6, 1), (90, 5, 64, 5, 1)])
+def test_dwn_backward_tile_major_output_uneven_long_lists(shape):
+    """Inputs read by 40 to 90 nodes each, drawn independently (lists of very different lengths, some beyond what the
+    gather for long lists keeps in registers): the tile-major input gradient against the row-major one of the same
+    entry point (same terms in the same order: bit-equal) and against the oracle."""
+    from difflut_amd import _native as nat
+    B, I, N, k, O = shape
+    ops = _ops()
+    lib = nat.lib()
+    rng = np.random.default_rng(sum(shape))
+    x = rng.random((B, I)).astype(np.float32)
+    idx = rng.integers(0, I, (N, k)).astype(np.int64)
+    idx[:, 0] = np.where(rng.random(N) < 0.5, 0, idx[:, 0])  # input 0 is read far more often than the others
+    luts = rng.uniform(-1, 1, (N, O, 1 << k)).astype(np.float32)
+    gy = rng.standard_normal((B, N, O)).astype(np.float32)
+    plan = ops.MappingPlan(dev(idx, torch.int32), I)
+    alpha, beta = 0.5 * 0.75 ** (k - 1), 1.0 / 3.0
+    dims = (B, I, N, k, O)
+    xd, ld, gd = dev(x), dev(luts), dev(gy.reshape(B, N * O))
+    y = torch.empty(B, N * O, device=DEV)
+    saved = torch.empty(lib.dl_dwn_saved_bytes(*dims), dtype=torch.uint8, device=DEV)
+    wf = torch.empty(lib.dl_dwn_fwd_workspace_bytes(*dims), dtype=torch.uint8, device=DEV)
+    wb = torch.empty(lib.dl_dwn_bwd_workspace_bytes(*dims), dtype=torch.uint8, device=DEV)
+    nat.check(lib.dl_dwn_layer_fwd(xd.data_ptr(), plan.idx32.data_ptr(), ld.data_ptr(), y.data_ptr(), saved.data_ptr(),
+                                   wf.data_ptr(), wf.numel(), *dims, nat.stream()))
+    BT = (B + 63) // 64
+    results = []
+    for tiled in (0, 1):
+        gx = torch.zeros(BT * I * 64 if tiled else B * I, device=DEV)
+        gl = torch.empty_like(ld)
+        nat.check(lib.dl_dwn_layer_bwd_tiled(saved.data_ptr(), plan.inv_ptr.data_ptr(), plan.inv_pos.data_ptr(), ld.data_ptr(),
+                                             gd.data_ptr(), 0, alpha, beta, gx.data_ptr(), tiled, gl.data_ptr(), wb.data_ptr(),
+                                             wb.numel(), *dims, nat.stream()))
+        results.append((gx, gl))
+    row_major = results[0][0].view(B, I)
+    tile_major = results[1][0].view(BT, I, 64).permute(0, 2, 1).reshape(BT * 64, I)[:B]
+    assert torch.equal(tile_major, row_major)
+    assert torch.equal(results[0][1], results[1][1])
+    wx, wl = orc.dwn_layer_backward(x, idx, luts, gy, np.float32(alpha), np.float32(beta))
+    # up to ~100 terms of size alpha*|gy|*|D| per input: rtol 1e-5, floor 2e-5
+    np.testing.assert_allclose(row_major.cpu().numpy(), wx, rtol=1e-5, atol=2e-5)
+    np.testing.assert_allclose(results[1][1].cpu().numpy(), wl, rtol=1e-5, atol=2e-4)
+
+
 def test_dwn_threshold_is_inclusive_and_exact_at_half():
     ops = _ops()
     x = np.array([[0.5, 0.49999997, 0.50000006, 0.0, 1.0, -3.0]], dtype=np.float32)
