@@ -133,6 +133,7 @@ FUSED_CHAIN_SHAPES = [  # (B, I0, k_front, I = nodes of the front layer, N, k)
     (130, 16, 3, 20, 40, 6),     # twelve entries per input: four inputs per wavefront
     (64, 12, 6, 70, 35, 2),      # every input read once
     (150, 20, 4, 96, 32, 6),     # every input read twice
+    (200, 24, 5, 64, 32, 6),     # three reads per input on average only (see the test)
 ]
 
 
@@ -148,6 +149,9 @@ def test_dwn_chained_backward_fills_the_table_gradient_of_the_layer_in_front(sha
     lib = nat.lib()
     x0, idx_f, luts_f, _ = make_case(sum(shape) % 991, B, I0, I, kf, 1, lo=0.0)
     _, idx, luts, gy = make_case(sum(shape) % 983, B, I, N, k, 1)
+    if shape == FUSED_CHAIN_SHAPES[-1]:
+        # N k = 3 I, but drawn independently: the lists are uneven although the host sees a whole fan-in
+        idx = np.random.default_rng(5).integers(0, I, (N, k)).astype(np.int64)
     plan_f = ops.MappingPlan(dev(idx_f, torch.int32), I0)
     plan = ops.MappingPlan(dev(idx, torch.int32), I)
     front, dims = (B, I0, I, kf, 1), (B, I, N, k, 1)
