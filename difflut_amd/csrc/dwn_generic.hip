@@ -59,6 +59,54 @@ __global__ __launch_bounds__(256) void dwn_generic_bwd_gx(const float *__restric
     gx[gid] = acc;
 }
 
+// The EFD weights alpha * beta^h are a product over the inputs, so the 2^k-term sum per (row, entry) above factors: with
+// the table smoothed along every input once, S[a] = alpha / (1 - beta) * sum_kappa lut[kappa] beta^popc(a ^ kappa), the
+// gradient term of slot j at address a is S[a | bit j] - S[a & ~bit j] (the S form of the k <= 6 path).  One block per
+// table: the table in LDS as doubles, k butterfly passes (v <- v + beta * v[a ^ bit m]), one rounding to float.
+// Amplifies rounding by (1 + |beta|)^k / (1 - beta): used for |beta| <= 1/2 only.
+__global__ __launch_bounds__(256) void dwn_generic_smooth(const float *__restrict__ luts, float *__restrict__ S, float alpha,
+                                                           float beta, const float *__restrict__ alpha_n,
+                                                           const float *__restrict__ beta_n, int K, int O) {
+    extern __shared__ double tab[];
+    const int L = 1 << K;
+    const size_t c = blockIdx.x;
+    const double al = alpha_n ? (double)alpha_n[c / O] : (double)alpha, be = beta_n ? (double)beta_n[c / O] : (double)beta;
+    for (int a = threadIdx.x; a < L; a += 256) tab[a] = (double)luts[c * L + a];
+    __syncthreads();
+    for (int m = 0; m < K; ++m) {
+        for (int a = threadIdx.x; a < L; a += 256) {
+            if (a & (1 << m)) continue;  // this thread updates the pair (a, a | bit m)
+            const double lo = tab[a], hi = tab[a | (1 << m)];
+            tab[a] = lo + be * hi;
+            tab[a | (1 << m)] = hi + be * lo;
+        }
+        __syncthreads();
+    }
+    for (int a = threadIdx.x; a < L; a += 256) S[c * L + a] = (float)(al / (1.0 - be) * tab[a]);
+}
+
+// the input gradient from the smoothed tables: per (row, input) the entries of the input in CSR order
+__global__ __launch_bounds__(256) void dwn_generic_bwd_gx_smooth(const float *__restrict__ x, const int *__restrict__ idx32,
+                                                                  const int *__restrict__ inv_ptr,
+                                                                  const int *__restrict__ inv_pos, const float *__restrict__ S,
+                                                                  const float *__restrict__ gy, float *__restrict__ gx, int B,
+                                                                  int I, int N, int K, int O) {
+    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= (long long)B * I) return;
+    const int b = (int)(gid / I), i = (int)(gid % I);
+    float acc = 0.0f;
+    for (int e = inv_ptr[i]; e < inv_ptr[i + 1]; ++e) {
+        const int p = inv_pos[e];
+        const int n = p / K, j = p - n * K;
+        const unsigned a = dwn_addr_generic(x + (size_t)b * I, idx32 + (size_t)n * K, K);
+        for (int d = 0; d < O; ++d) {
+            const float *row = S + (((size_t)n * O + d) << K);
+            acc += gy[((size_t)b * N + n) * O + d] * (row[a | (1u << j)] - row[a & ~(1u << j)]);
+        }
+    }
+    gx[gid] = acc;
+}
+
 __global__ __launch_bounds__(256) void dwn_generic_bwd_luts(const float *__restrict__ x, const int *__restrict__ idx32,
                                                              const float *__restrict__ gy, const float *__restrict__ scale,
                                                              float *__restrict__ gluts, int B, int I, int N, int K, int O) {
@@ -105,12 +153,24 @@ int dwn_generic_forward(const float *x, const int *idx32, const float *luts, flo
     return dl_launch_status();
 }
 
+size_t dwn_generic_smooth_bytes(int N, int k, int O) { return ((size_t)N * O << k) * sizeof(float); }
+
 int dwn_generic_backward(const float *x, const int *idx32, const int *inv_ptr, const int *inv_pos, const float *luts,
                          const float *gy, float alpha, float beta, const float *scale, float *gx, float *gluts, int B, int I,
-                         int N, int k, int O, hipStream_t s, const float *alpha_n, const float *beta_n) {
+                         int N, int k, int O, hipStream_t s, const float *alpha_n, const float *beta_n, float beta_abs_max,
+                         void *ws, size_t ws_bytes) {
     const long long NO = (long long)N * O;
     dwn_generic_zero<<<dl_ceil_div(NO << k, 256), 256, 0, s>>>(gluts, NO << k);
     dwn_generic_bwd_luts<<<dl_ceil_div((long long)B * NO, 256), 256, 0, s>>>(x, idx32, gy, scale, gluts, B, I, N, k, O);
+    // EFD weights with every |beta| <= 1/2 and room for the smoothed tables: two loads per (row, entry, output)
+    // instead of a 2^k-term sum
+    if (gx && !scale && beta_abs_max <= 0.5f && k <= 12 && ws && ws_bytes >= dwn_generic_smooth_bytes(N, k, O)) {  // 2^k doubles of LDS
+        float *S = (float *)ws;
+        dwn_generic_smooth<<<(unsigned)NO, 256, sizeof(double) << k, s>>>(luts, S, alpha, beta, alpha_n, beta_n, k, O);
+        dwn_generic_bwd_gx_smooth<<<dl_ceil_div((long long)B * I, 256), 256, 0, s>>>(x, idx32, inv_ptr, inv_pos, S, gy, gx, B,
+                                                                                   I, N, k, O);
+        return dl_launch_status();
+    }
     if (gx)
         dwn_generic_bwd_gx<<<dl_ceil_div((long long)B * I, 256), 256, 0, s>>>(x, idx32, inv_ptr, inv_pos, luts, gy, alpha,
                                                                             beta, scale, gx, B, I, N, k, O, alpha_n, beta_n);

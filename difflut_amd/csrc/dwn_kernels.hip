@@ -1097,7 +1097,7 @@ extern "C" size_t dl_dwn_fwd_workspace_bytes(int B, int I, int N, int k, int O) 
 extern "C" size_t dl_dwn_bwd_workspace_bytes(int B, int I, int N, int k, int O) {
     (void)I;
     return dwn_fast(N, k, O) ? dwn_table_bytes(N, k, O) + dwn_gyT_bytes(B, N, O) + dwn_partial_bytes(B, N, k, O)
-                             : 256;
+                             : dl_align256(dwn_generic_smooth_bytes(N, k, O));  // k > 6: the smoothed tables
 }
 
 template <int K>
@@ -1397,7 +1397,8 @@ extern "C" int dl_dwn_layer_bwd(const float *x, const void *saved, const int32_t
     hipStream_t s = (hipStream_t)stream;
     if (!dwn_fast(N, k, O)) {
         if (!x) return DL_ERR_NULL;
-        return dwn_generic_backward(x, idx32, inv_ptr, inv_pos, luts, gy, alpha, beta, nullptr, gx, gluts, B, I, N, k, O, s);
+        return dwn_generic_backward(x, idx32, inv_ptr, inv_pos, luts, gy, alpha, beta, nullptr, gx, gluts, B, I, N, k, O, s,
+                                    nullptr, nullptr, fabsf(beta), ws, ws_bytes);
     }
     if (!saved || !ws) return DL_ERR_NULL;
     if (ws_bytes < dl_dwn_bwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;
@@ -1418,7 +1419,7 @@ extern "C" int dl_dwn_layer_bwd_nodes(const float *x, const void *saved, const i
     if (!dwn_fast(N, k, O)) {
         if (!x) return DL_ERR_NULL;
         return dwn_generic_backward(x, idx32, inv_ptr, inv_pos, luts, gy, 0.0f, 0.0f, nullptr, gx, gluts, B, I, N, k, O, s,
-                                    alpha_n, beta_n);
+                                    alpha_n, beta_n, beta_abs_max, ws, ws_bytes);
     }
     if (!saved || !ws) return DL_ERR_NULL;
     if (ws_bytes < dl_dwn_bwd_workspace_bytes(B, I, N, k, O)) return DL_ERR_WORKSPACE;

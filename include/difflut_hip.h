@@ -109,7 +109,10 @@ int dl_dwn_layer_fwd_static(const float *x, const int32_t *idx32, const float *l
  *                 sum_kappa s(kappa_j) luts[n,d,kappa] beta^popc((addr ^ kappa) & ~(1<<j))
  *   gluts[n,d,e] = sum_b [addr(b,n) = e] gy[b,n,d]
  * gx may be null (input does not need a gradient); gx and gluts are overwritten.
- * x is only read when k > DL_MAX_FAST_K (then `saved` is unused) and may be null otherwise. */
+ * x is only read when k > DL_MAX_FAST_K (then `saved` is unused) and may be null otherwise.  For k > DL_MAX_FAST_K the
+ * workspace is optional (ws may be null): with dl_dwn_bwd_workspace_bytes of it, |beta| <= 1/2 and k <= 12 the input
+ * gradient is taken from tables smoothed once per call (two loads per row and connection); without, from the 2^k-term
+ * sum of the formula per row and connection.  The table gradient of that path is summed with atomics. */
 int dl_dwn_layer_bwd(const float *x, const void *saved, const int32_t *idx32,
                      const int32_t *inv_ptr, const int32_t *inv_pos,
                      const float *luts, const float *gy, float alpha, float beta,

@@ -307,6 +307,25 @@ def test_dwn_backward_other_alpha_beta(beta):
     np.testing.assert_allclose(lt.grad.cpu().numpy(), gl, rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("beta", [1.0 / 3.0, -0.5, 0.9])
+@pytest.mark.parametrize("shape", [(70, 40, 25, 8, 1), (33, 24, 9, 7, 2), (20, 64, 5, 10, 1)])
+def test_dwn_backward_more_than_six_inputs(shape, beta):
+    """k > 6: the input gradient from tables smoothed once per call (|beta| <= 1/2) and from the 2^k-term sum
+    (beta = 0.9), both against the oracle; the smoothed form amplifies rounding by (1 + |beta|)^k / (1 - beta) <= 52,
+    hence rtol 1e-5 with a floor of 2e-5."""
+    ops = _ops()
+    B, I, N, k, O = shape
+    x, idx, luts, gy = make_case(sum(shape), *shape)
+    plan = ops.MappingPlan(dev(idx, torch.int32), I)
+    xt = dev(x).requires_grad_(); lt = dev(luts).requires_grad_()
+    y = ops.DWNLayerFunction.apply(xt, lt, plan, 0.3, beta)
+    assert np.array_equal(y.detach().cpu().numpy().reshape(B, N, O), orc.dwn_layer_forward(x, idx, luts))
+    y.backward(dev(gy.reshape(B, -1)))
+    gx, gl = orc.dwn_layer_backward(x, idx, luts, gy, np.float32(0.3), np.float32(beta))
+    np.testing.assert_allclose(xt.grad.cpu().numpy(), gx, rtol=1e-5, atol=2e-5 * max(1.0, float(np.abs(gx).max())))
+    np.testing.assert_allclose(lt.grad.cpu().numpy(), gl, rtol=1e-5, atol=1e-5)
+
+
 def test_dwn_no_input_grad_and_unused_inputs():
     ops = _ops()
     B, I, N, k, O = 40, 50, 3, 2, 1  # 44 of the 50 inputs feed no node: their gradient must be 0
