@@ -837,29 +837,54 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT,
 }
 
 // ---------------------------------------------------------------------------------
-// bwd_gx_hist: the input gradient of a chained layer, written tile-major, with the table-gradient histogram of the
-// layer IN FRONT folded in.  In a chain the input gradient of layer l + 1 is the output gradient of layer l: column i of
-// it, together with the addresses layer l saved, is all layer l's histogram needs - and here it sits in the LDS the
-// moment it is complete.  So the wavefront that has just summed its inputs' rows of a batch tile adds them into the
-// bins of those columns (the quad merge of hist_tiled) before it moves on, and the separate pass that re-reads the
-// [B, I] fp32 gradient for layer l's histogram is gone.  Bins have to live across batch tiles, so a block keeps its
-// slab and walks `tiles_per_block` tiles of its class (t = cls + ncls i); it ends with its bins as one partial set
-// ([set][column][bin]), the sets are added in set order afterwards (dwn_reduce_partials): fixed order, no atomics.
-// The gather itself is dwn_bwd_gx's (O == 1, S form): the unrolled path for sixteen inputs of three entries, the
-// general loop otherwise; same order of additions.
-template <int K, int WI, int FAN>
-__global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__ gyT, const uint8_t *__restrict__ addrT,
+// bwd_gx_walk: the input gradient by blocks that keep their slab of 64 inputs and walk batch tiles, in two roles.
+// HIST (chained layers): written tile-major, with the table-gradient histogram of the layer IN FRONT folded in.  In a
+// chain the input gradient of layer l + 1 is the output gradient of layer l: column i of it, together with the addresses
+// layer l saved, is all layer l's histogram needs - and here it sits in the LDS the moment it is complete.  So the
+// wavefront that has just summed its inputs' rows of a batch tile adds them into the bins of those columns (the quad
+// merge of hist_tiled) before it moves on, and the separate pass that re-reads the [B, I] fp32 gradient for layer l's
+// histogram is gone.  Bins have to live across batch tiles, so a block keeps its slab and walks `tiles_per_block` tiles
+// of its class (t = cls + ncls i); it ends with its bins as one partial set ([set][column][bin]), the sets are added
+// in set order afterwards (dwn_reduce_partials): fixed order, no atomics.
+// ROWS (a single big layer): the row-major gradient gx [B, I] through the block's LDS tile, the blocks paced (below).
+// The gather itself is dwn_bwd_gx's (O == 1, S form): the unrolled path for sixteen inputs of FAN entries each, with
+// the entries' coefficient rows kept in registers over all tiles, the general loop otherwise; same order of additions.
+// Pacing of the walking gather (ROWS).  Its blocks are independent; left alone they spread over several batch tiles and
+// every tile's rows are fetched into an XCD's L2 more than once (measured at the headline shape: 692 MiB against 320
+// compulsory, 55 % L2 misses, 160 us).  So every block starts its tile number i no earlier than i * pace after its own
+// start (the 100 MHz clock all CUs share: no memory traffic, no signal between CUs), which keeps the blocks of an XCD on
+// one tile as long as the pace is one they can hold.  Too fast a pace and more and more blocks fall behind for good
+// (they then run unpaced, as before); too slow costs its own length.  Measured at that shape, step of the layer per
+// pace: 6.4 us per tile 0.297 ms, 6.8 0.285, 7.0 0.275, 7.2 0.277, 7.6 0.283 (in-order gather: 0.294); a quarter of the
+// blocks sampled, 19 % of their tile starts are late at 7.0 us, 13 % at 7.1, 10 % at 7.2, 4 % at 7.6.  The pace is
+// therefore steered, per shape, on the device: every fourth block adds up how many of its tile starts were late, the
+// first block of the next launch of that shape moves the scale by +0.5 % above DWN_PACE_LATE_HI per cent late starts
+// (+3 % above 40: far off) and by -0.25 % below DWN_PACE_LATE_LO, which settles just on the slow side of the best
+// pace (0.278-0.280 ms).  Timing only: the sums and their order do not depend on it.
+#define DWN_PACE_LATE_LO 6
+#define DWN_PACE_LATE_HI 11
+#define DWN_PACE_LINES 16  // counters of the sampled blocks, spread over as many cache lines
+struct DwnPace {
+    float scale;  // multiplies the launch's base pace; 0 = not yet set (1)
+    int pad[31];
+    struct { int late, starts, pad[30]; } seen[DWN_PACE_LINES];  // since the scale was last moved
+};
+#define DWN_PACE_SLOTS 16
+static __device__ DwnPace dwn_pace_state[DWN_PACE_SLOTS];
+template <int K, int WI, int FAN, bool HIST = true, bool ROWS = false>
+__global__ __launch_bounds__(256) void dwn_bwd_gx_walk(const float *__restrict__ gyT, const uint8_t *__restrict__ addrT,
                                                         const float *__restrict__ S, const int *__restrict__ inv_ptr,
                                                         const int *__restrict__ inv_pos, float *__restrict__ gx,
                                                         const uint8_t *__restrict__ prev_addrT, float *__restrict__ prev_partial,
                                                         int I, int N, int BT, int slabs, int split, int part,
-                                                        int tiles_per_block, int Lp, int gather_blocks, DwnReduce red) {
+                                                        int tiles_per_block, int Lp, int gather_blocks, DwnReduce red,
+                                                        int B = 0, int pace = 0, int pace_slot = 0) {
     // the fixed-order sum of this layer's own histogram partials rides behind the gather's blocks
     if ((int)blockIdx.x >= gather_blocks) return dwn_reduce_block(red, (int)blockIdx.x - gather_blocks);
     constexpr int IS = 4 * WI;  // inputs per block
     constexpr int L = 1 << K;
-    __shared__ float tile[IS][65];  // [input][row]
-    __shared__ float hist[IS][65];  // [input = column of the layer in front][bin]
+    __shared__ float tile[IS][65];             // [input][row]
+    __shared__ float hist[HIST ? IS : 1][65];  // [input = column of the layer in front][bin]
     // `split` XCDs share a class of tiles, each with its own part of the slabs (at most as many as stay resident on an
     // XCD): the blocks that read a tile on one XCD then all run at once, and a tile's rows pass through that L2 once.
     const int xcd = blockIdx.x % DL_XCDS, q = blockIdx.x / DL_XCDS;
@@ -874,8 +899,10 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
     const int myptr = inv_ptr[min(i0 + wbeg + min(lane, WI), I)];
     const int ebeg = __builtin_amdgcn_readlane(myptr, 0);
     const int eend = __builtin_amdgcn_readlane(myptr, WI);
+    if (HIST) {
 #pragma unroll
-    for (int r = 0; r < WI; ++r) hist[wbeg + r][lane] = 0.0f;  // my columns' bins (wave-local rows of the array)
+        for (int r = 0; r < WI; ++r) hist[wbeg + r][lane] = 0.0f;  // my columns' bins (wave-local rows of the array)
+    }
     // histogram role of this lane: column (of my wavefront's WI) and the sixteen rows 16 hr .. 16 hr + 15 of a tile
     const int hcl = lane >> 2, hr = lane & 3;
     const bool hlive = hcl < WI && wbeg + hcl < iend;  // whole quads share the column
@@ -886,7 +913,28 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
         const unsigned w = h < 4 ? haw.x : h < 8 ? haw.y : h < 12 ? haw.z : haw.w;
         const unsigned a = (w >> (8 * (h & 3))) & 0xffu;
         float sum;
-        if (dwn_quad_merge(a, hv[h], hr, sum)) dwn_bin_add(&hist[hc][a], sum);
+        if (dwn_quad_merge(a, hv[h], hr, sum)) dwn_bin_add(&hist[HIST ? hc : 0][a], sum);
+    };
+    auto store_rows = [&](int t) {
+        __syncthreads();
+        if (IS % 4 == 0 && iend == IS && t * 64 + 64 <= B && (I & 3) == 0 && (((uintptr_t)gx) & 15) == 0) {
+            typedef float f4v __attribute__((ext_vector_type(4)));
+#pragma unroll
+            for (int pass = 0; pass < (64 * IS / 4 + 255) / 256; ++pass) {
+                const int e = pass * 256 + threadIdx.x;
+                if (64 * IS / 4 % 256 != 0 && e >= 64 * IS / 4) break;
+                const int r = e / (IS / 4), i4 = (e % (IS / 4)) * 4;
+                const f4v v = {tile[i4][r], tile[i4 + 1][r], tile[i4 + 2][r], tile[i4 + 3][r]};
+                __builtin_nontemporal_store(v, reinterpret_cast<f4v *>(&gx[(size_t)(t * 64 + r) * I + i0 + i4]));
+            }
+        } else {
+            for (int e = threadIdx.x; e < 64 * IS; e += 256) {
+                const int r = e / IS, ii = e % IS;
+                const int b = t * 64 + r;
+                if (b < B && ii < iend) __builtin_nontemporal_store(tile[ii][r], &gx[(size_t)b * I + i0 + ii]);
+            }
+        }
+        __syncthreads();
     };
     // FAN > 0: the host found N K = FAN I, which is what a mapping built from whole permutations of the inputs gives -
     // every input read exactly FAN times; checked per wavefront, anything else takes the general loop.
@@ -915,12 +963,42 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
 #pragma unroll
             for (int e = 0; e < WI * FAN; ++e)
                 coef[e] = S[(size_t)(__builtin_amdgcn_readlane(rec3, e) >> 3) * L + (lane & (L - 1))];
+            const unsigned long long t_start = __builtin_amdgcn_s_memrealtime();
+            int late = 0;
+            if (ROWS && pace > 0) {
+                DwnPace *st = &dwn_pace_state[pace_slot];
+                float scale = st->scale;
+                if (!(scale > 0.0f)) scale = 1.0f;
+                if (blockIdx.x == 0 && threadIdx.x == 0) {  // steer on what the sampled blocks of the last launch saw
+                    long long starts = 0, was_late = 0;
+                    for (int l = 0; l < DWN_PACE_LINES; ++l) {
+                        starts += st->seen[l].starts;
+                        was_late += st->seen[l].late;
+                        st->seen[l].starts = 0;
+                        st->seen[l].late = 0;
+                    }
+                    if (starts > 0) {
+                        if (was_late * 100 > starts * 40) scale *= 1.03f;  // far off: most blocks cannot hold the pace
+                        else if (was_late * 100 > starts * DWN_PACE_LATE_HI) scale *= 1.005f;
+                        else if (was_late * 100 < starts * DWN_PACE_LATE_LO) scale *= 0.9975f;
+                        scale = fminf(fmaxf(scale, 0.6f), 1.6f);
+                    }
+                    st->scale = scale;
+                }
+                pace = (int)((float)pace * scale);
+            }
             for (int ti = i_begin; ti < i_end; ++ti) {
+                if (ROWS && pace > 0 && ti > i_begin) {
+                    const unsigned long long due = (unsigned long long)(ti - i_begin) * pace;
+                    if (__builtin_amdgcn_s_memrealtime() - t_start >= due) ++late;
+                    while (__builtin_amdgcn_s_memrealtime() - t_start < due) __builtin_amdgcn_s_sleep(8);
+                }
                 const int t = cls + ncls * ti;
                 const uint8_t *addr_t = addrT + (size_t)t * N * 64 + lane;
                 const float *gy_t = gyT + (size_t)t * N * 64 + lane;
                 float *gx_t = gx + ((size_t)t * I + i0 + wbeg) * 64 + lane;
-                const uint4 haw = *reinterpret_cast<const uint4 *>(prev_addrT + (size_t)t * I * 64 + hcol);
+                uint4 haw = {0u, 0u, 0u, 0u};
+                if (HIST) haw = *reinterpret_cast<const uint4 *>(prev_addrT + (size_t)t * I * 64 + hcol);
                 float acc = 0.0f;
 #pragma unroll
                 for (int s0 = 0; s0 < WI * FAN; s0 += DWN_EG) {
@@ -943,21 +1021,30 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
                         const int sidx = s0 + qq;  // compile-time after unrolling
                         acc = (sidx % FAN == 0) ? 0.0f + term : acc + term;
                         if (sidx % FAN == FAN - 1) {
-                            tile[wbeg + sidx / FAN][lane] = acc;
+                            if (HIST || ROWS) tile[wbeg + sidx / FAN][lane] = acc;
                             // gx as [B/64][I][64], streamed past the L2 (which holds the rows the gather re-reads)
-                            __builtin_nontemporal_store(acc, gx_t + (size_t)(sidx / FAN) * 64);
+                            if (!ROWS) __builtin_nontemporal_store(acc, gx_t + (size_t)(sidx / FAN) * 64);
                         }
                     }
                 }
-                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-                __builtin_amdgcn_wave_barrier();
-                float hv[16];
+                if (ROWS) store_rows(t);
+                if (HIST) {
+                    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                    float hv[16];
 #pragma unroll
-                for (int h = 0; h < 16; ++h) hv[h] = tile[hc][hr * 16 + h];
+                    for (int h = 0; h < 16; ++h) hv[h] = tile[hc][hr * 16 + h];
 #pragma unroll
-                for (int h = 0; h < 16; ++h) hist_step(hv, haw, h);
-                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-                __builtin_amdgcn_wave_barrier();  // the next tile overwrites the rows just read
+                    for (int h = 0; h < 16; ++h) hist_step(hv, haw, h);
+                    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                    __builtin_amdgcn_wave_barrier();  // the next tile overwrites the rows just read
+                }
+            }
+            if (ROWS && pace > 0 && (blockIdx.x / DL_XCDS) % 4 == 0 && threadIdx.x == 0 && i_end - i_begin > 1) {
+                // every fourth slab of every XCD reports
+                auto &seen = dwn_pace_state[pace_slot].seen[(blockIdx.x / (4 * DL_XCDS) * DL_XCDS + blockIdx.x % DL_XCDS) % DWN_PACE_LINES];
+                atomicAdd(&seen.late, late);
+                atomicAdd(&seen.starts, i_end - i_begin - 1);
             }
     }
     }
@@ -967,7 +1054,8 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
             const uint8_t *addr_t = addrT + (size_t)t * N * 64 + lane;
             const float *gy_t = gyT + (size_t)t * N * 64 + lane;
             // the addresses of the layer in front for my column and rows: asked for now, used after the gather
-            const uint4 haw = *reinterpret_cast<const uint4 *>(prev_addrT + (size_t)t * I * 64 + hcol);
+            uint4 haw = {0u, 0u, 0u, 0u};
+            if (HIST) haw = *reinterpret_cast<const uint4 *>(prev_addrT + (size_t)t * I * 64 + hcol);
 #pragma unroll
             for (int r = 0; r < WI; ++r) tile[wbeg + r][lane] = 0.0f;  // inputs nobody reads keep 0
             float acc = 0.0f;
@@ -1011,15 +1099,20 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
                 }
             }
             if (cur >= 0) tile[wbeg + cur][lane] = acc;
-            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            // gx as [B/64][I][64]: my inputs, 256 B each, streamed past the L2 (which holds the rows the gather re-reads)
+            if (ROWS) {
+                store_rows(t);
+            } else {
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                // gx as [B/64][I][64]: my inputs, 256 B each, streamed past the L2 (which holds the rows the gather
+                // re-reads)
 #pragma unroll
-            for (int r = 0; r < WI; ++r)
-                if (wbeg + r < iend)
-                    __builtin_nontemporal_store(tile[wbeg + r][lane], &gx[((size_t)t * I + i0 + wbeg + r) * 64 + lane]);
+                for (int r = 0; r < WI; ++r)
+                    if (wbeg + r < iend)
+                        __builtin_nontemporal_store(tile[wbeg + r][lane], &gx[((size_t)t * I + i0 + wbeg + r) * 64 + lane]);
+            }
             // the same rows into the bins of the layer in front (rows past the batch carry 0 and add nothing)
-            if (hlive) {
+            if (HIST && hlive) {
                 float hv[16];
 #pragma unroll
                 for (int h = 0; h < 16; ++h) hv[h] = tile[hc][hr * 16 + h];
@@ -1031,6 +1124,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_hist(const float *__restrict__
         }
     
     }
+    if (!HIST) return;
     // my columns' bins as one partial set
     const int set = grp * ncls + cls;
     float *out = prev_partial + ((size_t)set * I + i0 + wbeg) * Lp;
@@ -1254,7 +1348,7 @@ struct DwnGroupHead {
     float inv_tau;
 };
 // The layer in front of this one in a chain (its N_prev * 1 outputs are this layer's I inputs): with its saved addresses
-// the gather can fill that layer's table-gradient bins from the input gradient it has just summed (dwn_bwd_gx_hist).
+// the gather can fill that layer's table-gradient bins from the input gradient it has just summed (dwn_bwd_gx_walk).
 struct DwnFusedPrev {
     const uint8_t *addrT;  // [B/64][I][64], what that layer's forward saved
     float *gluts;          // [I][2^k_prev] out
@@ -1299,6 +1393,18 @@ static inline size_t dwn_fused_partial_bytes(int B, int I, int N, int k, int k_p
     if (!wi) return 0;
     const DwnFusedSplit f = dwn_fused_split(dwn_bt(B), I, k_prev, 4 * wi);
     return dl_align256((size_t)f.sets * I * ((size_t)4 << k_prev));
+}
+// When the row-major input gradient is taken by the walking, paced gather instead of one block per (slab, tile): one
+// output per node, the S form, every input read three times on the host's count (N k = 3 I; wavefronts check their own
+// inputs), and a layer big enough that the rows of a tile crowd an XCD's L2.  Forward + backward of the layer, in-order
+// gather -> walking gather: 16384 -> 8192 nodes, B = 4096: 0.294 -> 0.278 ms; B = 8192: 0.675 -> 0.568; B = 16384:
+// 1.357 -> 1.195; 32768 -> 16384, B = 4096: 0.736 -> 0.594.  Inputs read once or twice lose by it (24576 -> 8192:
+// 0.340 -> 0.363 ms; 49152 -> 8192: 0.471 -> 0.531) and keep the in-order gather.
+#define DWN_PACE_GBS 5000.0  // base pace: the bytes of a tile step at this rate
+static inline bool dwn_walk_rows(int BT, int I, int N, int k, int O, bool sform, int gx_tiled) {
+    if (O != 1 || !sform || gx_tiled) return false;
+    if ((long long)N * k != 3LL * I) return false;
+    return (long long)N * 320 >= (2LL << 20) && BT >= 64;
 }
 static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos, const float *luts,
                              const float *gy, int gy_tiled, float alpha, float beta, const float *scale, float *gx,
@@ -1349,7 +1455,7 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
         const int fan = (long long)N * k % I == 0 ? (int)((long long)N * k / I) : 0;  // every input read `fan` times?
         const int gather_blocks = DL_XCDS * f.part * f.groups, grid = gather_blocks + dwn_reduce_blocks(red), Lp = 1 << prev->k;
 #define DWN_GXH(K_, WI_, FAN_)                                                                                                \
-    DL_TIMED("dwn_bwd_gx_hist", s, (dwn_bwd_gx_hist<K_, WI_, FAN_><<<grid, 256, 0, s>>>(src, addrT, D, inv_ptr, inv_pos, gx, prev->addrT, \
+    DL_TIMED("dwn_bwd_gx_hist", s, (dwn_bwd_gx_walk<K_, WI_, FAN_><<<grid, 256, 0, s>>>(src, addrT, D, inv_ptr, inv_pos, gx, prev->addrT, \
                                                                                   prev->partial, I, N, BT, f.slabs, f.split, f.part, f.tpb, Lp, gather_blocks, red)))
 #define DWN_GXH_K(K_)                                                \
     if (fused_wi != DWN_WI) DWN_GXH(K_, DWN_WI_SMALL, 0);            \
@@ -1369,6 +1475,37 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
 #undef DWN_GXH
         const DwnReduce pred = {prev->partial, prev->gluts, (long long)I * Lp, f.sets, nullptr, Lp, 1};
         DL_TIMED("dwn_reduce_partials", s, (dwn_reduce_partials<<<dwn_reduce_blocks(pred), 256, 0, s>>>(pred)));
+    } else if (gx && dwn_walk_rows(BT, I, N, k, O, sform, gx_tiled)) {
+        // row-major input gradient of a big layer whose inputs are all read three times: the walking gather, paced
+        const float *src = gy_tiled ? gy : gyT;
+        const int slabs = dl_ceil_div(I, 4 * DWN_WI);
+        int split = 1;
+        while (split < DL_XCDS && dl_ceil_div(slabs, split) > DWN_RESIDENT) split *= 2;
+        const int part = dl_ceil_div(slabs, split), ncls = DL_XCDS / split, tiles_cls = dl_ceil_div(BT, ncls);
+        int groups = DWN_RESIDENT / part;
+        if (groups > tiles_cls / 8) groups = tiles_cls / 8;  // at least eight tiles per block
+        if (groups < 1) groups = 1;
+        const int tpb = dl_ceil_div(tiles_cls, groups);
+        groups = dl_ceil_div(tiles_cls, tpb);
+        const int gb = DL_XCDS * part * groups;
+        // base pace: the bytes one tile step moves (every XCD reads the rows of `groups` tiles and writes its slabs'
+        // share of them) at DWN_PACE_GBS, in ticks of 10 ns; the device-side scale moves it from there
+        const double step_bytes = (double)DL_XCDS * groups * ((double)N * 320 + (double)I / split * 256);
+        const int pace = (int)(step_bytes / (DWN_PACE_GBS * 1e9) * 1e8);
+        const int slot = (int)(((unsigned)I * 2654435761u ^ (unsigned)N * 40503u ^ (unsigned)BT * 97u ^ (unsigned)k) % DWN_PACE_SLOTS);
+#define DWN_WALK(K_)                                                                                             \
+    DL_TIMED("dwn_bwd_gx", s,                                                                                    \
+             (dwn_bwd_gx_walk<K_, DWN_WI, 3, false, true><<<gb + dwn_reduce_blocks(red), 256, 0, s>>>(           \
+                 src, addrT, D, inv_ptr, inv_pos, gx, nullptr, nullptr, I, N, BT, slabs, split, part, tpb, 0, gb, red, B, pace, slot)))
+        switch (k) {
+            case 1: DWN_WALK(1); break;
+            case 2: DWN_WALK(2); break;
+            case 3: DWN_WALK(3); break;
+            case 4: DWN_WALK(4); break;
+            case 5: DWN_WALK(5); break;
+            default: DWN_WALK(6); break;
+        }
+#undef DWN_WALK
     } else if (gx) {
         const float *src = gy_tiled ? gy : gyT;
         switch (k) {

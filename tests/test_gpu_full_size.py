@@ -59,6 +59,53 @@ def test_single_dwn_layer_all_rows_against_c_restatement():
     assert torch.equal(l2.grad, luts.grad) and torch.equal(x2.grad, xg.grad)
 
 
+@pytest.mark.parametrize("mapping", ["whole permutations", "independent draws"])
+def test_row_major_input_gradient_of_a_big_layer_equals_the_tile_major_one(mapping):
+    """At this size the row-major input gradient is taken by the walking, paced gather, the tile-major one by the
+    one-block-per-(slab, tile) gather: the same terms in the same order, so the same bits - with every input read
+    exactly three times (the unrolled path with the coefficient rows in registers) and with the same number of
+    connections drawn independently (uneven lists: the general loop inside the walking kernel).  Three calls in a row
+    (the pace of the walking gather moves between launches; the sums must not)."""
+    from difflut_amd import _native as nat
+    from difflut_amd import ops
+    from difflut_amd.layers.random_layer import draw_mapping
+    lib = nat.lib()
+    torch.manual_seed(1)
+    B, I, N, k = 4096, 16384, 8192, 6
+    if mapping == "whole permutations":
+        idx = draw_mapping(I, N, k, seed=7)
+    else:
+        idx = torch.randint(0, I, (N, k))
+    plan = ops.MappingPlan(idx.to("cuda", torch.int32), I)
+    x = torch.rand(B, I, device="cuda")
+    luts = torch.rand(N, 1, 64, device="cuda") * 2 - 1
+    gy = torch.randn(B, N, device="cuda")
+    dims = (B, I, N, k, 1)
+    y = torch.empty(B, N, device="cuda")
+    saved = torch.empty(lib.dl_dwn_saved_bytes(*dims), dtype=torch.uint8, device="cuda")
+    wf = torch.empty(lib.dl_dwn_fwd_workspace_bytes(*dims), dtype=torch.uint8, device="cuda")
+    wb = torch.empty(lib.dl_dwn_bwd_workspace_bytes(*dims), dtype=torch.uint8, device="cuda")
+    nat.check(lib.dl_dwn_layer_fwd(x.data_ptr(), plan.idx32.data_ptr(), luts.data_ptr(), y.data_ptr(), saved.data_ptr(),
+                                   wf.data_ptr(), wf.numel(), *dims, nat.stream()))
+    alpha, beta = 0.5 * 0.75 ** 5, 1 / 3
+    BT = B // 64
+
+    def backward(tiled):
+        gx = torch.zeros(B * I, device="cuda")
+        gl = torch.empty_like(luts)
+        nat.check(lib.dl_dwn_layer_bwd_tiled(saved.data_ptr(), plan.inv_ptr.data_ptr(), plan.inv_pos.data_ptr(),
+                                             luts.data_ptr(), gy.data_ptr(), 0, alpha, beta, gx.data_ptr(), tiled, gl.data_ptr(),
+                                             wb.data_ptr(), wb.numel(), *dims, nat.stream()))
+        return gx, gl
+
+    tiles, gl_t = backward(1)
+    want = tiles.view(BT, I, 64).permute(0, 2, 1).reshape(B, I)
+    for _ in range(3):
+        rows, gl_r = backward(0)
+        assert torch.equal(rows.view(B, I), want)
+        assert torch.equal(gl_r, gl_t)
+
+
 def test_deep_stack_against_c_restatement_and_adam_step():
     REGISTRY, NodeConfig, _ = _api()
     from difflut_amd.layers import DWNStack
