@@ -871,7 +871,23 @@ struct DwnPace {
 };
 #define DWN_PACE_SLOTS 16
 static __device__ DwnPace dwn_pace_state[DWN_PACE_SLOTS];
-template <int K, int WI, int FAN, bool HIST = true, bool ROWS = false>
+// the coefficient row of an entry (node n, slot j) as a lane holds it, and what a row gives for an address: the S form
+// (one row per node, two lane reads and their difference) or the D form (one row of 2^(k-1) per slot, one lane read at the
+// address with bit j taken out) - as in dwn_bwd_gx
+template <int K, bool DFORM>
+__device__ __forceinline__ float dwn_walk_coef(const float *__restrict__ T, int n, int j, int lane) {
+    constexpr int L = 1 << K, Lh = K > 1 ? L >> 1 : 1;
+    return DFORM ? T[((size_t)n * K + j) * Lh + (lane & (Lh - 1))] : T[(size_t)n * L + (lane & (L - 1))];
+}
+template <bool DFORM>
+__device__ __forceinline__ float dwn_walk_diff(float coef, unsigned a, int j) {
+    if (DFORM) {
+        const unsigned ap = (a & ((1u << j) - 1u)) | ((a >> (j + 1)) << j);
+        return dl_lane_read(coef, (int)ap);
+    }
+    return dl_lane_read(coef, (int)(a | (1u << j))) - dl_lane_read(coef, (int)(a & ~(1u << j)));
+}
+template <int K, int WI, int FAN, bool HIST = true, bool ROWS = false, bool DFORM = false>
 __global__ __launch_bounds__(256) void dwn_bwd_gx_walk(const float *__restrict__ gyT, const uint8_t *__restrict__ addrT,
                                                         const float *__restrict__ S, const int *__restrict__ inv_ptr,
                                                         const int *__restrict__ inv_pos, float *__restrict__ gx,
@@ -962,7 +978,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_walk(const float *__restrict__
             float coef[FAN > 0 ? WI * FAN : 1];
 #pragma unroll
             for (int e = 0; e < WI * FAN; ++e)
-                coef[e] = S[(size_t)(__builtin_amdgcn_readlane(rec3, e) >> 3) * L + (lane & (L - 1))];
+                coef[e] = dwn_walk_coef<K, DFORM>(S, __builtin_amdgcn_readlane(rec3, e) >> 3, __builtin_amdgcn_readlane(rec3, e) & 7, lane);
             const unsigned long long t_start = __builtin_amdgcn_s_memrealtime();
             int late = 0;
             if (ROWS && pace > 0) {
@@ -1015,9 +1031,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_walk(const float *__restrict__
                     }
 #pragma unroll
                     for (int qq = 0; qq < DWN_EG; ++qq) {
-                        const float hi = dl_lane_read(coef[s0 + qq], (int)(a[qq] | (1u << rj[qq])));
-                        const float lo = dl_lane_read(coef[s0 + qq], (int)(a[qq] & ~(1u << rj[qq])));
-                        const float term = g[qq] * (hi - lo);
+                        const float term = g[qq] * dwn_walk_diff<DFORM>(coef[s0 + qq], a[qq], rj[qq]);
                         const int sidx = s0 + qq;  // compile-time after unrolling
                         acc = (sidx % FAN == 0) ? 0.0f + term : acc + term;
                         if (sidx % FAN == FAN - 1) {
@@ -1082,19 +1096,18 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_walk(const float *__restrict__
                         ri[qq] = r & 31;
                         a[qq] = addr_t[(size_t)rn * 64];
                         g[qq] = gy_t[(size_t)rn * 64];
-                        coef[qq] = S[(size_t)rn * L + (lane & (L - 1))];
+                        coef[qq] = dwn_walk_coef<K, DFORM>(S, rn, rj[qq], lane);
                     }
 #pragma unroll
                     for (int qq = 0; qq < DWN_EG; ++qq) {
                         if (s0 + qq >= cnt) break;  // wave-uniform
-                        const float hi = dl_lane_read(coef[qq], (int)(a[qq] | (1u << rj[qq])));
-                        const float lo = dl_lane_read(coef[qq], (int)(a[qq] & ~(1u << rj[qq])));
+                        const float diff = dwn_walk_diff<DFORM>(coef[qq], a[qq], rj[qq]);
                         if (ri[qq] != cur) {
                             if (cur >= 0) tile[wbeg + cur][lane] = acc;
                             acc = 0.0f;
                             cur = ri[qq];
                         }
-                        acc += g[qq] * (hi - lo);
+                        acc += g[qq] * diff;
                     }
                 }
             }
@@ -1401,8 +1414,8 @@ static inline size_t dwn_fused_partial_bytes(int B, int I, int N, int k, int k_p
 // 1.357 -> 1.195; 32768 -> 16384, B = 4096: 0.736 -> 0.594.  Inputs read once or twice lose by it (24576 -> 8192:
 // 0.340 -> 0.363 ms; 49152 -> 8192: 0.471 -> 0.531) and keep the in-order gather.
 #define DWN_PACE_GBS 5000.0  // base pace: the bytes of a tile step at this rate
-static inline bool dwn_walk_rows(int BT, int I, int N, int k, int O, bool sform, int gx_tiled) {
-    if (O != 1 || !sform || gx_tiled) return false;
+static inline bool dwn_walk_rows(int BT, int I, int N, int k, int O, int gx_tiled) {
+    if (O != 1 || gx_tiled) return false;
     if ((long long)N * k != 3LL * I) return false;
     return (long long)N * 320 >= (2LL << 20) && BT >= 64;
 }
@@ -1475,7 +1488,7 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
 #undef DWN_GXH
         const DwnReduce pred = {prev->partial, prev->gluts, (long long)I * Lp, f.sets, nullptr, Lp, 1};
         DL_TIMED("dwn_reduce_partials", s, (dwn_reduce_partials<<<dwn_reduce_blocks(pred), 256, 0, s>>>(pred)));
-    } else if (gx && dwn_walk_rows(BT, I, N, k, O, sform, gx_tiled)) {
+    } else if (gx && dwn_walk_rows(BT, I, N, k, O, gx_tiled)) {
         // row-major input gradient of a big layer whose inputs are all read three times: the walking gather, paced
         const float *src = gy_tiled ? gy : gyT;
         const int slabs = dl_ceil_div(I, 4 * DWN_WI);
@@ -1492,11 +1505,14 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
         // share of them) at DWN_PACE_GBS, in ticks of 10 ns; the device-side scale moves it from there
         const double step_bytes = (double)DL_XCDS * groups * ((double)N * 320 + (double)I / split * 256);
         const int pace = (int)(step_bytes / (DWN_PACE_GBS * 1e9) * 1e8);
-        const int slot = (int)(((unsigned)I * 2654435761u ^ (unsigned)N * 40503u ^ (unsigned)BT * 97u ^ (unsigned)k) % DWN_PACE_SLOTS);
-#define DWN_WALK(K_)                                                                                             \
+        const int slot = (int)(((unsigned)I * 2654435761u ^ (unsigned)N * 40503u ^ (unsigned)BT * 97u ^ (unsigned)k ^ (sform ? 0u : 7u)) % DWN_PACE_SLOTS);
+#define DWN_WALK_F(K_, DF_)                                                                                      \
     DL_TIMED("dwn_bwd_gx", s,                                                                                    \
-             (dwn_bwd_gx_walk<K_, DWN_WI, 3, false, true><<<gb + dwn_reduce_blocks(red), 256, 0, s>>>(           \
+             (dwn_bwd_gx_walk<K_, DWN_WI, 3, false, true, DF_><<<gb + dwn_reduce_blocks(red), 256, 0, s>>>(      \
                  src, addrT, D, inv_ptr, inv_pos, gx, nullptr, nullptr, I, N, BT, slabs, split, part, tpb, 0, gb, red, B, pace, slot)))
+#define DWN_WALK(K_)                   \
+    if (sform) DWN_WALK_F(K_, false);  \
+    else DWN_WALK_F(K_, true)
         switch (k) {
             case 1: DWN_WALK(1); break;
             case 2: DWN_WALK(2); break;
@@ -1506,6 +1522,7 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
             default: DWN_WALK(6); break;
         }
 #undef DWN_WALK
+#undef DWN_WALK_F
     } else if (gx) {
         const float *src = gy_tiled ? gy : gyT;
         switch (k) {

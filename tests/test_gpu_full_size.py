@@ -59,8 +59,10 @@ def test_single_dwn_layer_all_rows_against_c_restatement():
     assert torch.equal(l2.grad, luts.grad) and torch.equal(x2.grad, xg.grad)
 
 
-@pytest.mark.parametrize("mapping,B", [("whole permutations", 4096), ("independent draws", 4096), ("whole permutations", 4100)])
-def test_row_major_input_gradient_of_a_big_layer_equals_the_tile_major_one(mapping, B):
+@pytest.mark.parametrize("mapping,B,beta", [("whole permutations", 4096, 1 / 3), ("independent draws", 4096, 1 / 3),
+                                            ("whole permutations", 4100, 1 / 3), ("whole permutations", 4096, 0.9),
+                                            ("independent draws", 4100, 0.9)])
+def test_row_major_input_gradient_of_a_big_layer_equals_the_tile_major_one(mapping, B, beta):
     """At this size the row-major input gradient is taken by the walking, paced gather, the tile-major one by the
     one-block-per-(slab, tile) gather: the same terms in the same order, so the same bits - with every input read
     exactly three times (the unrolled path with the coefficient rows in registers) and with the same number of
@@ -87,7 +89,7 @@ def test_row_major_input_gradient_of_a_big_layer_equals_the_tile_major_one(mappi
     wb = torch.empty(lib.dl_dwn_bwd_workspace_bytes(*dims), dtype=torch.uint8, device="cuda")
     nat.check(lib.dl_dwn_layer_fwd(x.data_ptr(), plan.idx32.data_ptr(), luts.data_ptr(), y.data_ptr(), saved.data_ptr(),
                                    wf.data_ptr(), wf.numel(), *dims, nat.stream()))
-    alpha, beta = 0.5 * 0.75 ** 5, 1 / 3
+    alpha = 0.5 * 0.75 ** 5  # beta = 0.9: the other form of the coefficient table (one row per slot)
     BT = (B + 63) // 64
 
     def backward(tiled):
