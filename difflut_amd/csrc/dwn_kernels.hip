@@ -1412,12 +1412,14 @@ static inline size_t dwn_fused_partial_bytes(int B, int I, int N, int k, int k_p
 // inputs), and a layer big enough that the rows of a tile crowd an XCD's L2.  Forward + backward of the layer, in-order
 // gather -> walking gather: 16384 -> 8192 nodes, B = 4096: 0.294 -> 0.278 ms; B = 8192: 0.675 -> 0.568; B = 16384:
 // 1.357 -> 1.195; 32768 -> 16384, B = 4096: 0.736 -> 0.594.  Inputs read once or twice lose by it (24576 -> 8192:
-// 0.340 -> 0.363 ms; 49152 -> 8192: 0.471 -> 0.531) and keep the in-order gather.
+// 0.340 -> 0.363 ms; 49152 -> 8192: 0.471 -> 0.531) and keep the in-order gather, and so do layers with less than 2 MB of
+// rows per tile (8192 -> 4096: 0.143 -> 0.148 ms at B = 4096, 0.259 -> 0.269 at 8192; 10000 -> 5000, B = 8192: 0.338 ->
+// 0.387) and batches of fewer than 32 tiles (B = 2048: 0.161 -> 0.153 ms, B = 1024: no difference).
 #define DWN_PACE_GBS 5000.0  // base pace: the bytes of a tile step at this rate
 static inline bool dwn_walk_rows(int BT, int I, int N, int k, int O, int gx_tiled) {
     if (O != 1 || gx_tiled) return false;
     if ((long long)N * k != 3LL * I) return false;
-    return (long long)N * 320 >= (2LL << 20) && BT >= 64;
+    return (long long)N * 320 >= (2LL << 20) && BT >= 32;
 }
 static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos, const float *luts,
                              const float *gy, int gy_tiled, float alpha, float beta, const float *scale, float *gx,
