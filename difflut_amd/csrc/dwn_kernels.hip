@@ -1045,11 +1045,13 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_walk(const float *__restrict__
                 if (HIST) {
                     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
                     __builtin_amdgcn_wave_barrier();
-                    float hv[16];
+                    if (hcl < WI) {  // (every lane when WI = 16)
+                        float hv[16];
 #pragma unroll
-                    for (int h = 0; h < 16; ++h) hv[h] = tile[hc][hr * 16 + h];
+                        for (int h = 0; h < 16; ++h) hv[h] = tile[hc][hr * 16 + h];
 #pragma unroll
-                    for (int h = 0; h < 16; ++h) hist_step(hv, haw, h);
+                        for (int h = 0; h < 16; ++h) hist_step(hv, haw, h);
+                    }
                     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
                     __builtin_amdgcn_wave_barrier();  // the next tile overwrites the rows just read
                 }
@@ -1473,7 +1475,9 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
     DL_TIMED("dwn_bwd_gx_hist", s, (dwn_bwd_gx_walk<K_, WI_, FAN_><<<grid, 256, 0, s>>>(src, addrT, D, inv_ptr, inv_pos, gx, prev->addrT, \
                                                                                   prev->partial, I, N, BT, f.slabs, f.split, f.part, f.tpb, Lp, gather_blocks, red)))
 #define DWN_GXH_K(K_)                                                \
-    if (fused_wi != DWN_WI) DWN_GXH(K_, DWN_WI_SMALL, 0);            \
+    if (fused_wi != DWN_WI && fan == 6) DWN_GXH(K_, DWN_WI_SMALL, 6); \
+    else if (fused_wi != DWN_WI && fan == 12) DWN_GXH(K_, DWN_WI_SMALL, 12); \
+    else if (fused_wi != DWN_WI) DWN_GXH(K_, DWN_WI_SMALL, 0);       \
     else if (fan == 1) DWN_GXH(K_, DWN_WI, 1);                       \
     else if (fan == 2) DWN_GXH(K_, DWN_WI, 2);                       \
     else if (fan == 3) DWN_GXH(K_, DWN_WI, 3);                       \

@@ -133,6 +133,8 @@ FUSED_CHAIN_SHAPES = [  # (B, I0, k_front, I = nodes of the front layer, N, k)
     (130, 16, 3, 20, 40, 6),     # twelve entries per input: four inputs per wavefront
     (64, 12, 6, 70, 35, 2),      # every input read once
     (150, 20, 4, 96, 32, 6),     # every input read twice
+    (300, 16, 6, 48, 48, 6),     # every input read six times: four inputs per wavefront, unrolled
+    (150, 16, 4, 24, 48, 6),     # twelve times
     (200, 24, 5, 64, 32, 6),     # three reads per input on average only (see the test)
 ]
 
