@@ -566,7 +566,11 @@ def test_full_size_deep_stack_b8192():
 
 @pytest.mark.parametrize("case", [(130, 37, [60, 640], 6, 10, 1.0), (64, 100, [2000], 6, 10, 2.5), (700, 50, [300, 768], 4, 3, 0.5),
                                   (65, 30, [90, 130], 5, 2, 1.0), (256, 64, [512], 6, 8, 1.0), (33, 40, [1000], 6, 7, 1.0),
-                                  (100, 48, [70, 192], 4, 3, 1.0, 2)])
+                                  (100, 48, [70, 192], 4, 3, 1.0, 2),
+                                  # the head's gradient expanded inside the chained gather (at most 16 groups, short lists):
+                                  # inputs read three times, twice, unevenly; 16 groups; 20 groups (written out first)
+                                  (200, 40, [1280, 640], 6, 10, 1.0), (130, 33, [1000, 500], 4, 5, 2.0), (70, 20, [704, 520], 5, 8, 1.0),
+                                  (90, 20, [2048, 1024], 6, 16, 0.5), (90, 20, [2560, 1280], 6, 20, 1.0), (4100, 64, [1024, 512], 6, 8, 1.0)])
 def test_dwn_stack_with_group_sum_head(case):
     """DWNStack(..., head=GroupSum): the last layer sums its columns per group itself.  Against the
     layers one by one followed by GroupSum: logits to rtol 1e-5 (fp32 sums in another order), and
