@@ -363,7 +363,20 @@ __device__ __forceinline__ void dwn_efd_table_block(const DwnTables &tb, int blo
     if (tb.sform) {
         double v = v0;
         for (int m = 0; m < K; ++m) v += (double)beta * __shfl_xor(v, 1 << m);
-        if (live) D[(size_t)c * L + a] = (float)((double)alpha / (1.0 - (double)beta) * v);
+        const float sv = (float)((double)alpha / (1.0 - (double)beta) * v);
+        if (tb.sform == 2) {
+            // the differences a gather would take from the S form, taken here instead (same operands, same rounding)
+            // and laid out like the D form: two slots' rows then fill one 64-lane register
+            for (int j = 0; j < K; ++j) {
+                const float upper = __shfl_xor(sv, 1 << j);
+                if (live && !((a >> j) & 1)) {
+                    const int ap = (a & ((1 << j) - 1)) | ((a >> (j + 1)) << j);
+                    D[((size_t)c * K + j) * Lh + ap] = upper - sv;
+                }
+            }
+            return;
+        }
+        if (live) D[(size_t)c * L + a] = sv;
         return;
     }
     for (int j = 0; j < K; ++j) {
@@ -887,7 +900,16 @@ __device__ __forceinline__ float dwn_walk_diff(float coef, unsigned a, int j) {
     }
     return dl_lane_read(coef, (int)(a | (1u << j))) - dl_lane_read(coef, (int)(a & ~(1u << j)));
 }
-template <int K, int WI, int FAN, bool HIST = true, bool ROWS = false, bool DFORM = false>
+// D-form rows of two entries in one register: lanes 0-31 the even entry's, lanes 32-63 the odd one's
+__device__ __forceinline__ float dwn_walk_diff_packed(float coef, unsigned a, int j, int odd) {
+    const unsigned low = (1u << j) - 1u;
+    const unsigned ap = (a & low) | ((a >> 1) & ~low);  // the address without its bit j
+    return __int_as_float(__builtin_amdgcn_ds_bpermute((int)((ap << 2) | (odd ? 128u : 0u)), __float_as_int(coef)));
+}
+// PACK (with DFORM, without HIST): the D-form row of a slot has 2^(K-1) <= 32 values, so the rows of two entries share one
+// register (lanes 0-31 and 32-63) and a wavefront keeps 32 inputs' entries in the registers that 16 inputs' S-form rows
+// take: half as many blocks cover the inputs, and twice as many inputs are resident on an XCD.
+template <int K, int WI, int FAN, bool HIST = true, bool ROWS = false, bool DFORM = false, bool PACK = false>
 __global__ __launch_bounds__(256) void dwn_bwd_gx_walk(const float *__restrict__ gyT, const uint8_t *__restrict__ addrT,
                                                         const float *__restrict__ S, const int *__restrict__ inv_ptr,
                                                         const int *__restrict__ inv_pos, float *__restrict__ gx,
@@ -955,14 +977,19 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_walk(const float *__restrict__
     // FAN > 0: the host found N K = FAN I, which is what a mapping built from whole permutations of the inputs gives -
     // every input read exactly FAN times; checked per wavefront, anything else takes the general loop.
     bool uniform3 = false;
-    int rec3 = 0;
+    constexpr int NREC = FAN > 0 ? (WI * FAN + 63) / 64 : 1;
+    int rec3[NREC] = {};  // entry e of the wavefront: lane e % 64 of rec3[e / 64]
     if constexpr (FAN > 0) {
-        const int len = __shfl_down(myptr, 1) - myptr;  // lanes 0..15: entries of my input
+        static_assert(!PACK || (DFORM && !HIST && WI * FAN % 2 == 0), "packed rows: D form, no histogram role");
+        const int len = __shfl_down(myptr, 1) - myptr;  // lanes 0..WI-1: entries of my input
         uniform3 = __ballot(lane >= WI || len == FAN) == ~0ull;
         if (uniform3) {
-            const int p = lane < WI * FAN ? inv_pos[ebeg + lane] : 0;
-            const int n = p / K;
-            rec3 = (n << 3) | (p - n * K);
+#pragma unroll
+            for (int r = 0; r < NREC; ++r) {
+                const int p = r * 64 + lane < WI * FAN ? inv_pos[ebeg + r * 64 + lane] : 0;
+                const int n = p / K;
+                rec3[r] = (n << 3) | (p - n * K);
+            }
         }
     }
     const int tiles_cls = (BT - cls + ncls - 1) / ncls;  // tiles t = cls + ncls i < BT
@@ -975,10 +1002,22 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_walk(const float *__restrict__
             // The block keeps its entries over all its tiles, so the coefficient rows of the wavefront's 16 FAN entries
             // stay in registers: one load per entry and block instead of one per entry and tile, and the 256 B x N of
             // coefficient rows no longer share the L2 with the rows of the tiles.
-            float coef[FAN > 0 ? WI * FAN : 1];
+            float coef[FAN > 0 ? (PACK ? WI * FAN / 2 : WI * FAN) : 1];
+            if constexpr (PACK) {
+                constexpr int Lh = 1 << (K - 1);
 #pragma unroll
-            for (int e = 0; e < WI * FAN; ++e)
-                coef[e] = dwn_walk_coef<K, DFORM>(S, __builtin_amdgcn_readlane(rec3, e) >> 3, __builtin_amdgcn_readlane(rec3, e) & 7, lane);
+                for (int e = 0; e < WI * FAN; e += 2) {  // lanes 0-31: entry e, lanes 32-63: entry e + 1
+                    const int r0 = __builtin_amdgcn_readlane(rec3[e / 64], e % 64);
+                    const int r1 = __builtin_amdgcn_readlane(rec3[(e + 1) / 64], (e + 1) % 64);
+                    const int r = lane < 32 ? r0 : r1;
+                    coef[e / 2] = S[((size_t)(r >> 3) * K + (r & 7)) * Lh + (lane & (Lh - 1))];
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < WI * FAN; ++e)
+                    coef[e] = dwn_walk_coef<K, DFORM>(S, __builtin_amdgcn_readlane(rec3[e / 64], e % 64) >> 3,
+                                                      __builtin_amdgcn_readlane(rec3[e / 64], e % 64) & 7, lane);
+            }
             const unsigned long long t_start = __builtin_amdgcn_s_memrealtime();
             int late = 0;
             if (ROWS && pace > 0) {
@@ -1023,7 +1062,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_walk(const float *__restrict__
                     float g[DWN_EG];
 #pragma unroll
                     for (int qq = 0; qq < DWN_EG; ++qq) {
-                        const int r = __builtin_amdgcn_readlane(rec3, s0 + qq);
+                        const int r = __builtin_amdgcn_readlane(rec3[(s0 + qq) / 64], (s0 + qq) % 64);
                         const int rn = r >> 3;
                         rj[qq] = r & 7;
                         a[qq] = addr_t[(size_t)rn * 64];
@@ -1031,8 +1070,9 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_walk(const float *__restrict__
                     }
 #pragma unroll
                     for (int qq = 0; qq < DWN_EG; ++qq) {
-                        const float term = g[qq] * dwn_walk_diff<DFORM>(coef[s0 + qq], a[qq], rj[qq]);
                         const int sidx = s0 + qq;  // compile-time after unrolling
+                        const float term = g[qq] * (PACK ? dwn_walk_diff_packed(coef[PACK ? sidx / 2 : 0], a[qq], rj[qq], sidx & 1)
+                                                         : dwn_walk_diff<DFORM>(coef[PACK ? 0 : sidx], a[qq], rj[qq]));
                         acc = (sidx % FAN == 0) ? 0.0f + term : acc + term;
                         if (sidx % FAN == FAN - 1) {
                             if (HIST || ROWS) tile[wbeg + sidx / FAN][lane] = acc;
@@ -1441,7 +1481,11 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
     // The coefficient tables of the gather depend on the tables only, so their blocks ride in the histogram's launch
     // (extra rows of its grid, dispatched last: they fill the tail in which the histogram blocks drain); the
     // fixed-order sum of the histogram partials rides in the gather's launch the same way.
-    DwnTables tb = {gx ? luts : nullptr, D, scale, alpha_n, beta_n, alpha, beta, (int)NO, k, O, sform ? 1 : 0};
+    // the walking gather of a layer too wide for one XCD's resident blocks packs two D-form rows into a register; for
+    // |beta| <= 1/2 its table then holds the differences of the S form (the bits the other gathers compute from it)
+    const bool walk_rows = gx && dwn_walk_rows(BT, I, N, k, O, gx_tiled);
+    const bool walk_pack = walk_rows && !scale && dl_ceil_div(I, 4 * DWN_WI) > DWN_RESIDENT;
+    DwnTables tb = {gx ? luts : nullptr, D, scale, alpha_n, beta_n, alpha, beta, (int)NO, k, O, sform ? (walk_pack ? 2 : 1) : 0};
     const dim3 hgrid(col_tiles, chunks + dl_ceil_div(dwn_table_blocks(tb), col_tiles));
     if (!gluts) {
         // the table gradient of this layer is already there (the gather of the layer behind filled its bins): only the
@@ -1494,10 +1538,10 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
 #undef DWN_GXH
         const DwnReduce pred = {prev->partial, prev->gluts, (long long)I * Lp, f.sets, nullptr, Lp, 1};
         DL_TIMED("dwn_reduce_partials", s, (dwn_reduce_partials<<<dwn_reduce_blocks(pred), 256, 0, s>>>(pred)));
-    } else if (gx && dwn_walk_rows(BT, I, N, k, O, gx_tiled)) {
+    } else if (walk_rows) {
         // row-major input gradient of a big layer whose inputs are all read three times: the walking gather, paced
         const float *src = gy_tiled ? gy : gyT;
-        const int slabs = dl_ceil_div(I, 4 * DWN_WI);
+        const int slabs = dl_ceil_div(I, 4 * (walk_pack ? 2 * DWN_WI : DWN_WI));
         int split = 1;
         while (split < DL_XCDS && dl_ceil_div(slabs, split) > DWN_RESIDENT) split *= 2;
         const int part = dl_ceil_div(slabs, split), ncls = DL_XCDS / split, tiles_cls = dl_ceil_div(BT, ncls);
@@ -1516,8 +1560,12 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
     DL_TIMED("dwn_bwd_gx", s,                                                                                    \
              (dwn_bwd_gx_walk<K_, DWN_WI, 3, false, true, DF_><<<gb + dwn_reduce_blocks(red), 256, 0, s>>>(      \
                  src, addrT, D, inv_ptr, inv_pos, gx, nullptr, nullptr, I, N, BT, slabs, split, part, tpb, 0, gb, red, B, pace, slot)))
-#define DWN_WALK(K_)                   \
-    if (sform) DWN_WALK_F(K_, false);  \
+#define DWN_WALK(K_)                                                                                             \
+    if (walk_pack)                                                                                               \
+        DL_TIMED("dwn_bwd_gx", s,                                                                                \
+                 (dwn_bwd_gx_walk<K_, 2 * DWN_WI, 3, false, true, true, true><<<gb + dwn_reduce_blocks(red), 256, 0, s>>>( \
+                     src, addrT, D, inv_ptr, inv_pos, gx, nullptr, nullptr, I, N, BT, slabs, split, part, tpb, 0, gb, red, B, pace, slot))); \
+    else if (sform) DWN_WALK_F(K_, false);                                                                       \
     else DWN_WALK_F(K_, true)
         switch (k) {
             case 1: DWN_WALK(1); break;
