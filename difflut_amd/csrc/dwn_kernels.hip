@@ -863,23 +863,29 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT,
 // The gather itself is dwn_bwd_gx's (O == 1, S form): the unrolled path for sixteen inputs of FAN entries each, with
 // the entries' coefficient rows kept in registers over all tiles, the general loop otherwise; same order of additions.
 // Pacing of the walking gather (ROWS).  Its blocks are independent; left alone they spread over several batch tiles and
-// every tile's rows are fetched into an XCD's L2 more than once (measured at the headline shape: 692 MiB against 320
-// compulsory, 55 % L2 misses, 160 us).  So every block starts its tile number i no earlier than i * pace after its own
-// start (the 100 MHz clock all CUs share: no memory traffic, no signal between CUs), which keeps the blocks of an XCD on
-// one tile as long as the pace is one they can hold.  Too fast a pace and more and more blocks fall behind for good
-// (they then run unpaced, as before); too slow costs its own length.  Measured at that shape, step of the layer per
-// pace: 6.4 us per tile 0.297 ms, 6.8 0.285, 7.0 0.275, 7.2 0.277, 7.6 0.283 (in-order gather: 0.294); a quarter of the
-// blocks sampled, 19 % of their tile starts are late at 7.0 us, 13 % at 7.1, 10 % at 7.2, 4 % at 7.6.  The pace is
-// therefore steered, per shape, on the device: every fourth block adds up how many of its tile starts were late, the
-// first block of the next launch of that shape moves the scale by +0.5 % above DWN_PACE_LATE_HI per cent late starts
-// (+3 % above 40: far off) and by -0.25 % below DWN_PACE_LATE_LO, which settles just on the slow side of the best
-// pace (0.278-0.280 ms).  Timing only: the sums and their order do not depend on it.
-#define DWN_PACE_LATE_LO 6
-#define DWN_PACE_LATE_HI 11
+// every tile's rows are fetched into an XCD's L2 more than once (measured at the headline shape, 16 inputs per
+// wavefront: 692 MiB against 320 compulsory, 55 % L2 misses, 160 us).  So every block starts its tile number i no
+// earlier than i * pace after its own start (the 100 MHz clock all CUs share: no memory traffic, no signal between CUs),
+// which keeps the blocks of an XCD on one tile as long as the pace is one they can hold.  Too fast a pace and more and
+// more blocks fall behind for good (they then run unpaced, as before); too slow costs its own length.  Measured at that
+// shape with 32 inputs per wavefront (PACK), step of the layer per pace, given as the rate at which a tile step's bytes
+// would move: 4600 GB/s 0.259 ms with 8 % of the sampled tile starts late, 4800 0.255 (14 %), 4900 0.253 (18 %), 5000
+// 0.253 (22 %), 5100 0.258 (31 %), 5200 0.267 (54 %), no pacing 0.284.  The pace is therefore steered, per shape, on the
+// device: every fourth block adds up how many of its tile starts were late, the first block of the next launch of that
+// shape moves the scale by +0.5 % above the band's upper per cent of late starts (+3 % above 40: far off, and the pace
+// is then held for DWN_PACE_HOLD launches before it may become faster again) and by -0.25 % below the lower one.
+// Timing only: the sums and their order do not depend on it.
+#define DWN_PACE_LATE_LO 15  // per cent of late tile starts: the band while the rows come from the Infinity Cache
+#define DWN_PACE_LATE_HI 24
+#define DWN_PACE_EDGE_LO 1   // and beyond that size
+#define DWN_PACE_EDGE_HI 5
+#define DWN_PACE_CACHE_MB 260.0
+#define DWN_PACE_HOLD 64   // launches the pace is kept after a step back from far off
 #define DWN_PACE_LINES 16  // counters of the sampled blocks, spread over as many cache lines
 struct DwnPace {
     float scale;  // multiplies the launch's base pace; 0 = not yet set (1)
-    int pad[31];
+    int hold;  // launches for which the pace is not made faster again
+    int pad[30];
     struct { int late, starts, pad[30]; } seen[DWN_PACE_LINES];  // since the scale was last moved
 };
 #define DWN_PACE_SLOTS 16
@@ -1021,6 +1027,8 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_walk(const float *__restrict__
             const unsigned long long t_start = __builtin_amdgcn_s_memrealtime();
             int late = 0;
             if (ROWS && pace > 0) {
+                const int late_lo = (pace_slot >> 8) & 255, late_hi = (pace_slot >> 16) & 255;
+                pace_slot &= 255;
                 DwnPace *st = &dwn_pace_state[pace_slot];
                 float scale = st->scale;
                 if (!(scale > 0.0f)) scale = 1.0f;
@@ -1033,9 +1041,16 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_walk(const float *__restrict__
                         st->seen[l].late = 0;
                     }
                     if (starts > 0) {
-                        if (was_late * 100 > starts * 40) scale *= 1.03f;  // far off: most blocks cannot hold the pace
-                        else if (was_late * 100 > starts * DWN_PACE_LATE_HI) scale *= 1.005f;
-                        else if (was_late * 100 < starts * DWN_PACE_LATE_LO) scale *= 0.9975f;
+                        if (was_late * 100 > starts * 40) {  // far off: most blocks cannot hold the pace
+                            scale *= 1.03f;
+                            st->hold = DWN_PACE_HOLD;
+                        } else if (was_late * 100 > starts * late_hi) {
+                            scale *= 1.005f;
+                            st->hold = DWN_PACE_HOLD / 4;
+                        } else if (was_late * 100 < starts * late_lo) {
+                            if (st->hold > 0) --st->hold;  // stay a while where the last step back led
+                            else scale *= 0.9975f;
+                        }
                         scale = fminf(fmaxf(scale, 0.6f), 1.6f);
                     }
                     st->scale = scale;
@@ -1450,13 +1465,15 @@ static inline size_t dwn_fused_partial_bytes(int B, int I, int N, int k, int k_p
     return dl_align256((size_t)f.sets * I * ((size_t)4 << k_prev));
 }
 // When the row-major input gradient is taken by the walking, paced gather instead of one block per (slab, tile): one
-// output per node, the S form, every input read three times on the host's count (N k = 3 I; wavefronts check their own
-// inputs), and a layer big enough that the rows of a tile crowd an XCD's L2.  Forward + backward of the layer, in-order
-// gather -> walking gather: 16384 -> 8192 nodes, B = 4096: 0.294 -> 0.278 ms; B = 8192: 0.675 -> 0.568; B = 16384:
-// 1.357 -> 1.195; 32768 -> 16384, B = 4096: 0.736 -> 0.594.  Inputs read once or twice lose by it (24576 -> 8192:
-// 0.340 -> 0.363 ms; 49152 -> 8192: 0.471 -> 0.531) and keep the in-order gather, and so do layers with less than 2 MB of
-// rows per tile (8192 -> 4096: 0.143 -> 0.148 ms at B = 4096, 0.259 -> 0.269 at 8192; 10000 -> 5000, B = 8192: 0.338 ->
-// 0.387) and batches of fewer than 32 tiles (B = 2048: 0.161 -> 0.153 ms, B = 1024: no difference).
+// output per node, every input read three times on the host's count (N k = 3 I; wavefronts check their own inputs), and
+// a layer big enough that the rows of a tile crowd an XCD's L2.  Forward + backward of the layer, in-order gather ->
+// walking gather with 16 inputs per wavefront -> with 32 (PACK, when the 64-input slabs outnumber an XCD's resident
+// blocks): 16384 -> 8192 nodes, B = 4096: 0.294 -> 0.278 -> 0.253 ms; B = 8192: 0.675 -> 0.568 -> 0.578; B = 16384:
+// 1.357 -> 1.195 -> 1.15; 32768 -> 16384, B = 4096: 0.736 -> 0.594 -> 0.593; 24576 -> 12288: 0.416.  Inputs read once or
+// twice lose by it (24576 -> 8192: 0.340 -> 0.363 ms; 49152 -> 8192: 0.471 -> 0.531) and keep the in-order gather, and
+// so do layers with less than 2 MB of rows per tile (8192 -> 4096: 0.143 -> 0.148 ms at B = 4096, 0.259 -> 0.269 at
+// 8192; 10000 -> 5000, B = 8192: 0.338 -> 0.387) and batches of fewer than 32 tiles (B = 2048, 32 tiles: 0.161 -> 0.153 ->
+// 0.144 ms; B = 1024: no difference).
 #define DWN_PACE_GBS 5000.0  // base pace: the bytes of a tile step at this rate
 static inline bool dwn_walk_rows(int BT, int I, int N, int k, int O, int gx_tiled) {
     if (O != 1 || gx_tiled) return false;
@@ -1555,7 +1572,14 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
         // share of them) at DWN_PACE_GBS, in ticks of 10 ns; the device-side scale moves it from there
         const double step_bytes = (double)DL_XCDS * groups * ((double)N * 320 + (double)I / split * 256);
         const int pace = (int)(step_bytes / (DWN_PACE_GBS * 1e9) * 1e8);
-        const int slot = (int)(((unsigned)I * 2654435761u ^ (unsigned)N * 40503u ^ (unsigned)BT * 97u ^ (unsigned)k ^ (sform ? 0u : 7u)) % DWN_PACE_SLOTS);
+        // the band of late tile starts the steering aims for: where the rows the gather reads (the gradient the histogram
+        // has just written, the saved addresses) still sit in the 256 MB Infinity Cache, falling behind costs little and
+        // the best pace has 15-24 % late starts; beyond that size the step time has an edge (B = 8192 at the headline's
+        // widths: 0.579 ms at 3200 GB/s with no late starts, 0.590 at 3400 with 0.2 %, 0.614 at 3600 with 63 %) and the
+        // pace stays just on its slow side
+        const bool cached = (double)N * BT * 64 * 5 <= DWN_PACE_CACHE_MB * 1e6;
+        const int band = cached ? (DWN_PACE_LATE_LO << 8) | (DWN_PACE_LATE_HI << 16) : (DWN_PACE_EDGE_LO << 8) | (DWN_PACE_EDGE_HI << 16);
+        const int slot = band + (int)(((unsigned)I * 2654435761u ^ (unsigned)N * 40503u ^ (unsigned)BT * 97u ^ (unsigned)k ^ (sform ? 0u : 7u)) % DWN_PACE_SLOTS);
 #define DWN_WALK_F(K_, DF_)                                                                                      \
     DL_TIMED("dwn_bwd_gx", s,                                                                                    \
              (dwn_bwd_gx_walk<K_, DWN_WI, 3, false, true, DF_><<<gb + dwn_reduce_blocks(red), 256, 0, s>>>(      \
