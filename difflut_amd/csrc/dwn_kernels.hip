@@ -1501,7 +1501,7 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
     // the walking gather of a layer too wide for one XCD's resident blocks packs two D-form rows into a register; for
     // |beta| <= 1/2 its table then holds the differences of the S form (the bits the other gathers compute from it)
     const bool walk_rows = gx && dwn_walk_rows(BT, I, N, k, O, gx_tiled);
-    const bool walk_pack = walk_rows && !scale && dl_ceil_div(I, 4 * DWN_WI) > DWN_RESIDENT;
+    const bool walk_pack = walk_rows && dl_ceil_div(I, 4 * DWN_WI) > DWN_RESIDENT;
     DwnTables tb = {gx ? luts : nullptr, D, scale, alpha_n, beta_n, alpha, beta, (int)NO, k, O, sform ? (walk_pack ? 2 : 1) : 0};
     const dim3 hgrid(col_tiles, chunks + dl_ceil_div(dwn_table_blocks(tb), col_tiles));
     if (!gluts) {
