@@ -59,28 +59,34 @@ def test_single_dwn_layer_all_rows_against_c_restatement():
     assert torch.equal(l2.grad, luts.grad) and torch.equal(x2.grad, xg.grad)
 
 
-@pytest.mark.parametrize("mapping,B,beta", [("whole permutations", 4096, 1 / 3), ("independent draws", 4096, 1 / 3),
-                                            ("whole permutations", 4100, 1 / 3), ("whole permutations", 4096, 0.9),
-                                            ("independent draws", 4100, 0.9)])
-def test_row_major_input_gradient_of_a_big_layer_equals_the_tile_major_one(mapping, B, beta):
-    """At this size the row-major input gradient is taken by the walking, paced gather, the tile-major one by the
-    one-block-per-(slab, tile) gather: the same terms in the same order, so the same bits - with every input read
-    exactly three times (the unrolled path with the coefficient rows in registers) and with the same number of
-    connections drawn independently (uneven lists: the general loop inside the walking kernel).  Three calls in a row
-    (the pace of the walking gather moves between launches; the sums must not)."""
+@pytest.mark.parametrize("mapping,B,beta,shape", [
+    ("whole permutations", 4096, 1 / 3, (16384, 8192, 6)), ("independent draws", 4096, 1 / 3, (16384, 8192, 6)),
+    ("whole permutations", 4100, 1 / 3, (16384, 8192, 6)), ("whole permutations", 4096, 0.9, (16384, 8192, 6)),
+    ("independent draws", 4100, 0.9, (16384, 8192, 6)),
+    # fewer inputs per node: rows of 4 and 8 values, two of them per register all the same
+    ("whole permutations", 2100, 1 / 3, (16384, 16384, 3)), ("whole permutations", 2048, 0.9, (16384, 12288, 4)),
+    # 8000 inputs fit one XCD's resident blocks at 16 inputs per wavefront: the walking gather without the packing
+    ("whole permutations", 2100, 1 / 3, (8000, 8000, 3))])
+def test_row_major_input_gradient_of_a_big_layer_equals_the_tile_major_one(mapping, B, beta, shape):
+    """At this size the row-major input gradient is taken by the walking, paced gather (two entries' rows of table
+    differences per register, 32 inputs per wavefront), the tile-major one by the one-block-per-(slab, tile) gather:
+    the same terms in the same order, so the same bits - with every input read exactly three times (the unrolled path
+    with the coefficient rows in registers) and with the same number of connections drawn independently (uneven lists:
+    the general loop inside the walking kernel).  Three calls in a row (the pace of the walking gather moves between
+    launches; the sums must not)."""
     from difflut_amd import _native as nat
     from difflut_amd import ops
     from difflut_amd.layers.random_layer import draw_mapping
     lib = nat.lib()
     torch.manual_seed(1)
-    I, N, k = 16384, 8192, 6  # B = 4100: a last batch tile of four rows
+    I, N, k = shape  # B = 4100: a last batch tile of four rows
     if mapping == "whole permutations":
         idx = draw_mapping(I, N, k, seed=7)
     else:
         idx = torch.randint(0, I, (N, k))
     plan = ops.MappingPlan(idx.to("cuda", torch.int32), I)
     x = torch.rand(B, I, device="cuda")
-    luts = torch.rand(N, 1, 64, device="cuda") * 2 - 1
+    luts = torch.rand(N, 1, 1 << k, device="cuda") * 2 - 1
     gy = torch.randn(B, N, device="cuda")
     dims = (B, I, N, k, 1)
     y = torch.empty(B, N, device="cuda")
