@@ -7,7 +7,7 @@
  * dl_profile_read, which waits for the kernels it reports on): outputs and
  * workspaces come from the caller, kernels are enqueued on `stream`.
  * The library itself holds two things in device memory, per GPU, for the life of the process: the scratch of
- * dl_dwn_layer_fwd_static (DL_DWN_STATIC_SCRATCH_BYTES) and 33 KB of pacing state of the input-gradient kernel
+ * dl_dwn_layer_fwd_static (DL_DWN_STATIC_SCRATCH_BYTES) and 34 KB of pacing state of the input-gradient kernel
  * for big layers (how fast its blocks step through the batch, adjusted from launch to launch; it changes
  * durations only, never a result).
  *
