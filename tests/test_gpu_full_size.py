@@ -66,7 +66,9 @@ def test_single_dwn_layer_all_rows_against_c_restatement():
     # fewer inputs per node: rows of 4 and 8 values, two of them per register all the same
     ("whole permutations", 2100, 1 / 3, (16384, 16384, 3)), ("whole permutations", 2048, 0.9, (16384, 12288, 4)),
     # 8000 inputs fit one XCD's resident blocks at 16 inputs per wavefront: the walking gather without the packing
-    ("whole permutations", 2100, 1 / 3, (8000, 8000, 3))])
+    ("whole permutations", 2100, 1 / 3, (8000, 8000, 3)),
+    # widths that are no multiple of a block's 128 inputs or of four (scalar stores, a last block with two inputs)
+    ("whole permutations", 2100, 1 / 3, (16386, 8193, 6))])
 def test_row_major_input_gradient_of_a_big_layer_equals_the_tile_major_one(mapping, B, beta, shape):
     """At this size the row-major input gradient is taken by the walking, paced gather (two entries' rows of table
     differences per register, 32 inputs per wavefront), the tile-major one by the one-block-per-(slab, tile) gather:
