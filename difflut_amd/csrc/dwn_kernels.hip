@@ -23,6 +23,7 @@
 //                           floating-point atomics anywhere)
 // k > 6 goes to the one-thread-per-element kernels of dwn_generic.hip.
 #include "dl_common.h"
+#include <algorithm>
 #include <mutex>
 #include <type_traits>
 #include "dwn_generic.h"
@@ -1223,10 +1224,34 @@ static inline void dwn_hist_grid(long long NO, int BT, int &col_tiles, int &chun
     tpc = dl_ceil_div(BT, chunks);
     chunks = dl_ceil_div(BT, tpc);
 }
+// A big layer's backward with row-major gradients (the walking gather, dwn_walk_rows) is taken in chunks of about
+// DWN_ROW_CHUNK_BYTES worth of batch tiles, histogram and gather of one chunk after the other: the tile-major copy of a chunk's
+// gy (and its saved addresses) is then still in the 256 MB Infinity Cache when the gather reads it.  Measured at
+// 16384 -> 8192 nodes: the gather takes 109 us for 4096 rows but 284 us for 8192 and 566 us for 16384 in one piece.
+// Every chunk leaves its own partial sets of the table gradient; the last chunk's launch adds all of them, in order.
+#define DWN_ROW_CHUNK_BYTES 172e6  // gy tile-major + saved addresses of a chunk (the headline's 4096 rows: 168 MB)
+static inline bool dwn_walk_rows(int BT, int I, int N, int k, int O, int gx_tiled);
+static inline int dwn_row_chunks(int BT, int I, int N, int k, int O) {
+    int tiles = (int)(DWN_ROW_CHUNK_BYTES / ((double)N * O * 320));
+    if (tiles < 32) tiles = 32;  // (the walking gather wants 32 tiles)
+    if (2 * BT < 3 * tiles || !dwn_walk_rows(BT, I, N, k, O, 0)) return 1;
+    if (dl_ceil_div((long long)N * O, DWN_HC) > 512) return 1;  // (a chunk's histogram must leave partial sets)
+    return (BT + tiles / 2) / tiles;
+}
 // chunk partials of the table gradient (none when one chunk covers the batch)
-static inline size_t dwn_partial_bytes(int B, int N, int k, int O) {
+static inline size_t dwn_partial_bytes(int B, int I, int N, int k, int O) {
     int col_tiles, chunks, tpc;
-    dwn_hist_grid((long long)N * O, dwn_bt(B), col_tiles, chunks, tpc);
+    const int BT = dwn_bt(B), n = dwn_row_chunks(BT, I, N, k, O);
+    if (n > 1) {
+        const int tc = dl_ceil_div(BT, n);
+        size_t sets = 0;
+        for (int c = 0; c < n; ++c) {
+            dwn_hist_grid((long long)N * O, BT - c * tc < tc ? BT - c * tc : tc, col_tiles, chunks, tpc);
+            sets += chunks;
+        }
+        return dl_align256(sets * N * O * sizeof(float) << k);
+    }
+    dwn_hist_grid((long long)N * O, BT, col_tiles, chunks, tpc);
     return chunks > 1 ? dl_align256((size_t)chunks * N * O * sizeof(float) << k) : 0;
 }
 
@@ -1259,8 +1284,7 @@ extern "C" size_t dl_dwn_fwd_workspace_bytes(int B, int I, int N, int k, int O) 
     return dwn_fast(N, k, O) ? dwn_planes_bytes(B, I) : 256;
 }
 extern "C" size_t dl_dwn_bwd_workspace_bytes(int B, int I, int N, int k, int O) {
-    (void)I;
-    return dwn_fast(N, k, O) ? dwn_table_bytes(N, k, O) + dwn_gyT_bytes(B, N, O) + dwn_partial_bytes(B, N, k, O)
+    return dwn_fast(N, k, O) ? dwn_table_bytes(N, k, O) + dwn_gyT_bytes(B, N, O) + dwn_partial_bytes(B, I, N, k, O)
                              : dl_align256(dwn_generic_smooth_bytes(N, k, O));  // k > 6: the smoothed tables
 }
 
@@ -1426,6 +1450,13 @@ struct DwnFusedPrev {
     float *partial;        // [sets][I][2^k_prev] scratch
 };
 __global__ __launch_bounds__(256) void dwn_build_tables(DwnTables tb) { dwn_table_block(tb, blockIdx.x); }
+// one chunk of rows of a backward taken in several (dwn_row_chunks)
+struct DwnRowChunk {
+    float *partial_base;  // the partial sets of all chunks
+    int set_offset;       // where this chunk's sets start
+    int total_sets;       // > 0: the last chunk, whose launch adds all sets
+    bool first;           // builds the coefficient tables
+};
 // How the fused gather is laid over the chip.  An XCD keeps DWN_RESIDENT of its blocks at a time; blocks that read the
 // same tile through the same L2 should all be among them, or the tile's rows are fetched once per round of blocks.  So
 // `split` XCDs (1, 2, 4 or 8) share a class of tiles, each taking `part` <= DWN_RESIDENT of the slabs, and where a part
@@ -1468,8 +1499,9 @@ static inline size_t dwn_fused_partial_bytes(int B, int I, int N, int k, int k_p
 // output per node, every input read three times on the host's count (N k = 3 I; wavefronts check their own inputs), and
 // a layer big enough that the rows of a tile crowd an XCD's L2.  Forward + backward of the layer, in-order gather ->
 // walking gather with 16 inputs per wavefront -> with 32 (PACK, when the 64-input slabs outnumber an XCD's resident
-// blocks): 16384 -> 8192 nodes, B = 4096: 0.294 -> 0.278 -> 0.253 ms; B = 8192: 0.675 -> 0.568 -> 0.578; B = 16384:
-// 1.357 -> 1.195 -> 1.15; 32768 -> 16384, B = 4096: 0.736 -> 0.594 -> 0.593; 24576 -> 12288: 0.416.  Inputs read once or
+// blocks): 16384 -> 8192 nodes, B = 4096: 0.294 -> 0.278 -> 0.253 ms; B = 8192: 0.675 -> 0.568 -> 0.578 (0.513 in chunks
+// of rows, dwn_row_chunks); B = 16384: 1.357 -> 1.195 -> 1.15 (1.046); 32768 -> 16384, B = 4096: 0.736 -> 0.594 -> 0.593
+// (0.589); 24576 -> 12288: 0.416.  Inputs read once or
 // twice lose by it (24576 -> 8192: 0.340 -> 0.363 ms; 49152 -> 8192: 0.471 -> 0.531) and keep the in-order gather, and
 // so do layers with less than 2 MB of rows per tile (8192 -> 4096: 0.143 -> 0.148 ms at B = 4096, 0.259 -> 0.269 at
 // 8192; 10000 -> 5000, B = 8192: 0.338 -> 0.387) and batches of fewer than 32 tiles (B = 2048, 32 tiles: 0.161 -> 0.153 ->
@@ -1484,7 +1516,8 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
                              const float *gy, int gy_tiled, float alpha, float beta, const float *scale, float *gx,
                              int gx_tiled, float *gluts, void *ws, int B, int I, int N, int k, int O, hipStream_t s,
                              const DwnGroupHead *head = nullptr, const float *alpha_n = nullptr,
-                             const float *beta_n = nullptr, const DwnFusedPrev *prev = nullptr) {
+                             const float *beta_n = nullptr, const DwnFusedPrev *prev = nullptr,
+                             const DwnRowChunk *rc = nullptr) {
     const long long NO = (long long)N * O;
     const int L = 1 << k;
     const uint8_t *addrT = (const uint8_t *)saved;
@@ -1493,6 +1526,29 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
     const int BT = dwn_bt(B), BP = BT * 64;
     float *partial = (float *)((char *)ws + dwn_table_bytes(N, k, O) + dwn_gyT_bytes(B, N, O));
     int col_tiles, chunks, tpc;
+    if (!rc && gx && gluts && !prev && !head && !gy_tiled && !gx_tiled) {
+        const int n = dwn_row_chunks(BT, I, N, k, O);
+        if (n > 1) {  // in chunks of rows, each through this function again
+            const int tc = dl_ceil_div(BT, n);
+            int total = 0, sets = 0;
+            for (int c = 0; c < n; ++c) {
+                dwn_hist_grid(NO, std::min(tc, BT - c * tc), col_tiles, chunks, tpc);
+                total += chunks;
+            }
+            for (int c = 0; c < n; ++c) {
+                const int t0 = c * tc, tiles = std::min(tc, BT - t0), rows = std::min(B - t0 * 64, tiles * 64);
+                const DwnRowChunk r = {partial, sets, c == n - 1 ? total : 0, c == 0};
+                const int rcode = dwn_backward_fast(addrT + (size_t)t0 * N * 64, inv_ptr, inv_pos, luts, gy + (size_t)t0 * 64 * NO, 0,
+                                                    alpha, beta, scale, gx + (size_t)t0 * 64 * I, 0, gluts, ws, rows, I, N, k, O, s,
+                                                    nullptr, alpha_n, beta_n, nullptr, &r);
+                if (rcode) return rcode;
+                dwn_hist_grid(NO, tiles, col_tiles, chunks, tpc);
+                sets += chunks;
+            }
+            return DL_OK;
+        }
+    }
+    if (rc) partial = rc->partial_base + (size_t)rc->set_offset * NO * L;
     dwn_hist_grid(NO, BT, col_tiles, chunks, tpc);
     const bool sform = !scale && beta >= -0.5f && beta <= 0.5f;
     // The coefficient tables of the gather depend on the tables only, so their blocks ride in the histogram's launch
@@ -1502,7 +1558,7 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
     // |beta| <= 1/2 its table then holds the differences of the S form (the bits the other gathers compute from it)
     const bool walk_rows = gx && dwn_walk_rows(BT, I, N, k, O, gx_tiled);
     const bool walk_pack = walk_rows && dl_ceil_div(I, 4 * DWN_WI) > DWN_RESIDENT;
-    DwnTables tb = {gx ? luts : nullptr, D, scale, alpha_n, beta_n, alpha, beta, (int)NO, k, O, sform ? (walk_pack ? 2 : 1) : 0};
+    DwnTables tb = {gx && (!rc || rc->first) ? luts : nullptr, D, scale, alpha_n, beta_n, alpha, beta, (int)NO, k, O, sform ? (walk_pack ? 2 : 1) : 0};
     const dim3 hgrid(col_tiles, chunks + dl_ceil_div(dwn_table_blocks(tb), col_tiles));
     if (!gluts) {
         // the table gradient of this layer is already there (the gather of the layer behind filled its bins): only the
@@ -1523,6 +1579,10 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
                                                   gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc, partial, scale, chunks, tb)));
     // (the row-major histogram's scale is applied in the sum; the tile-major ones scale afterwards)
     DwnReduce red = {gluts && chunks > 1 ? partial : nullptr, gluts, NO * L, chunks, (head || gy_tiled) ? nullptr : scale, L, O};
+    if (rc) {  // a chunk of rows: the last one adds the sets of all chunks
+        red.partial = rc->total_sets ? rc->partial_base : nullptr;
+        red.chunks = rc->total_sets;
+    }
     const int fused_wi = prev && gx && gx_tiled && O == 1 && sform ? dwn_fused_wi(I, N, k) : 0;
     if (!gx && dwn_reduce_blocks(red))
         DL_TIMED("dwn_reduce_partials", s, (dwn_reduce_partials<<<dwn_reduce_blocks(red), 256, 0, s>>>(red)));

@@ -68,7 +68,10 @@ def test_single_dwn_layer_all_rows_against_c_restatement():
     # 8000 inputs fit one XCD's resident blocks at 16 inputs per wavefront: the walking gather without the packing
     ("whole permutations", 2100, 1 / 3, (8000, 8000, 3)),
     # widths that are no multiple of a block's 128 inputs or of four (scalar stores, a last block with two inputs)
-    ("whole permutations", 2100, 1 / 3, (16386, 8193, 6))])
+    ("whole permutations", 2100, 1 / 3, (16386, 8193, 6)),
+    # more than 6000 rows: the backward is taken in chunks of about 4096 rows (two here, the last tile with eight rows;
+    # three of 53 or 54 tiles each), and the table gradient adds the chunks' partial sums one after the other
+    ("whole permutations", 8200, 1 / 3, (16384, 8192, 6)), ("independent draws", 10250, 0.9, (16384, 8192, 6))])
 def test_row_major_input_gradient_of_a_big_layer_equals_the_tile_major_one(mapping, B, beta, shape):
     """At this size the row-major input gradient is taken by the walking, paced gather (two entries' rows of table
     differences per register, 32 inputs per wavefront), the tile-major one by the one-block-per-(slab, tile) gather:
@@ -113,7 +116,11 @@ def test_row_major_input_gradient_of_a_big_layer_equals_the_tile_major_one(mappi
     for _ in range(3):
         rows, gl_r = backward(0)
         assert torch.equal(rows.view(B, I), want)
-        assert torch.equal(gl_r, gl_t)
+        if BT < 96:
+            assert torch.equal(gl_r, gl_t)
+        else:  # the same terms, grouped by chunk of rows: bins of about B / 64 values of size ~1
+            torch.testing.assert_close(gl_r, gl_t, rtol=1e-5, atol=2e-5)
+        del rows
 
 
 def test_deep_stack_against_c_restatement_and_adam_step():
