@@ -1093,7 +1093,7 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_walk(const float *__restrict__
                         if (sidx % FAN == FAN - 1) {
                             if (HIST || ROWS) tile[wbeg + sidx / FAN][lane] = acc;
                             // gx as [B/64][I][64], streamed past the L2 (which holds the rows the gather re-reads)
-                            if (!ROWS) __builtin_nontemporal_store(acc, gx_t + (size_t)(sidx / FAN) * 64);
+                            if (!ROWS && gx) __builtin_nontemporal_store(acc, gx_t + (size_t)(sidx / FAN) * 64);
                         }
                     }
                 }
@@ -1176,11 +1176,13 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_walk(const float *__restrict__
                 __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
                 __builtin_amdgcn_wave_barrier();
                 // gx as [B/64][I][64]: my inputs, 256 B each, streamed past the L2 (which holds the rows the gather
-                // re-reads)
+                // re-reads); gx == null: the sums are only wanted for the bins of the layer in front
+                if (gx) {
 #pragma unroll
-                for (int r = 0; r < WI; ++r)
-                    if (wbeg + r < iend)
-                        __builtin_nontemporal_store(tile[wbeg + r][lane], &gx[((size_t)t * I + i0 + wbeg + r) * 64 + lane]);
+                    for (int r = 0; r < WI; ++r)
+                        if (wbeg + r < iend)
+                            __builtin_nontemporal_store(tile[wbeg + r][lane], &gx[((size_t)t * I + i0 + wbeg + r) * 64 + lane]);
+                }
             }
             // the same rows into the bins of the layer in front (rows past the batch carry 0 and add nothing)
             if (HIST && hlive) {
@@ -1558,7 +1560,8 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
     // |beta| <= 1/2 its table then holds the differences of the S form (the bits the other gathers compute from it)
     const bool walk_rows = gx && dwn_walk_rows(BT, I, N, k, O, gx_tiled);
     const bool walk_pack = walk_rows && dl_ceil_div(I, 4 * DWN_WI) > DWN_RESIDENT;
-    DwnTables tb = {gx && (!rc || rc->first) ? luts : nullptr, D, scale, alpha_n, beta_n, alpha, beta, (int)NO, k, O, sform ? (walk_pack ? 2 : 1) : 0};
+    const bool gather = gx || prev;  // (prev without gx: the input gradient is summed for the bins in front, not stored)
+    DwnTables tb = {gather && (!rc || rc->first) ? luts : nullptr, D, scale, alpha_n, beta_n, alpha, beta, (int)NO, k, O, sform ? (walk_pack ? 2 : 1) : 0};
     const dim3 hgrid(col_tiles, chunks + dl_ceil_div(dwn_table_blocks(tb), col_tiles));
     if (!gluts) {
         // the table gradient of this layer is already there (the gather of the layer behind filled its bins): only the
@@ -1566,12 +1569,12 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
         if (dwn_table_blocks(tb)) DL_TIMED("dwn_build_tables", s, (dwn_build_tables<<<dwn_table_blocks(tb), 256, 0, s>>>(tb)));
     } else if (head)
         DL_TIMED("dwn_bwd_hist_groups", s, (dwn_bwd_hist_tiled<true><<<hgrid, 256, 0, s>>>(
-                                               gy, addrT, gluts, (int)NO, O, L, BT, tpc, partial, chunks, tb, gx ? gyT : nullptr, B,
+                                               gy, addrT, gluts, (int)NO, O, L, BT, tpc, partial, chunks, tb, gather ? gyT : nullptr, B,
                                                head->groups, head->gsize, head->inv_tau)));
     else if (gy_tiled)
         DL_TIMED("dwn_bwd_hist_tiled", s,
                  (dwn_bwd_hist_tiled<false><<<hgrid, 256, 0, s>>>(gy, addrT, gluts, (int)NO, O, L, BT, tpc, partial, chunks, tb)));
-    else if (gx)
+    else if (gather)
         DL_TIMED("dwn_bwd_transpose_hist", s, (dwn_bwd_transpose_hist<true><<<hgrid, 256, 0, s>>>(
                                                   gy, addrT, gyT, gluts, B, (int)NO, O, L, BP, BT, tpc, partial, scale, chunks, tb)));
     else
@@ -1583,8 +1586,8 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
         red.partial = rc->total_sets ? rc->partial_base : nullptr;
         red.chunks = rc->total_sets;
     }
-    const int fused_wi = prev && gx && gx_tiled && O == 1 && sform ? dwn_fused_wi(I, N, k) : 0;
-    if (!gx && dwn_reduce_blocks(red))
+    const int fused_wi = prev && (gx_tiled || !gx) && O == 1 && sform ? dwn_fused_wi(I, N, k) : 0;
+    if (!gather && dwn_reduce_blocks(red))
         DL_TIMED("dwn_reduce_partials", s, (dwn_reduce_partials<<<dwn_reduce_blocks(red), 256, 0, s>>>(red)));
     if (fused_wi) {
         // the gather that also fills the bins of the layer in front
@@ -2183,10 +2186,10 @@ extern "C" int dl_dwn_layer_bwd_chain_fused(const void *saved, const int32_t *in
                                             float *prev_gluts, void *ws, size_t ws_bytes, int B, int I, int N, int k, int O,
                                             void *stream) {
     if (!saved || !luts || !gy || !ws || !alpha_n || !beta_n) return DL_ERR_NULL;
-    if (gx && (!inv_ptr || !inv_pos)) return DL_ERR_NULL;
+    if ((gx || prev_saved) && (!inv_ptr || !inv_pos)) return DL_ERR_NULL;
     if (gy_form < 0 || gy_form > 2) return DL_ERR_SHAPE;
     if (!gluts && gy_form != 1) return DL_ERR_SHAPE;
-    if (!gluts && !gx) return DL_ERR_NULL;  // nothing to do
+    if (!gluts && !gx && !prev_saved) return DL_ERR_NULL;  // nothing to do
     int rc = dwn_check(B, I, N, k, O);
     if (rc) return rc;
     if (gy_form == 2 && (groups <= 0 || !(tau > 0.0f))) return DL_ERR_SHAPE;
@@ -2194,7 +2197,7 @@ extern "C" int dl_dwn_layer_bwd_chain_fused(const void *saved, const int32_t *in
     DwnFusedPrev prev = {nullptr, nullptr, 0, nullptr};
     size_t need = dl_dwn_bwd_workspace_bytes(B, I, N, k, O);
     if (prev_saved) {
-        if (!prev_gluts || !gx || !gx_tiled) return DL_ERR_NULL;
+        if (!prev_gluts || (gx && !gx_tiled)) return DL_ERR_NULL;  // gx == NULL: only the bins of the layer in front
         if ((uintptr_t)prev_saved & 15) return DL_ERR_UNSUPPORTED;  // its addresses are read sixteen at a time
         if (!dl_dwn_chain_fusable(B, I, N, k, O, k_prev, beta_abs_max)) return DL_ERR_UNSUPPORTED;
         prev = DwnFusedPrev{(const uint8_t *)prev_saved, prev_gluts, k_prev, (float *)((char *)ws + need)};

@@ -278,13 +278,15 @@ class DWNStackFunction(torch.autograd.Function):
         luts, saved = ctx.saved_tensors[:n], ctx.saved_tensors[n:]
         lib = nat.lib()
         g, tiled = _f32(gy), 0
+        device = g.device
         grads = [None] * n
         have_tables = [False] * n  # table gradient already produced by the call for the layer behind
         for l in range(n - 1, -1, -1):
             B, I, N, k, O = dims = ctx.dims_all[l]
             plan = ctx.plans[l]
+            first_wants_input_grad = ctx.needs_input_grad[0] and not ctx.encoded
             if l > 0:
-                gx = torch.empty(lib.dl_dwn_tiled_bytes(B, I) // 4, dtype=torch.float32, device=g.device)
+                gx = torch.empty(lib.dl_dwn_tiled_bytes(B, I) // 4, dtype=torch.float32, device=device)
                 gx_tiled = 1
             else:
                 want = ctx.needs_input_grad[0] and not ctx.encoded
@@ -292,12 +294,12 @@ class DWNStackFunction(torch.autograd.Function):
                 if not want:
                     gx = None
                 elif gx_tiled:
-                    gx = torch.empty(lib.dl_dwn_tiled_bytes(B, I) // 4, dtype=torch.float32, device=g.device)
+                    gx = torch.empty(lib.dl_dwn_tiled_bytes(B, I) // 4, dtype=torch.float32, device=device)
                 else:
-                    gx = torch.empty((B, I), dtype=torch.float32, device=g.device)
+                    gx = torch.empty((B, I), dtype=torch.float32, device=device)
             if not have_tables[l]:
                 grads[l] = torch.empty_like(luts[l])
-            ws = _bytes(lib.dl_dwn_bwd_workspace_bytes(*dims), g.device)
+            ws = _bytes(lib.dl_dwn_bwd_workspace_bytes(*dims), device)
             headed = l == n - 1 and ctx.head is not None
             groups, tau = ctx.head if headed else (1, 1.0)
             if len(ctx.scalars[l]) == 3:  # every node's own alpha and beta
@@ -315,7 +317,9 @@ class DWNStackFunction(torch.autograd.Function):
                 if fuse:
                     grads[l - 1] = torch.empty_like(luts[l - 1])
                     have_tables[l - 1] = True
-                    ws = _bytes(lib.dl_dwn_bwd_fused_workspace_bytes(*dims, k_prev), g.device)
+                    ws = _bytes(lib.dl_dwn_bwd_fused_workspace_bytes(*dims, k_prev), device)
+                    if l == 1 and not first_wants_input_grad:
+                        gx = None  # the first layer's table gradient is all that is left: nobody reads this gradient
                 nat.check(lib.dl_dwn_layer_bwd_chain_fused(
                     nat.ptr(saved[l]), nat.ptr(plan.inv_ptr), nat.ptr(plan.inv_pos), nat.ptr(luts[l]), nat.ptr(g),
                     2 if headed else tiled, int(groups), float(tau), nat.ptr(alpha_n), nat.ptr(beta_n), float(beta_max),
@@ -338,7 +342,7 @@ class DWNStackFunction(torch.autograd.Function):
             g, tiled = gx, gx_tiled
         if ctx.image is not None and g is not None:
             shape, geom = ctx.image
-            gimg = torch.empty(shape, dtype=torch.float32, device=g.device)
+            gimg = torch.empty(shape, dtype=torch.float32, device=device)
             nat.check(lib.dl_fold(nat.ptr(g), 1, nat.ptr(gimg), *shape, *geom, nat.stream()))
             g = gimg
         return (g, None, None, None, None, *grads)

@@ -184,7 +184,10 @@ int dl_dwn_layer_bwd_chain_nodes(const void *saved, const int32_t *inv_ptr, cons
  *     workspace dl_dwn_bwd_fused_workspace_bytes.  Bins are summed per block and then in block order: reproducible,
  *     but a different order of additions than dl_dwn_layer_bwd_tiled's for the same table.
  *   gluts (nullable): NULL when this layer's own table gradient has already been produced by the call for the layer
- *     behind it; gy must then be tile-major (gy_form 1) and gx non-NULL. */
+ *     behind it; gy must then be tile-major (gy_form 1) and gx or prev_saved non-NULL.
+ *   gx (nullable with prev_saved): NULL when nobody reads this layer's input gradient after the bins of the layer in
+ *     front are filled (that layer is the first of the chain and its input needs no gradient): the sums are then made
+ *     for the bins only and not stored (B x I x 4 bytes less to write). */
 int dl_dwn_chain_fusable(int B, int I, int N, int k, int O, int k_prev, float beta_abs_max);
 size_t dl_dwn_bwd_fused_workspace_bytes(int B, int I, int N, int k, int O, int k_prev);
 int dl_dwn_layer_bwd_chain_fused(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos, const float *luts,

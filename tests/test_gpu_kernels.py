@@ -216,6 +216,14 @@ def test_dwn_chained_backward_fills_the_table_gradient_of_the_layer_in_front(sha
                                                wsx.data_ptr(), wsx.numel(), *dims, nat.stream()))
     assert torch.equal(gx2, gx_ref)
     assert torch.equal(glf2, glf)  # fixed order of additions: the same bits on every call
+    # no buffer for the input gradient (nobody behind the front layer reads it): the same bins, the same bits, and the
+    # layer's own table gradient as before
+    glf4, gl4 = torch.empty_like(lf), torch.empty_like(ld)
+    nat.check(lib.dl_dwn_layer_bwd_chain_fused(saved.data_ptr(), plan.inv_ptr.data_ptr(), plan.inv_pos.data_ptr(), ld.data_ptr(),
+                                               gd.data_ptr(), 0, 1, 1.0, alpha_n.data_ptr(), beta_n.data_ptr(), beta_max,
+                                               None, 1, gl4.data_ptr(), saved_f.data_ptr(), kf, glf4.data_ptr(),
+                                               wsx.data_ptr(), wsx.numel(), *dims, nat.stream()))
+    assert torch.equal(glf4, glf) and torch.equal(gl4, gl_ref)
     # and without a front layer it is the plain chained backward
     gx3 = torch.zeros_like(gx)
     nat.check(lib.dl_dwn_layer_bwd_chain_fused(saved.data_ptr(), plan.inv_ptr.data_ptr(), plan.inv_pos.data_ptr(), ld.data_ptr(),
