@@ -861,8 +861,10 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx(const float *__restrict__ gyT,
 // of its class (t = cls + ncls i); it ends with its bins as one partial set ([set][column][bin]), the sets are added
 // in set order afterwards (dwn_reduce_partials): fixed order, no atomics.
 // ROWS (a single big layer): the row-major gradient gx [B, I] through the block's LDS tile, the blocks paced (below).
-// The gather itself is dwn_bwd_gx's (O == 1, S form): the unrolled path for sixteen inputs of FAN entries each, with
-// the entries' coefficient rows kept in registers over all tiles, the general loop otherwise; same order of additions.
+// The gather itself is dwn_bwd_gx's (O == 1): the unrolled path for WI inputs of FAN entries each per wavefront, with
+// the entries' coefficient rows kept in registers over all tiles (S form: one row of 64 per entry, WI = 16 or 4; PACK:
+// two D-form rows of 32 per register, WI = 32), the general loop otherwise; same order of additions.
+// gx == null (HIST only): the sums are made for the bins of the layer in front and not stored.
 // Pacing of the walking gather (ROWS).  Its blocks are independent; left alone they spread over several batch tiles and
 // every tile's rows are fetched into an XCD's L2 more than once (measured at the headline shape, 16 inputs per
 // wavefront: 692 MiB against 320 compulsory, 55 % L2 misses, 160 us).  So every block starts its tile number i no
