@@ -297,6 +297,9 @@ class DWNStackFunction(torch.autograd.Function):
                     gx = torch.empty(lib.dl_dwn_tiled_bytes(B, I) // 4, dtype=torch.float32, device=device)
                 else:
                     gx = torch.empty((B, I), dtype=torch.float32, device=device)
+            if have_tables[l] and gx is None:  # nothing left to compute for this layer
+                g = None
+                continue
             if not have_tables[l]:
                 grads[l] = torch.empty_like(luts[l])
             ws = _bytes(lib.dl_dwn_bwd_workspace_bytes(*dims), device)
@@ -311,9 +314,6 @@ class DWNStackFunction(torch.autograd.Function):
                 k_prev = ctx.dims_all[l - 1][3] if l > 0 else 0
                 fuse = (l > 0 and gx_tiled == 1 and ctx.dims_all[l - 1][4] == 1
                         and lib.dl_dwn_chain_fusable(*dims, k_prev, float(beta_max)) == 1)
-                if have_tables[l] and gx is None:  # nothing left to compute for this layer
-                    g = None
-                    continue
                 if fuse:
                     grads[l - 1] = torch.empty_like(luts[l - 1])
                     have_tables[l - 1] = True
