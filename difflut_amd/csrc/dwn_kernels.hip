@@ -915,7 +915,7 @@ __device__ __forceinline__ float dwn_walk_diff_packed(float coef, unsigned a, in
     const unsigned ap = (a & low) | ((a >> 1) & ~low);  // the address without its bit j
     return __int_as_float(__builtin_amdgcn_ds_bpermute((int)((ap << 2) | (odd ? 128u : 0u)), __float_as_int(coef)));
 }
-// PACK (with DFORM, without HIST): the D-form row of a slot has 2^(K-1) <= 32 values, so the rows of two entries share one
+// PACK (with DFORM; with HIST only up to 16 inputs per wavefront): the D-form row of a slot has 2^(K-1) <= 32 values, so the rows of two entries share one
 // register (lanes 0-31 and 32-63) and a wavefront keeps 32 inputs' entries in the registers that 16 inputs' S-form rows
 // take: half as many blocks cover the inputs, and twice as many inputs are resident on an XCD.
 template <int K, int WI, int FAN, bool HIST = true, bool ROWS = false, bool DFORM = false, bool PACK = false>
@@ -989,7 +989,8 @@ __global__ __launch_bounds__(256) void dwn_bwd_gx_walk(const float *__restrict__
     constexpr int NREC = FAN > 0 ? (WI * FAN + 63) / 64 : 1;
     int rec3[NREC] = {};  // entry e of the wavefront: lane e % 64 of rec3[e / 64]
     if constexpr (FAN > 0) {
-        static_assert(!PACK || (DFORM && !HIST && WI * FAN % 2 == 0), "packed rows: D form, no histogram role");
+        static_assert(!PACK || (DFORM && (!HIST || WI <= 16) && WI * FAN % 2 == 0),
+                      "packed rows: D form; the histogram role covers sixteen columns per wavefront");
         const int len = __shfl_down(myptr, 1) - myptr;  // lanes 0..WI-1: entries of my input
         uniform3 = __ballot(lane >= WI || len == FAN) == ~0ull;
         if (uniform3) {
@@ -1493,8 +1494,14 @@ static inline int dwn_fused_wi(int I, int N, int K) {
     if ((long long)N * K >= 32LL * I) return 0;
     return (long long)N * K >= 6LL * I ? DWN_WI_SMALL : DWN_WI;
 }
+// Inputs that are all read six times (equal widths at k = 6) take the packed rows: two D-form rows per register, so a
+// wavefront keeps 16 inputs' 96 entries instead of 4 inputs' 24, and a quarter as many blocks cover the inputs (an
+// 8000-input layer then fits one XCD's resident blocks, and a tile is read through one L2 instead of four).
+static inline bool dwn_fused_pack(int I, int N, int K) {
+    return dwn_fused_wi(I, N, K) == DWN_WI_SMALL && (long long)N * K == 6LL * I;
+}
 static inline size_t dwn_fused_partial_bytes(int B, int I, int N, int k, int k_prev) {
-    const int wi = dwn_fused_wi(I, N, k);
+    const int wi = dwn_fused_pack(I, N, k) ? DWN_WI : dwn_fused_wi(I, N, k);
     if (!wi) return 0;
     const DwnFusedSplit f = dwn_fused_split(dwn_bt(B), I, k_prev, 4 * wi);
     return dl_align256((size_t)f.sets * I * ((size_t)4 << k_prev));
@@ -1563,7 +1570,10 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
     const bool walk_rows = gx && dwn_walk_rows(BT, I, N, k, O, gx_tiled);
     const bool walk_pack = walk_rows && dl_ceil_div(I, 4 * DWN_WI) > DWN_RESIDENT;
     const bool gather = gx || prev;  // (prev without gx: the input gradient is summed for the bins in front, not stored)
-    DwnTables tb = {gather && (!rc || rc->first) ? luts : nullptr, D, scale, alpha_n, beta_n, alpha, beta, (int)NO, k, O, sform ? (walk_pack ? 2 : 1) : 0};
+    const int fused_wi = prev && (gx_tiled || !gx) && O == 1 && sform ? dwn_fused_wi(I, N, k) : 0;
+    const bool fused_pack = fused_wi && dwn_fused_pack(I, N, k);
+    DwnTables tb = {gather && (!rc || rc->first) ? luts : nullptr, D, scale, alpha_n, beta_n, alpha, beta, (int)NO, k, O,
+                    sform ? (walk_pack || fused_pack ? 2 : 1) : 0};
     const dim3 hgrid(col_tiles, chunks + dl_ceil_div(dwn_table_blocks(tb), col_tiles));
     if (!gluts) {
         // the table gradient of this layer is already there (the gather of the layer behind filled its bins): only the
@@ -1588,20 +1598,22 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
         red.partial = rc->total_sets ? rc->partial_base : nullptr;
         red.chunks = rc->total_sets;
     }
-    const int fused_wi = prev && (gx_tiled || !gx) && O == 1 && sform ? dwn_fused_wi(I, N, k) : 0;
     if (!gather && dwn_reduce_blocks(red))
         DL_TIMED("dwn_reduce_partials", s, (dwn_reduce_partials<<<dwn_reduce_blocks(red), 256, 0, s>>>(red)));
     if (fused_wi) {
         // the gather that also fills the bins of the layer in front
         const float *src = gy_tiled ? gy : gyT;
-        const DwnFusedSplit f = dwn_fused_split(BT, I, prev->k, 4 * fused_wi);
+        const DwnFusedSplit f = dwn_fused_split(BT, I, prev->k, 4 * (fused_pack ? DWN_WI : fused_wi));
         const int fan = (long long)N * k % I == 0 ? (int)((long long)N * k / I) : 0;  // every input read `fan` times?
         const int gather_blocks = DL_XCDS * f.part * f.groups, grid = gather_blocks + dwn_reduce_blocks(red), Lp = 1 << prev->k;
 #define DWN_GXH(K_, WI_, FAN_)                                                                                                \
     DL_TIMED("dwn_bwd_gx_hist", s, (dwn_bwd_gx_walk<K_, WI_, FAN_><<<grid, 256, 0, s>>>(src, addrT, D, inv_ptr, inv_pos, gx, prev->addrT, \
                                                                                   prev->partial, I, N, BT, f.slabs, f.split, f.part, f.tpb, Lp, gather_blocks, red)))
 #define DWN_GXH_K(K_)                                                \
-    if (fused_wi != DWN_WI && fan == 6) DWN_GXH(K_, DWN_WI_SMALL, 6); \
+    if (fused_pack)                                                  \
+        DL_TIMED("dwn_bwd_gx_hist", s, (dwn_bwd_gx_walk<K_, DWN_WI, 6, true, false, true, true><<<grid, 256, 0, s>>>(src, addrT, D, inv_ptr, inv_pos, gx, prev->addrT, \
+                                                                                  prev->partial, I, N, BT, f.slabs, f.split, f.part, f.tpb, Lp, gather_blocks, red))); \
+    else if (fused_wi != DWN_WI && fan == 6) DWN_GXH(K_, DWN_WI_SMALL, 6); \
     else if (fused_wi != DWN_WI && fan == 12) DWN_GXH(K_, DWN_WI_SMALL, 12); \
     else if (fused_wi != DWN_WI) DWN_GXH(K_, DWN_WI_SMALL, 0);       \
     else if (fan == 1) DWN_GXH(K_, DWN_WI, 1);                       \
