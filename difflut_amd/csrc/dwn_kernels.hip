@@ -1229,29 +1229,33 @@ static inline void dwn_hist_grid(long long NO, int BT, int &col_tiles, int &chun
     tpc = dl_ceil_div(BT, chunks);
     chunks = dl_ceil_div(BT, tpc);
 }
-// A big layer's backward with row-major gradients (the walking gather, dwn_walk_rows) is taken in chunks of about
-// DWN_ROW_CHUNK_BYTES worth of batch tiles, histogram and gather of one chunk after the other: the tile-major copy of a chunk's
+// A big layer's backward with row-major gradients is taken in chunks of about DWN_ROW_CHUNK_BYTES worth of batch tiles,
+// histogram and gather of one chunk after the other (whichever gather the layer takes; 8192 -> 8192 nodes with the
+// in-order one, B = 8192: 0.592 -> 0.502 ms): the tile-major copy of a chunk's
 // gy (and its saved addresses) is then still in the 256 MB Infinity Cache when the gather reads it.  Measured at
 // 16384 -> 8192 nodes: the gather takes 109 us for 4096 rows but 284 us for 8192 and 566 us for 16384 in one piece.
 // Every chunk leaves its own partial sets of the table gradient; the last chunk's launch adds all of them, in order.
 #define DWN_ROW_CHUNK_BYTES 172e6  // gy tile-major + saved addresses of a chunk (the headline's 4096 rows: 168 MB)
-static inline bool dwn_walk_rows(int BT, int I, int N, int k, int O, int gx_tiled);
+static inline int dwn_walk_rows(int BT, int I, int N, int k, int O, int gx_tiled);
 static inline int dwn_row_chunks(int BT, int I, int N, int k, int O) {
+    (void)I, (void)k;
     int tiles = (int)(DWN_ROW_CHUNK_BYTES / ((double)N * O * 320));
     if (tiles < 32) tiles = 32;  // (the walking gather wants 32 tiles)
-    if (2 * BT < 3 * tiles || !dwn_walk_rows(BT, I, N, k, O, 0)) return 1;
+    if (2 * BT < 3 * tiles) return 1;
     if (dl_ceil_div((long long)N * O, DWN_HC) > 512) return 1;  // (a chunk's histogram must leave partial sets)
     return (BT + tiles / 2) / tiles;
 }
+// the tiles of chunk c of n: as even as they come (BT / n each, the first BT % n one more), so that no chunk is tiny
+static inline int dwn_row_chunk_tiles(int BT, int n, int c) { return BT / n + (c < BT % n ? 1 : 0); }
+static inline int dwn_row_chunk_begin(int BT, int n, int c) { return c * (BT / n) + (c < BT % n ? c : BT % n); }
 // chunk partials of the table gradient (none when one chunk covers the batch)
 static inline size_t dwn_partial_bytes(int B, int I, int N, int k, int O) {
     int col_tiles, chunks, tpc;
     const int BT = dwn_bt(B), n = dwn_row_chunks(BT, I, N, k, O);
     if (n > 1) {
-        const int tc = dl_ceil_div(BT, n);
         size_t sets = 0;
         for (int c = 0; c < n; ++c) {
-            dwn_hist_grid((long long)N * O, BT - c * tc < tc ? BT - c * tc : tc, col_tiles, chunks, tpc);
+            dwn_hist_grid((long long)N * O, dwn_row_chunk_tiles(BT, n, c), col_tiles, chunks, tpc);
             sets += chunks;
         }
         return dl_align256(sets * N * O * sizeof(float) << k);
@@ -1518,10 +1522,16 @@ static inline size_t dwn_fused_partial_bytes(int B, int I, int N, int k, int k_p
 // 8192; 10000 -> 5000, B = 8192: 0.338 -> 0.387) and batches of fewer than 32 tiles (B = 2048, 32 tiles: 0.161 -> 0.153 ->
 // 0.144 ms; B = 1024: no difference).
 #define DWN_PACE_GBS 5000.0  // base pace: the bytes of a tile step at this rate
-static inline bool dwn_walk_rows(int BT, int I, int N, int k, int O, int gx_tiled) {
-    if (O != 1 || gx_tiled) return false;
-    if ((long long)N * k != 3LL * I) return false;
-    return (long long)N * 320 >= (2LL << 20) && BT >= 32;
+// Inputs read six times (equal widths at k = 6) take it with the packed rows and sixteen inputs per wavefront once the
+// 64-input slabs outnumber an XCD's resident blocks: 12288 -> 12288 at B = 4096 0.433 -> 0.352 ms, 16384 -> 16384 0.640 ->
+// 0.591; at 8192 -> 8192 the in-order gather stays ahead (0.253 against 0.268 ms).
+// Returns the fan-in it applies to (3 or 6), 0 = the in-order gather.
+static inline int dwn_walk_rows(int BT, int I, int N, int k, int O, int gx_tiled) {
+    if (O != 1 || gx_tiled) return 0;
+    if ((long long)N * 320 < (2LL << 20) || BT < 32) return 0;
+    if ((long long)N * k == 3LL * I) return 3;
+    if ((long long)N * k == 6LL * I && I > 64 * DWN_RESIDENT) return 6;
+    return 0;
 }
 static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const int32_t *inv_pos, const float *luts,
                              const float *gy, int gy_tiled, float alpha, float beta, const float *scale, float *gx,
@@ -1540,14 +1550,14 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
     if (!rc && gx && gluts && !prev && !head && !gy_tiled && !gx_tiled) {
         const int n = dwn_row_chunks(BT, I, N, k, O);
         if (n > 1) {  // in chunks of rows, each through this function again
-            const int tc = dl_ceil_div(BT, n);
             int total = 0, sets = 0;
             for (int c = 0; c < n; ++c) {
-                dwn_hist_grid(NO, std::min(tc, BT - c * tc), col_tiles, chunks, tpc);
+                dwn_hist_grid(NO, dwn_row_chunk_tiles(BT, n, c), col_tiles, chunks, tpc);
                 total += chunks;
             }
             for (int c = 0; c < n; ++c) {
-                const int t0 = c * tc, tiles = std::min(tc, BT - t0), rows = std::min(B - t0 * 64, tiles * 64);
+                const int t0 = dwn_row_chunk_begin(BT, n, c), tiles = dwn_row_chunk_tiles(BT, n, c);
+                const int rows = std::min(B - t0 * 64, tiles * 64);
                 const DwnRowChunk r = {partial, sets, c == n - 1 ? total : 0, c == 0};
                 const int rcode = dwn_backward_fast(addrT + (size_t)t0 * N * 64, inv_ptr, inv_pos, luts, gy + (size_t)t0 * 64 * NO, 0,
                                                     alpha, beta, scale, gx + (size_t)t0 * 64 * I, 0, gluts, ws, rows, I, N, k, O, s,
@@ -1567,8 +1577,8 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
     // fixed-order sum of the histogram partials rides in the gather's launch the same way.
     // the walking gather of a layer too wide for one XCD's resident blocks packs two D-form rows into a register; for
     // |beta| <= 1/2 its table then holds the differences of the S form (the bits the other gathers compute from it)
-    const bool walk_rows = gx && dwn_walk_rows(BT, I, N, k, O, gx_tiled);
-    const bool walk_pack = walk_rows && dl_ceil_div(I, 4 * DWN_WI) > DWN_RESIDENT;
+    const int walk_rows = gx ? dwn_walk_rows(BT, I, N, k, O, gx_tiled) : 0;
+    const bool walk_pack = walk_rows == 6 || (walk_rows == 3 && dl_ceil_div(I, 4 * DWN_WI) > DWN_RESIDENT);
     const bool gather = gx || prev;  // (prev without gx: the input gradient is summed for the bins in front, not stored)
     const int fused_wi = prev && (gx_tiled || !gx) && O == 1 && sform ? dwn_fused_wi(I, N, k) : 0;
     const bool fused_pack = fused_wi && dwn_fused_pack(I, N, k);
@@ -1635,7 +1645,7 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
     } else if (walk_rows) {
         // row-major input gradient of a big layer whose inputs are all read three times: the walking gather, paced
         const float *src = gy_tiled ? gy : gyT;
-        const int slabs = dl_ceil_div(I, 4 * (walk_pack ? 2 * DWN_WI : DWN_WI));
+        const int slabs = dl_ceil_div(I, 4 * (walk_pack && walk_rows == 3 ? 2 * DWN_WI : DWN_WI));
         int split = 1;
         while (split < DL_XCDS && dl_ceil_div(slabs, split) > DWN_RESIDENT) split *= 2;
         const int part = dl_ceil_div(slabs, split), ncls = DL_XCDS / split, tiles_cls = dl_ceil_div(BT, ncls);
@@ -1662,7 +1672,11 @@ static int dwn_backward_fast(const void *saved, const int32_t *inv_ptr, const in
              (dwn_bwd_gx_walk<K_, DWN_WI, 3, false, true, DF_><<<gb + dwn_reduce_blocks(red), 256, 0, s>>>(      \
                  src, addrT, D, inv_ptr, inv_pos, gx, nullptr, nullptr, I, N, BT, slabs, split, part, tpb, 0, gb, red, B, pace, slot)))
 #define DWN_WALK(K_)                                                                                             \
-    if (walk_pack)                                                                                               \
+    if (walk_rows == 6)                                                                                          \
+        DL_TIMED("dwn_bwd_gx", s,                                                                                \
+                 (dwn_bwd_gx_walk<K_, DWN_WI, 6, false, true, true, true><<<gb + dwn_reduce_blocks(red), 256, 0, s>>>( \
+                     src, addrT, D, inv_ptr, inv_pos, gx, nullptr, nullptr, I, N, BT, slabs, split, part, tpb, 0, gb, red, B, pace, slot))); \
+    else if (walk_pack)                                                                                          \
         DL_TIMED("dwn_bwd_gx", s,                                                                                \
                  (dwn_bwd_gx_walk<K_, 2 * DWN_WI, 3, false, true, true, true><<<gb + dwn_reduce_blocks(red), 256, 0, s>>>( \
                      src, addrT, D, inv_ptr, inv_pos, gx, nullptr, nullptr, I, N, BT, slabs, split, part, tpb, 0, gb, red, B, pace, slot))); \

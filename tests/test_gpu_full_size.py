@@ -71,7 +71,11 @@ def test_single_dwn_layer_all_rows_against_c_restatement():
     ("whole permutations", 2100, 1 / 3, (16386, 8193, 6)),
     # more than 6000 rows: the backward is taken in chunks of about 4096 rows (two here, the last tile with eight rows;
     # three of 53 or 54 tiles each), and the table gradient adds the chunks' partial sums one after the other
-    ("whole permutations", 8200, 1 / 3, (16384, 8192, 6)), ("independent draws", 10250, 0.9, (16384, 8192, 6))])
+    ("whole permutations", 8200, 1 / 3, (16384, 8192, 6)), ("independent draws", 10250, 0.9, (16384, 8192, 6)),
+    # equal widths, every input read six times: sixteen inputs per wavefront with the packed rows; and the in-order
+    # gather in chunks of rows (8192 inputs: the walking gather does not apply)
+    ("whole permutations", 2100, 1 / 3, (12288, 12288, 6)), ("whole permutations", 2050, 0.9, (12288, 12288, 6)),
+    ("whole permutations", 8200, 1 / 3, (8192, 8192, 6))])
 def test_row_major_input_gradient_of_a_big_layer_equals_the_tile_major_one(mapping, B, beta, shape):
     """At this size the row-major input gradient is taken by the walking, paced gather (two entries' rows of table
     differences per register, 32 inputs per wavefront), the tile-major one by the one-block-per-(slab, tile) gather:
