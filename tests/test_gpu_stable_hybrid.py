@@ -314,6 +314,42 @@ def test_full_size_properties_stable_and_hybrid_k6_b4096_n8192():
         assert torch.isfinite(gx).all() and gx.abs().max().item() > 0
 
 
+@pytest.mark.parametrize("kind", ["stable", "dwn two outputs per node"])
+def test_backward_in_chunks_of_rows_equals_the_halves(kind):
+    """From about 6000 rows on the backward of a big layer runs chunk after chunk of rows inside one call.  Against the
+    two half batches on their own (too small for chunks): the input gradient is the same rows bit for bit (a row's
+    sums do not depend on the rows around it), the table gradient the sum of the two (other grouping of the same
+    terms: rtol 1e-5).  The stabilised node (its scale enters where the chunks' partial sums are added, once) and a
+    DWN layer with two outputs per node (columns are not nodes)."""
+    ops = _ops()
+    B, k = 8200, 6
+    I, N, O = (16384, 8192, 1) if kind == "stable" else (8192, 4096, 2)
+    g = torch.Generator(device="cpu").manual_seed(3)
+    x = torch.rand((B, I), generator=g).to(DEV)
+    idx = orc.random_mapping(I, N, k, seed=11).to(DEV, torch.int32)
+    plan = ops.MappingPlan(idx, I)
+    luts = (torch.rand((N, O, 64), generator=g) * 2 - 1).to(DEV)
+    gy = torch.randn((B, N * O), generator=g).to(DEV)
+    scale = (torch.rand((N,), generator=g) + 0.5).to(DEV)
+
+    def run(rows):
+        xt = x[rows].clone().requires_grad_()
+        tt = luts.clone().requires_grad_()
+        if kind == "stable":
+            y = ops.DWNStableLayerFunction.apply(xt, tt, scale, plan)
+        else:
+            y = ops.DWNLayerFunction.apply(xt, tt, plan, 0.1, 1.0 / 3.0)
+        y.backward(gy[rows])
+        return xt.grad, tt.grad
+
+    gx, gl = run(slice(0, B))
+    half = 4096  # a multiple of 64: the halves' batch tiles are the whole batch's
+    gx_a, gl_a = run(slice(0, half))
+    gx_b, gl_b = run(slice(half, B))
+    assert torch.equal(gx[:half], gx_a) and torch.equal(gx[half:], gx_b)
+    torch.testing.assert_close(gl, gl_a + gl_b, rtol=1e-5, atol=2e-5 * float(gl.abs().max()))
+
+
 @pytest.mark.parametrize("name,kind", [("dwn_stable", "stable"), ("hybrid", "hybrid")])
 @pytest.mark.parametrize("tag", ["k6o1", "k3o2"])
 def test_nodes_against_reference_vectors(golden_next, name, kind, tag):
