@@ -29,6 +29,8 @@ __device__ __forceinline__ int dl_uniform(int v) { return __builtin_amdgcn_readf
 // of one outer index run on the same XCD, so what they share is fetched into one L2 once.
 // Launch with dl_xcd_grid(inner_count, outer_count) blocks; blocks mapped past the end return false.
 #define DL_XCDS 8
+// fourth word of a raw buffer descriptor on gfx9 (32-bit data format, range check against num_records)
+#define DL_BUFFER_WORD3 0x00020000
 static inline int dl_xcd_grid(int inner_count, int outer_count) {
     return DL_XCDS * inner_count * ((outer_count + DL_XCDS - 1) / DL_XCDS);
 }

@@ -1,6 +1,7 @@
 // RandomLayer index gather and its adjoint, LearnableLayer hard selection, thermometer
 // encoding and GroupSum: the streaming pieces either side of the node kernels.
 #include "dl_common.h"
+#include <algorithm>
 
 // m[b,n,j] = x[b, idx[n,j]]: one block per (row, slab of the flattened [N*k] axis).  The row of
 // x is read through the cache (random but inside one 4*I-byte row), writes are coalesced.
@@ -27,6 +28,101 @@ __global__ __launch_bounds__(256) void gather_bwd_kernel(const float *__restrict
         float acc = 0.0f;
         for (int e = inv_ptr[i]; e < inv_ptr[i + 1]; ++e) acc += row[inv_pos[e]];
         gx[(size_t)b * I + i] = acc;
+    }
+}
+
+// The same two operations with the row that is read at random staged in the LDS: a wavefront's 64 random 4-byte reads
+// of a row in memory cost the texture addresser 64 cycles (the kernels above reach 1.25 and 0.95 TB/s at 4096 x 16384
+// -> 8192 x 6), from the LDS a few.  Blocks of 1024 threads walk the rows; global reads and writes are all coalesced.
+// fwd: the row of x (I floats, at most DL_GATHER_LDS_FLOATS) is staged, m[b][p] = row[idx[p]].
+#define DL_GATHER_LDS_FLOATS 32768  // 128 KB of the CU's 160
+#define DL_GATHER_BWD_FLOATS 24576  // pieces of the adjoint's rows: 96 KB, six 16-byte loads per thread
+template <typename index_t>
+__global__ __launch_bounds__(1024) void gather_fwd_lds(const float *__restrict__ x, const index_t *__restrict__ idx,
+                                                        float *__restrict__ m, int B, int I, long long NK) {
+    extern __shared__ float dl_gather_row[];
+    float *row = dl_gather_row;
+    const bool vec = (I & 3) == 0 && (((uintptr_t)x) & 15) == 0;
+    for (int b = blockIdx.x; b < B; b += gridDim.x) {
+        const float *xrow = x + (size_t)b * I;
+        __syncthreads();  // the readers of the row before are done
+        if (vec) {
+            for (int i = threadIdx.x * 4; i < I; i += 4096)
+                *reinterpret_cast<float4 *>(row + i) = *reinterpret_cast<const float4 *>(xrow + i);
+        } else {
+            for (int i = threadIdx.x; i < I; i += 1024) row[i] = xrow[i];
+        }
+        __syncthreads();
+        float *out = m + (size_t)b * NK;
+        long long p = threadIdx.x;
+        for (; p + 3 * 1024 < NK; p += 4 * 1024) {  // four in flight
+            const int i0 = idx[p], i1 = idx[p + 1024], i2 = idx[p + 2048], i3 = idx[p + 3072];
+            const float v0 = row[i0], v1 = row[i1], v2 = row[i2], v3 = row[i3];
+            __builtin_nontemporal_store(v0, out + p);
+            __builtin_nontemporal_store(v1, out + p + 1024);
+            __builtin_nontemporal_store(v2, out + p + 2048);
+            __builtin_nontemporal_store(v3, out + p + 3072);
+        }
+        for (; p < NK; p += 1024) __builtin_nontemporal_store(row[idx[p]], out + p);
+    }
+}
+// bwd: the row of gm is staged piece by piece (CH floats); a thread owns inputs tid, tid + T, ... and walks each
+// one's CSR list, whose positions ascend: the additions happen in list order, as in gather_bwd_kernel.  NK < 2^31 - 1
+// (positions are int32).
+template <int QI>
+__global__ __launch_bounds__(1024) void gather_bwd_lds(const float *__restrict__ gm, const int *__restrict__ inv_ptr,
+                                                        const int *__restrict__ inv_pos, float *__restrict__ gx, int B,
+                                                        int I, long long NK, int CH, int i_begin, int i_end) {
+    extern __shared__ float dl_gather_row[];
+    float *piece = dl_gather_row;
+    constexpr int NONE = 0x7fffffff;
+    const bool vec = (NK & 3) == 0 && (CH & 3) == 0 && (((uintptr_t)gm) & 15) == 0;
+    // positions through a buffer descriptor: one register of offset per load in flight instead of a 64-bit address
+    const __amdgpu_buffer_rsrc_t rs_pos = __builtin_amdgcn_make_buffer_rsrc((void *)inv_pos, 0, (int)(NK * 4), DL_BUFFER_WORD3);
+    auto position = [&](int e) { return (int)__builtin_amdgcn_raw_buffer_load_b32(rs_pos, e * 4, 0, 0); };
+    for (int b = blockIdx.x; b < B; b += gridDim.x) {
+        const float *grow = gm + (size_t)b * NK;
+        float acc[QI];
+        int cur[QI], e1[QI], nxt[QI];  // nxt: the position of the entry at the cursor (NONE: list done)
+#pragma unroll
+        for (int q = 0; q < QI; ++q) {  // (the list bounds are read again for every row: registers are short at QI = 16)
+            const int i = i_begin + threadIdx.x + 1024 * q;
+            acc[q] = 0.0f;
+            cur[q] = i < i_end ? inv_ptr[i] : 0;
+            e1[q] = i < i_end ? inv_ptr[i + 1] : 0;
+            nxt[q] = cur[q] < e1[q] ? position(cur[q]) : NONE;
+        }
+        for (long long base = 0; base < NK; base += CH) {
+            const int len = (int)min((long long)CH, NK - base);
+            __syncthreads();  // the readers of the piece before are done
+            if (vec) {
+                for (int i = threadIdx.x * 4; i < len; i += 4096)
+                    *reinterpret_cast<float4 *>(piece + i) = *reinterpret_cast<const float4 *>(grow + base + i);
+            } else {
+                for (int i = threadIdx.x; i < len; i += 1024) piece[i] = grow[base + i];
+            }
+            __syncthreads();
+            // one entry per input and sweep: the loads of the next positions of all my inputs are in flight together
+            const long long end = base + len;
+            bool moved = true;
+            while (moved) {
+                moved = false;
+#pragma unroll
+                for (int q = 0; q < QI; ++q) {
+                    if (nxt[q] < end) {
+                        if (nxt[q] >= base) acc[q] += piece[nxt[q] - base];  // (before the piece: not ascending as promised)
+                        ++cur[q];
+                        nxt[q] = cur[q] < e1[q] ? position(cur[q]) : NONE;
+                        moved = true;
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < QI; ++q) {
+            const int i = i_begin + threadIdx.x + 1024 * q;
+            if (i < i_end) __builtin_nontemporal_store(acc[q], gx + (size_t)b * I + i);
+        }
     }
 }
 
@@ -164,12 +260,32 @@ __global__ __launch_bounds__(256) void cross_entropy_mean(const float *__restric
 }
 
 // ---------------------------------------------------------------------------------
+// more than 64 KB of dynamic LDS has to be asked for, once per kernel (any thread may be the first)
+static int dl_gather_lds_attr(const void *fn, size_t bytes) {
+    if (bytes <= 64 * 1024) return 0;
+    return (int)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+}
+
 extern "C" int dl_gather_fwd(const float *x, const void *idx, int idx_bits, float *m, int B, int I, int N, int k,
                              void *stream) {
     if (!x || !idx || !m) return DL_ERR_NULL;
     if (B <= 0 || I <= 0 || N <= 0 || k <= 0) return DL_ERR_SHAPE;
     if (idx_bits != 16 && idx_bits != 32) return DL_ERR_UNSUPPORTED;
     const long long NK = (long long)N * k;
+    if (I <= DL_GATHER_LDS_FLOATS && NK >= 4096) {  // the row of x through the LDS
+        const size_t lds = (size_t)I * sizeof(float);
+        const int per_cu = (int)std::max<size_t>(1, std::min<size_t>(2, (160 * 1024) / (lds + 1024)));
+        const int blocks = std::min(B, 256 * per_cu);
+        hipStream_t s = (hipStream_t)stream;
+        if (idx_bits == 16) {
+            if (int rc = dl_gather_lds_attr(reinterpret_cast<const void *>(&gather_fwd_lds<int16_t>), lds)) return rc;
+            DL_TIMED("gather_fwd", s, (gather_fwd_lds<int16_t><<<blocks, 1024, lds, s>>>(x, (const int16_t *)idx, m, B, I, NK)));
+        } else {
+            if (int rc = dl_gather_lds_attr(reinterpret_cast<const void *>(&gather_fwd_lds<int32_t>), lds)) return rc;
+            DL_TIMED("gather_fwd", s, (gather_fwd_lds<int32_t><<<blocks, 1024, lds, s>>>(x, (const int32_t *)idx, m, B, I, NK)));
+        }
+        return dl_launch_status();
+    }
     dim3 grid(dl_ceil_div(NK, 1024), B < 65535 ? B : 65535);
     if (idx_bits == 16)
         gather_fwd_kernel<int16_t><<<grid, 256, 0, (hipStream_t)stream>>>(x, (const int16_t *)idx, m, B, I, NK);
@@ -182,6 +298,31 @@ extern "C" int dl_gather_bwd(const float *gm, const int32_t *inv_ptr, const int3
                              int N, int k, void *stream) {
     if (!gm || !inv_ptr || !inv_pos || !gx) return DL_ERR_NULL;
     if (B <= 0 || I <= 0 || N <= 0 || k <= 0) return DL_ERR_SHAPE;
+    const long long NK = (long long)N * k;
+    if (NK >= 4096 && NK < 0x7fffffffLL) {  // the row of gm through the LDS, piece by piece
+        const long long pieces = dl_ceil_div(NK, (long long)DL_GATHER_BWD_FLOATS);
+        const int CH = (int)((dl_ceil_div(NK, pieces) + 3) / 4 * 4);
+        const size_t lds = (size_t)CH * sizeof(float);
+        const int per_cu = (int)std::max<size_t>(1, std::min<size_t>(2, (160 * 1024) / (lds + 1024)));
+        const int blocks = std::min(B, 256 * per_cu);
+        hipStream_t s = (hipStream_t)stream;
+        // a thread has at most 16 inputs, so wider layers are taken 16384 inputs at a time (the row of gm is then staged
+        // once per such window)
+        for (int i0 = 0; i0 < I; i0 += 16384) {
+            const int i1 = std::min(I, i0 + 16384), In = i1 - i0;
+#define DL_GBWD(QI_)                                                                                                   \
+    do {                                                                                                               \
+        if (int rc = dl_gather_lds_attr(reinterpret_cast<const void *>(&gather_bwd_lds<QI_>), lds)) return rc;         \
+        DL_TIMED("gather_bwd", s,                                                                                      \
+                 (gather_bwd_lds<QI_><<<blocks, 1024, lds, s>>>(gm, inv_ptr, inv_pos, gx, B, I, NK, CH, i0, i1)));      \
+    } while (0)
+            if (In <= 1024) DL_GBWD(1);
+            else if (In <= 4096) DL_GBWD(4);
+            else DL_GBWD(16);
+#undef DL_GBWD
+        }
+        return dl_launch_status();
+    }
     gather_bwd_kernel<<<dim3(dl_ceil_div(I, 256), B < 65535 ? B : 65535), 256, 0, (hipStream_t)stream>>>(
         gm, inv_ptr, inv_pos, gx, B, I, (long long)N * k);
     return dl_launch_status();

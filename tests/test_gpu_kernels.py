@@ -453,6 +453,33 @@ def test_gather_forward_backward(dtype):
     np.testing.assert_allclose(xt.grad.cpu().numpy(), orc.gather_backward(gm, idx, I), rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("shape", [(70, 1031, 700, 6, torch.int16),      # 4200 connections: one piece, odd widths (scalar staging)
+                                   (33, 3136, 2000, 6, torch.int16),     # cfg 1's layer: lists of three and four
+                                   (25, 4096, 4096, 4, torch.int32),     # whole permutations, four inputs per thread
+                                   (9, 16384, 8192, 6, torch.int32),     # two pieces per row, sixteen inputs per thread
+                                   (5, 20001, 9000, 5, torch.int32),     # two windows of inputs, pieces of odd length
+                                   (3, 300, 48000, 1, torch.int32)])     # hard selection's shape: long lists, one input each
+def test_gather_through_the_lds(shape):
+    """From 4096 connections on the row that is read at random (x forward, gm backward) is staged in the LDS.  The
+    forward is a copy: exact.  The backward adds a list in its order, like the oracle's loop: exact as well."""
+    ops = _ops()
+    B, I, N, k, dtype = shape
+    rng = np.random.default_rng(I + N)
+    x = rng.standard_normal((B, I)).astype(np.float32)
+    idx = orc.random_mapping(I, N, k, seed=5).numpy().astype(np.int64)
+    it = dev(idx, dtype)
+    xt = dev(x).requires_grad_()
+    m = ops.GatherFunction.apply(xt, it, ops.MappingPlan(it, I))
+    assert np.array_equal(m.detach().cpu().numpy(), x[:, idx])
+    gm = rng.standard_normal((B, N, k)).astype(np.float32)
+    m.backward(dev(gm))
+    want = np.zeros((B, I), np.float32)
+    flat = gm.reshape(B, -1)
+    for p, i in enumerate(idx.reshape(-1)):  # ascending position within every input: the order of the CSR lists
+        want[:, i] += flat[:, p]
+    assert np.array_equal(xt.grad.cpu().numpy(), want)
+
+
 # ------------------------------------------------------------------------------ probabilistic
 PROB_SHAPES = [(32, 40, 24, 4, 2), (64, 128, 300, 4, 1), (17, 30, 9, 6, 1), (20, 9, 5, 1, 1), (10, 50, 7, 2, 3),
                (6, 40, 5, 7, 2), (200, 300, 260, 4, 1), (130, 70, 33, 5, 2), (65, 1000, 515, 3, 1),
