@@ -134,9 +134,26 @@ __global__ __launch_bounds__(256) void row_argmax_kernel(const float *__restrict
     const float *w = W + (size_t)row * I;
     float best = -INFINITY;
     int arg = 0x7fffffff;
-    for (int i = lane; i < I; i += 64) {
-        const float v = w[i];
+    auto take = [&](float v, int i) {
         if (v > best || (v == best && i < arg) || arg == 0x7fffffff) { best = v; arg = i; }
+    };
+    if ((I & 3) == 0 && (((uintptr_t)W) & 15) == 0) {  // 16 bytes per lane and load, four loads in flight
+        int i = lane * 4;
+        for (; i + 768 < I; i += 1024) {
+            float4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const float4 *>(w + i + 256 * u);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                take(v[u].x, i + 256 * u); take(v[u].y, i + 256 * u + 1); take(v[u].z, i + 256 * u + 2); take(v[u].w, i + 256 * u + 3);
+            }
+        }
+        for (; i < I; i += 256) {
+            const float4 v = *reinterpret_cast<const float4 *>(w + i);
+            take(v.x, i); take(v.y, i + 1); take(v.z, i + 2); take(v.w, i + 3);
+        }
+    } else {
+        for (int i = lane; i < I; i += 64) take(w[i], i);
     }
     for (int off = 32; off > 0; off >>= 1) {
         const float ob = __shfl_xor(best, off);
@@ -148,12 +165,26 @@ __global__ __launch_bounds__(256) void row_argmax_kernel(const float *__restrict
 
 __global__ __launch_bounds__(256) void thermometer_kernel(const float *__restrict__ x, const float *__restrict__ thr,
                                                            float *__restrict__ bits, long long total, int FB, int nbits) {
-    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (gid >= total) return;
-    const long long b = gid / FB;
-    const int fb = (int)(gid % FB);
-    const int f = fb / nbits;
-    bits[gid] = x[b * (FB / nbits) + f] > thr[fb] ? 1.0f : 0.0f;  // strict compare
+    // four consecutive outputs per thread, one 16-byte store (FB a multiple of four: they stay within a row)
+    const long long g4 = ((long long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (g4 >= total) return;
+    if ((FB & 3) == 0 && (((uintptr_t)bits) & 15) == 0) {
+        const long long b = g4 / FB;
+        const int fb = (int)(g4 % FB);
+        const float *xrow = x + b * (FB / nbits);
+        float4 out;
+        out.x = xrow[fb / nbits] > thr[fb] ? 1.0f : 0.0f;  // strict compare
+        out.y = xrow[(fb + 1) / nbits] > thr[fb + 1] ? 1.0f : 0.0f;
+        out.z = xrow[(fb + 2) / nbits] > thr[fb + 2] ? 1.0f : 0.0f;
+        out.w = xrow[(fb + 3) / nbits] > thr[fb + 3] ? 1.0f : 0.0f;
+        *reinterpret_cast<float4 *>(bits + g4) = out;
+        return;
+    }
+    for (long long gid = g4; gid < min(total, g4 + 4); ++gid) {
+        const long long b = gid / FB;
+        const int fb = (int)(gid % FB);
+        bits[gid] = x[b * (FB / nbits) + fb / nbits] > thr[fb] ? 1.0f : 0.0f;
+    }
 }
 
 // Thermometer bits as bit-planes for a following DWN layer: word (t, f*nbits + j) holds, in bit r,
@@ -349,7 +380,7 @@ extern "C" int dl_thermometer_encode(const float *x, const float *thr, float *bi
     if (!x || !thr || !bits) return DL_ERR_NULL;
     if (B <= 0 || F <= 0 || nbits <= 0) return DL_ERR_SHAPE;
     const long long total = (long long)B * F * nbits;
-    thermometer_kernel<<<dl_ceil_div(total, 256), 256, 0, (hipStream_t)stream>>>(x, thr, bits, total, F * nbits, nbits);
+    thermometer_kernel<<<dl_ceil_div(total, 1024), 256, 0, (hipStream_t)stream>>>(x, thr, bits, total, F * nbits, nbits);
     return dl_launch_status();
 }
 

@@ -604,6 +604,14 @@ def test_row_argmax_ties_and_sizes():
     W[6, :] = -1.0
     sel = ops.row_argmax(dev(W)).cpu().numpy()
     assert np.array_equal(sel, W.argmax(1)) and sel[5] == 17 and sel[6] == 0
+    # widths that are no multiple of four (one value per lane and load), of four but not of 1024 (a tail of 16-byte
+    # loads), and a tie that straddles two lanes' pieces
+    for M, I in ((9, 1031), (5, 2052), (7, 4096), (3, 12)):
+        W = rng.standard_normal((M, I)).astype(np.float32)
+        W[1, I - 1] = W[1, 2] = 7.0
+        W[2, :] = 0.5
+        sel = ops.row_argmax(dev(W)).cpu().numpy()
+        assert np.array_equal(sel, W.argmax(1)) and sel[1] == 2 and sel[2] == 0
 
 
 # ------------------------------------------------------------------------------ encoder / head
@@ -618,6 +626,14 @@ def test_thermometer_and_group_sum(golden):
     gy = np.random.default_rng(0).standard_normal((6, 5)).astype(np.float32)
     y.backward(dev(gy))
     np.testing.assert_allclose(xt.grad.cpu().numpy(), np.repeat(gy, 4, 1) / 2.0, rtol=1e-6)
+    # rows of bits that are and are not a multiple of four values (16-byte stores or one value at a time), strict compare
+    for B, F, nb in ((7, 5, 3), (64, 12, 4), (3, 6, 2), (130, 784, 4), (5, 1, 1)):
+        rs = np.random.default_rng(B * F + nb)
+        xs = rs.random((B, F)).astype(np.float32)
+        th = np.sort(rs.random((F, nb)).astype(np.float32), axis=1)
+        xs[0, 0] = th[0, 0]  # equal to a threshold: not above it
+        got = ops.thermometer_encode(dev(xs), dev(th)).cpu().numpy().reshape(B, F, nb)
+        assert np.array_equal(got, (xs[:, :, None] > th[None]).astype(np.float32))
     x = np.random.default_rng(1).standard_normal((3, 10)).astype(np.float32)  # 10 features, 4 groups: padded
     y = ops.GroupSumFunction.apply(dev(x), 4, 1.0)
     np.testing.assert_allclose(y.cpu().numpy(), orc.group_sum(x, 4, 1.0), rtol=1e-6, atol=1e-6)
