@@ -330,7 +330,7 @@ extern "C" int dl_gather_bwd(const float *gm, const int32_t *inv_ptr, const int3
     if (!gm || !inv_ptr || !inv_pos || !gx) return DL_ERR_NULL;
     if (B <= 0 || I <= 0 || N <= 0 || k <= 0) return DL_ERR_SHAPE;
     const long long NK = (long long)N * k;
-    if (NK >= 4096 && NK < 0x7fffffffLL) {  // the row of gm through the LDS, piece by piece
+    if (NK >= 4096 && NK < (1LL << 29)) {  // the row of gm through the LDS, piece by piece (byte offsets of positions: 32-bit)
         const long long pieces = dl_ceil_div(NK, (long long)DL_GATHER_BWD_FLOATS);
         const int CH = (int)((dl_ceil_div(NK, pieces) + 3) / 4 * 4);
         const size_t lds = (size_t)CH * sizeof(float);
