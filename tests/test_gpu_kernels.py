@@ -363,7 +363,10 @@ def test_dwn_eval_forward(shape):
         assert np.array_equal(y[:, n], orc.dwn_eval_forward(m[:, n], luts[n]))
 
 
-@pytest.mark.parametrize("shape", [(130, 40, 150, 6, 1), (64, 36, 70, 4, 2), (257, 33, 129, 5, 1)])
+@pytest.mark.parametrize("shape", [(130, 40, 150, 6, 1), (64, 36, 70, 4, 2), (257, 33, 129, 5, 1),
+                                   # from 1024 columns on the literal-address kernel stages the row of x in the LDS:
+                                   # odd widths, two outputs per node, two windows of columns
+                                   (37, 1031, 1100, 5, 1), (5, 300, 600, 3, 2), (9, 4096, 9000, 6, 1)])
 def test_dwn_eval_forward_any_input_values(shape):
     """The eval entry point with a workspace answers through the bit-plane kernels when every input is 0 or 1 and
     through the literal float address otherwise; both against the oracle, including inputs where the two
