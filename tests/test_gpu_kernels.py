@@ -45,6 +45,8 @@ DWN_SHAPES = [  # (B, I, N, k, O)
     (200, 1030, 515, 6, 2),
     (9, 30, 11, 7, 2),     # k > 6: generic kernels
     (5, 64, 6, 9, 1),
+    (21, 1031, 1100, 7, 1),  # k > 6 from 1024 columns on: the row of x through the LDS (odd width: scalar staging)
+    (6, 512, 520, 8, 2),     # the same with two outputs per node
 ]
 
 
