@@ -126,6 +126,71 @@ __global__ __launch_bounds__(1024) void gather_bwd_lds(const float *__restrict__
     }
 }
 
+// The adjoint for short lists: the first FMAX positions of every list of a thread's inputs stay in registers over all
+// the block's rows (QI x FMAX of them), so a row costs no index reads at all; used when no list is longer (checked by
+// the host through the average: N k <= FMAX I, and by every thread for its own lists - a longer one is finished through
+// its cursor, in order).
+template <int QI, int FMAX>
+__global__ __launch_bounds__(1024) void gather_bwd_lds_short(const float *__restrict__ gm, const int *__restrict__ inv_ptr,
+                                                              const int *__restrict__ inv_pos, float *__restrict__ gx, int B,
+                                                              int I, long long NK, int CH, int i_begin, int i_end) {
+    extern __shared__ float dl_gather_row[];
+    float *piece = dl_gather_row;
+    constexpr int NONE = 0x7fffffff;
+    int pos[QI][FMAX];
+    bool longer = false;  // one of my lists has more than FMAX entries
+#pragma unroll
+    for (int q = 0; q < QI; ++q) {
+        const int i = i_begin + threadIdx.x + 1024 * q;
+        const int e0 = i < i_end ? inv_ptr[i] : 0, e1 = i < i_end ? inv_ptr[i + 1] : 0;
+#pragma unroll
+        for (int f = 0; f < FMAX; ++f) pos[q][f] = e0 + f < e1 ? inv_pos[e0 + f] : NONE;
+        longer = longer || e1 - e0 > FMAX;
+    }
+    const bool vec = (NK & 3) == 0 && (CH & 3) == 0 && (((uintptr_t)gm) & 15) == 0;
+    for (int b = blockIdx.x; b < B; b += gridDim.x) {
+        const float *grow = gm + (size_t)b * NK;
+        float acc[QI];
+#pragma unroll
+        for (int q = 0; q < QI; ++q) acc[q] = 0.0f;
+        for (long long base = 0; base < NK; base += CH) {
+            const int len = (int)min((long long)CH, NK - base);
+            __syncthreads();  // the readers of the piece before are done
+            if (vec) {
+                for (int i = threadIdx.x * 4; i < len; i += 4096)
+                    *reinterpret_cast<float4 *>(piece + i) = *reinterpret_cast<const float4 *>(grow + base + i);
+            } else {
+                for (int i = threadIdx.x; i < len; i += 1024) piece[i] = grow[base + i];
+            }
+            __syncthreads();
+            const long long end = base + len;
+#pragma unroll
+            for (int q = 0; q < QI; ++q) {
+#pragma unroll
+                for (int f = 0; f < FMAX; ++f)
+                    if (pos[q][f] >= base && pos[q][f] < end) acc[q] += piece[pos[q][f] - base];
+            }
+            if (longer) {  // the rest of a long list, in order, after its first FMAX entries (positions ascend)
+                for (int q = 0; q < QI; ++q) {
+                    const int i = i_begin + threadIdx.x + 1024 * q;
+                    if (i >= i_end) break;
+                    const int e1 = inv_ptr[i + 1];
+                    for (int e = inv_ptr[i] + FMAX; e < e1; ++e) {
+                        const long long p = inv_pos[e];
+                        if (p >= end) break;
+                        if (p >= base) acc[q] += piece[p - base];
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < QI; ++q) {
+            const int i = i_begin + threadIdx.x + 1024 * q;
+            if (i < i_end) __builtin_nontemporal_store(acc[q], gx + (size_t)b * I + i);
+        }
+    }
+}
+
 // One wavefront per row of W; lowest index wins ties.
 __global__ __launch_bounds__(256) void row_argmax_kernel(const float *__restrict__ W, int *__restrict__ sel, int M, int I) {
     const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -347,7 +412,11 @@ extern "C" int dl_gather_bwd(const float *gm, const int32_t *inv_ptr, const int3
         DL_TIMED("gather_bwd", s,                                                                                      \
                  (gather_bwd_lds<QI_><<<blocks, 1024, lds, s>>>(gm, inv_ptr, inv_pos, gx, B, I, NK, CH, i0, i1)));      \
     } while (0)
-            if (In <= 1024) DL_GBWD(1);
+            if (In > 4096 && NK <= 3LL * I) {  // short lists: their positions in registers
+                if (int rc = dl_gather_lds_attr(reinterpret_cast<const void *>(&gather_bwd_lds_short<16, 3>), lds)) return rc;
+                DL_TIMED("gather_bwd", s, (gather_bwd_lds_short<16, 3><<<blocks, 1024, lds, s>>>(gm, inv_ptr, inv_pos, gx, B, I, NK,
+                                                                                              CH, i0, i1)));
+            } else if (In <= 1024) DL_GBWD(1);
             else if (In <= 4096) DL_GBWD(4);
             else DL_GBWD(16);
 #undef DL_GBWD
