@@ -809,11 +809,85 @@ extern "C" int dl_prob_layer_eval_ws_nodes(const float *x, const int32_t *idx32,
     return prob_eval_ws(x, idx32, raw_w, prob_temp(1.0f, temperature_n), y, ws, ws_bytes, B, I, N, k, O, stream);
 }
 
+// The same for k <= 6 with the row of x staged in the LDS by persistent blocks of 1024 threads: a thread keeps the input
+// indices of its (up to eight) columns and their binarised tables - bit a of a 64-bit mask = (sigmoid(w[a] / T) >= 0.5),
+// taken with the expression of prob_eval_kernel - in registers over all its rows.
+template <int K>
+__global__ __launch_bounds__(1024) void prob_eval_lds(const float *__restrict__ x, const int *__restrict__ idx32,
+                                                       const float *__restrict__ raw, ProbTemp T, float *__restrict__ y,
+                                                       int B, int I, long long NO, int O, long long c_begin, long long c_end) {
+    extern __shared__ float prob_eval_row[];
+    float *row = prob_eval_row;
+    constexpr int L = 1 << K, QC = 8;
+    int ix[QC][K];
+    unsigned long long mask[QC];
+#pragma unroll
+    for (int q = 0; q < QC; ++q) {
+        const long long c = c_begin + threadIdx.x + 1024LL * q;
+        mask[q] = 0ull;
+#pragma unroll
+        for (int j = 0; j < K; ++j) ix[q][j] = 0;
+        if (c < c_end) {
+            const int n = (int)(c / O), d = (int)(c % O);
+            const float inv_t = prob_inv_t_of(T, n);
+#pragma unroll
+            for (int j = 0; j < K; ++j) ix[q][j] = idx32[(size_t)n * K + j];
+            for (int a = 0; a < L; ++a)
+                mask[q] |= (dl_sigmoid(raw[((size_t)n * L + a) * O + d] * inv_t) >= 0.5f ? 1ull : 0ull) << a;
+        }
+    }
+    const bool vec = (I & 3) == 0 && (((uintptr_t)x) & 15) == 0;
+    for (int b = blockIdx.x; b < B; b += gridDim.x) {
+        const float *xrow = x + (size_t)b * I;
+        __syncthreads();  // the readers of the row before are done
+        if (vec) {
+            for (int i = threadIdx.x * 4; i < I; i += 4096)
+                *reinterpret_cast<float4 *>(row + i) = *reinterpret_cast<const float4 *>(xrow + i);
+        } else {
+            for (int i = threadIdx.x; i < I; i += 1024) row[i] = xrow[i];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < QC; ++q) {
+            const long long c = c_begin + threadIdx.x + 1024LL * q;
+            if (c >= c_end) break;
+            float sum = 0.0f;
+#pragma unroll
+            for (int j = 0; j < K; ++j) sum += row[ix[q][j]] * (float)(1 << j);  // the order of prob_eval_kernel's loop
+            long long a = (long long)sum;
+            a = a < 0 ? 0 : (a > L - 1 ? L - 1 : a);
+            __builtin_nontemporal_store(((mask[q] >> a) & 1ull) ? 1.0f : 0.0f, y + (size_t)b * NO + c);
+        }
+    }
+}
+
 extern "C" int dl_prob_layer_eval(const float *x, const int32_t *idx32, const float *raw_w, float temperature, float *y,
                                   int B, int I, int N, int k, int O, void *stream) {
     if (!x || !idx32 || !raw_w || !y) return DL_ERR_NULL;
     int rc = prob_check(B, I, N, k, O);
     if (rc) return rc;
+    const long long NO = (long long)N * O;
+    if (k <= 6 && I <= 32768 && NO >= 1024) {
+        hipStream_t s = (hipStream_t)stream;
+        const size_t lds = (size_t)I * sizeof(float);
+        const ProbTemp T = prob_temp(temperature, nullptr);
+        for (long long c0 = 0; c0 < NO; c0 += 8192) {  // windows of 8192 columns: eight per thread
+            const long long c1 = c0 + 8192 < NO ? c0 + 8192 : NO;
+#define CALL(KK)                                                                                                       \
+    do {                                                                                                               \
+        if (lds > 64 * 1024) {                                                                                         \
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&prob_eval_lds<KK>),               \
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);            \
+            if (e != hipSuccess) return (int)e;                                                                        \
+        }                                                                                                              \
+        DL_TIMED("prob_eval_kernel", s,                                                                                \
+                 (prob_eval_lds<KK><<<B < 256 ? B : 256, 1024, lds, s>>>(x, idx32, raw_w, T, y, B, I, NO, O, c0, c1))); \
+    } while (0)
+            PROB_DISPATCH(k, CALL)
+#undef CALL
+        }
+        return dl_launch_status();
+    }
     DL_TIMED("prob_eval_kernel", (hipStream_t)stream, (prob_eval_kernel<<<dl_ceil_div((long long)B * N * O, 256), 256, 0, (hipStream_t)stream>>>(
         x, idx32, raw_w, prob_temp(temperature, nullptr), y, B, I, N, k, O)));
     return dl_launch_status();

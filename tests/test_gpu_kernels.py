@@ -393,7 +393,9 @@ def test_dwn_eval_forward_any_input_values(shape):
                 assert np.array_equal(want, orc.dwn_eval_forward(m[:, n], luts[n]))
 
 
-@pytest.mark.parametrize("shape", [(130, 40, 150, 4, 1), (64, 36, 70, 6, 2), (200, 33, 90, 3, 1)])
+@pytest.mark.parametrize("shape", [(130, 40, 150, 4, 1), (64, 36, 70, 6, 2), (200, 33, 90, 3, 1),
+                                   # from 1024 columns on both literal-address kernels stage the row of x in the LDS
+                                   (33, 1031, 1100, 4, 1), (7, 300, 520, 6, 2)])
 def test_prob_eval_forward_any_input_values(shape):
     """Probabilistic eval through the workspace entry point (binarised sigmoid table looked up by the DWN eval
     path) against the oracle, for 0/1 inputs (bit-plane kernels), arbitrary inputs and a single odd value
